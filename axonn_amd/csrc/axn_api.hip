@@ -1,0 +1,310 @@
+// The C ABI of libaxn_gfx950.so (declared in axn.h): argument validation and
+// dispatch only.  Validation runs before any HIP call so that bad arguments are
+// reported the same way on a host without a GPU.
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+
+#include "axn_internal.h"
+
+namespace axn {
+
+static thread_local char g_err[512] = "";
+
+void set_error(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+}
+
+int hip_fail(hipError_t e, const char* what) {
+  set_error("HIP error %d (%s) in %s", (int)e, hipGetErrorString(e), what);
+  return AXN_EHIP;
+}
+
+namespace {
+
+bool aligned16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
+
+#define REQUIRE(cond, code, ...)   \
+  do {                             \
+    if (!(cond)) {                 \
+      set_error(__VA_ARGS__);      \
+      return (code);               \
+    }                              \
+  } while (0)
+
+int check_gemm(const char* name, const void* a, const void* b, const void* c,
+               int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb,
+               int64_t ldc, int64_t min_lda, int64_t min_ldb, int64_t min_ldc) {
+  REQUIRE(a && b && c, AXN_EINVAL, "%s: null operand pointer", name);
+  REQUIRE(M >= 1 && N >= 1 && K >= 1, AXN_EINVAL,
+          "%s: M, N, K must be >= 1 (got %lld, %lld, %lld)", name, (long long)M,
+          (long long)N, (long long)K);
+  REQUIRE(M <= 0x7fffffff && N <= 0x7fffffff && K <= 0x7fffffff, AXN_ELIMIT,
+          "%s: dimension exceeds 2^31-1", name);
+  REQUIRE(N % 8 == 0 && K % 8 == 0, AXN_ESHAPE,
+          "%s: N and K must be multiples of 8 (got N=%lld, K=%lld)", name,
+          (long long)N, (long long)K);
+  REQUIRE(lda >= min_lda && ldb >= min_ldb && ldc >= min_ldc, AXN_EINVAL,
+          "%s: leading dimension smaller than the row length", name);
+  REQUIRE(lda % 8 == 0 && ldb % 8 == 0 && ldc % 8 == 0, AXN_EALIGN,
+          "%s: leading dimensions must be multiples of 8", name);
+  REQUIRE(aligned16(a) && aligned16(b) && aligned16(c), AXN_EALIGN,
+          "%s: operand pointers must be 16-byte aligned", name);
+  return AXN_OK;
+}
+
+int check_epilogue(const char* name, int epilogue, const float* bias) {
+  REQUIRE(epilogue >= AXN_EPI_NONE && epilogue <= AXN_EPI_GELU, AXN_EINVAL,
+          "%s: unknown epilogue %d", name, epilogue);
+  const bool needs_bias = epilogue == AXN_EPI_BIAS || epilogue == AXN_EPI_BIAS_GELU;
+  REQUIRE(!needs_bias || bias != nullptr, AXN_EINVAL,
+          "%s: epilogue %d needs a bias vector", name, epilogue);
+  REQUIRE(!needs_bias || aligned16(bias), AXN_EALIGN,
+          "%s: bias must be 16-byte aligned", name);
+  return AXN_OK;
+}
+
+int check_f32(const char* name, const void* a, const void* b, const void* c,
+              int64_t M, int64_t N, int64_t K) {
+  REQUIRE(a && b && c, AXN_EINVAL, "%s: null operand pointer", name);
+  REQUIRE(M >= 1 && N >= 1 && K >= 1, AXN_EINVAL,
+          "%s: M, N, K must be >= 1 (got %lld, %lld, %lld)", name, (long long)M,
+          (long long)N, (long long)K);
+  REQUIRE(M <= 0x7fffffff && N <= 0x7fffffff && K <= 0x7fffffff, AXN_ELIMIT,
+          "%s: dimension exceeds 2^31-1", name);
+  REQUIRE((((uintptr_t)a | (uintptr_t)b | (uintptr_t)c) & 3u) == 0, AXN_EALIGN,
+          "%s: operand pointers must be 4-byte aligned", name);
+  return AXN_OK;
+}
+
+bool known_dtype(int dt) { return dt == AXN_BF16 || dt == AXN_F16 || dt == AXN_F32; }
+
+int check_list(const char* name, const void* const* h_ptrs, const char* what,
+               const int64_t* h_sizes, int64_t n, int elem_size) {
+  for (int64_t i = 0; i < n; ++i) {
+    if (h_sizes[i] == 0) continue;
+    REQUIRE(h_ptrs[i] != nullptr, AXN_EINVAL, "%s: %s[%lld] is null", name, what,
+            (long long)i);
+    REQUIRE(((uintptr_t)h_ptrs[i] % (uintptr_t)elem_size) == 0, AXN_EALIGN,
+            "%s: %s[%lld] is not aligned to its element size", name, what,
+            (long long)i);
+  }
+  return AXN_OK;
+}
+
+int check_sizes(const char* name, const int64_t* h_sizes, int64_t n) {
+  REQUIRE(n >= 0, AXN_EINVAL, "%s: negative tensor count", name);
+  REQUIRE(n == 0 || h_sizes != nullptr, AXN_EINVAL, "%s: null size array", name);
+  for (int64_t i = 0; i < n; ++i)
+    REQUIRE(h_sizes[i] >= 0, AXN_EINVAL, "%s: sizes[%lld] is negative", name,
+            (long long)i);
+  return AXN_OK;
+}
+
+}  // namespace
+}  // namespace axn
+
+using namespace axn;
+
+extern "C" {
+
+int axn_abi_version(void) { return AXN_ABI_VERSION; }
+
+const char* axn_last_error(void) { return g_err; }
+
+int axn_gemm_fwd(const void* X, const void* W, const float* bias, void* Y,
+                 void* Zsave, int64_t M, int64_t N, int64_t K, int64_t ldx,
+                 int64_t ldw, int64_t ldy, int epilogue, void* stream) {
+  int rc = check_gemm("axn_gemm_fwd", X, W, Y, M, N, K, ldx, ldw, ldy, K, K, N);
+  if (rc) return rc;
+  rc = check_epilogue("axn_gemm_fwd", epilogue, bias);
+  if (rc) return rc;
+  REQUIRE(Zsave == nullptr || aligned16(Zsave), AXN_EALIGN,
+          "axn_gemm_fwd: Zsave must be 16-byte aligned");
+  GemmArgs g = {};
+  g.A = (const uint16_t*)X;
+  g.B = (const uint16_t*)W;
+  g.C = Y;
+  g.bias = bias;
+  g.Z = (uint16_t*)Zsave;
+  g.M = (int)M;
+  g.N = (int)N;
+  g.Kc = (int)K;
+  g.lda = ldx;
+  g.ldb = ldw;
+  g.ldc = ldy;
+  g.beta = 0;
+  return launch_gemm_bf16(GEMM_NT, g, epilogue, false, (hipStream_t)stream);
+}
+
+int axn_gemm_dgrad(const void* dY, const void* W, void* dX, int64_t M, int64_t N,
+                   int64_t K, int64_t lddy, int64_t ldw, int64_t lddx,
+                   void* stream) {
+  int rc = check_gemm("axn_gemm_dgrad", dY, W, dX, M, N, K, lddy, ldw, lddx, N, K, K);
+  if (rc) return rc;
+  GemmArgs g = {};
+  g.A = (const uint16_t*)dY;  // [M][N]: rows of the output, contraction contiguous
+  g.B = (const uint16_t*)W;   // [N][K]: contraction-major
+  g.C = dX;
+  g.M = (int)M;
+  g.N = (int)K;
+  g.Kc = (int)N;
+  g.lda = lddy;
+  g.ldb = ldw;
+  g.ldc = lddx;
+  g.beta = 0;
+  return launch_gemm_bf16(GEMM_NN, g, AXN_EPI_NONE, false, (hipStream_t)stream);
+}
+
+int axn_gemm_wgrad(const void* dY, const void* X, void* dW, int64_t M, int64_t N,
+                   int64_t K, int64_t lddy, int64_t ldx, int64_t lddw, int beta,
+                   int dw_dtype, void* stream) {
+  int rc = check_gemm("axn_gemm_wgrad", dY, X, dW, M, N, K, lddy, ldx, lddw, N, K, K);
+  if (rc) return rc;
+  REQUIRE(beta == 0 || beta == 1, AXN_EINVAL, "axn_gemm_wgrad: beta must be 0 or 1");
+  REQUIRE(dw_dtype == AXN_BF16 || dw_dtype == AXN_F32, AXN_EINVAL,
+          "axn_gemm_wgrad: dW must be bf16 or fp32");
+  GemmArgs g = {};
+  g.A = (const uint16_t*)dY;  // [M][N]: contraction-major, output rows = N
+  g.B = (const uint16_t*)X;   // [M][K]: contraction-major, output cols = K
+  g.C = dW;
+  g.M = (int)N;
+  g.N = (int)K;
+  g.Kc = (int)M;
+  g.lda = lddy;
+  g.ldb = ldx;
+  g.ldc = lddw;
+  g.beta = beta;
+  return launch_gemm_bf16(GEMM_TN, g, AXN_EPI_NONE, dw_dtype == AXN_F32,
+                          (hipStream_t)stream);
+}
+
+size_t axn_dgelu_dbias_workspace_bytes(int64_t M, int64_t N) {
+  return dgelu_dbias_workspace_bytes(M, N);
+}
+
+int axn_dgelu_dbias(const void* dY, const void* Z, void* dZ, int dtype,
+                    float* dbias, int64_t M, int64_t N, int64_t ld, int beta,
+                    void* workspace, size_t workspace_bytes, void* stream) {
+  const char* name = "axn_dgelu_dbias";
+  REQUIRE(dY != nullptr, AXN_EINVAL, "%s: dY is null", name);
+  REQUIRE(dtype == AXN_BF16 || dtype == AXN_F32, AXN_EINVAL,
+          "%s: dtype must be bf16 or fp32", name);
+  REQUIRE(M >= 1 && N >= 1, AXN_EINVAL, "%s: M and N must be >= 1", name);
+  REQUIRE(N % 8 == 0, AXN_ESHAPE, "%s: N must be a multiple of 8", name);
+  REQUIRE(ld >= N && ld % 8 == 0, AXN_EALIGN,
+          "%s: ld must be >= N and a multiple of 8", name);
+  REQUIRE((Z == nullptr) == (dZ == nullptr), AXN_EINVAL,
+          "%s: Z and dZ must be given together", name);
+  REQUIRE(Z != nullptr || dbias != nullptr, AXN_EINVAL, "%s: nothing to compute", name);
+  REQUIRE(aligned16(dY) && aligned16(Z) && aligned16(dZ), AXN_EALIGN,
+          "%s: pointers must be 16-byte aligned", name);
+  REQUIRE(beta == 0 || beta == 1, AXN_EINVAL, "%s: beta must be 0 or 1", name);
+  return launch_dgelu_dbias(dY, Z, dZ, dtype, dbias, M, N, ld, beta, workspace,
+                            workspace_bytes, (hipStream_t)stream);
+}
+
+int axn_gemm_fwd_f32(const float* X, const float* W, const float* bias, float* Y,
+                     float* Zsave, int64_t M, int64_t N, int64_t K, int epilogue,
+                     void* stream) {
+  int rc = check_f32("axn_gemm_fwd_f32", X, W, Y, M, N, K);
+  if (rc) return rc;
+  REQUIRE(epilogue >= AXN_EPI_NONE && epilogue <= AXN_EPI_GELU, AXN_EINVAL,
+          "axn_gemm_fwd_f32: unknown epilogue %d", epilogue);
+  const bool needs_bias = epilogue == AXN_EPI_BIAS || epilogue == AXN_EPI_BIAS_GELU;
+  REQUIRE(!needs_bias || bias != nullptr, AXN_EINVAL,
+          "axn_gemm_fwd_f32: epilogue %d needs a bias vector", epilogue);
+  return launch_gemm_f32(GEMM_NT, X, W, Y, bias, Zsave, (int)M, (int)N, (int)K,
+                         epilogue, 0, (hipStream_t)stream);
+}
+
+int axn_gemm_dgrad_f32(const float* dY, const float* W, float* dX, int64_t M,
+                       int64_t N, int64_t K, void* stream) {
+  int rc = check_f32("axn_gemm_dgrad_f32", dY, W, dX, M, N, K);
+  if (rc) return rc;
+  return launch_gemm_f32(GEMM_NN, dY, W, dX, nullptr, nullptr, (int)M, (int)K,
+                         (int)N, AXN_EPI_NONE, 0, (hipStream_t)stream);
+}
+
+int axn_gemm_wgrad_f32(const float* dY, const float* X, float* dW, int64_t M,
+                       int64_t N, int64_t K, int beta, void* stream) {
+  int rc = check_f32("axn_gemm_wgrad_f32", dY, X, dW, M, N, K);
+  if (rc) return rc;
+  REQUIRE(beta == 0 || beta == 1, AXN_EINVAL, "axn_gemm_wgrad_f32: beta must be 0 or 1");
+  return launch_gemm_f32(GEMM_TN, dY, X, dW, nullptr, nullptr, (int)N, (int)K,
+                         (int)M, AXN_EPI_NONE, beta, (hipStream_t)stream);
+}
+
+size_t axn_mt_scan_workspace_bytes(int64_t n, int64_t total) {
+  return mt_scan_workspace_bytes(n, total);
+}
+
+int axn_mt_scan(const void* const* h_g, const int64_t* h_sizes, int64_t n,
+                int g_dtype, float inv_scale, float max_norm,
+                axn_scan_result* result, void* workspace, size_t workspace_bytes,
+                void* stream) {
+  const char* name = "axn_mt_scan";
+  int rc = check_sizes(name, h_sizes, n);
+  if (rc) return rc;
+  REQUIRE(known_dtype(g_dtype), AXN_EINVAL, "%s: unknown gradient dtype %d", name, g_dtype);
+  REQUIRE(n == 0 || h_g != nullptr, AXN_EINVAL, "%s: null pointer array", name);
+  REQUIRE(result != nullptr, AXN_EINVAL, "%s: result is null", name);
+  REQUIRE(((uintptr_t)result & 7u) == 0, AXN_EALIGN, "%s: result must be 8-byte aligned", name);
+  REQUIRE(workspace != nullptr || workspace_bytes == 0, AXN_EINVAL, "%s: null workspace", name);
+  REQUIRE(((uintptr_t)workspace & 15u) == 0, AXN_EALIGN,
+          "%s: workspace must be 16-byte aligned", name);
+  rc = check_list(name, h_g, "g", h_sizes, n, g_dtype == AXN_F32 ? 4 : 2);
+  if (rc) return rc;
+  return launch_mt_scan(h_g, h_sizes, n, g_dtype, inv_scale, max_norm, result,
+                        workspace, workspace_bytes, (hipStream_t)stream);
+}
+
+int axn_mt_adam(const void* const* h_g, void* const* h_p, void* const* h_m,
+                void* const* h_v, void* const* h_plow, const int64_t* h_sizes,
+                int64_t n, int g_dtype, int plow_dtype, float inv_scale,
+                const axn_scan_result* scan, const axn_adam_hparams* hp,
+                void* stream) {
+  const char* name = "axn_mt_adam";
+  int rc = check_sizes(name, h_sizes, n);
+  if (rc) return rc;
+  REQUIRE(known_dtype(g_dtype), AXN_EINVAL, "%s: unknown gradient dtype %d", name, g_dtype);
+  REQUIRE(h_plow == nullptr || plow_dtype == AXN_BF16 || plow_dtype == AXN_F16,
+          AXN_EINVAL, "%s: low-precision copy must be bf16 or fp16", name);
+  REQUIRE(hp != nullptr, AXN_EINVAL, "%s: hyper-parameters are null", name);
+  REQUIRE(n == 0 || (h_g && h_p && h_m && h_v), AXN_EINVAL, "%s: null pointer array", name);
+  rc = check_list(name, h_g, "g", h_sizes, n, g_dtype == AXN_F32 ? 4 : 2);
+  if (rc) return rc;
+  rc = check_list(name, (const void* const*)h_p, "p", h_sizes, n, 4);
+  if (rc) return rc;
+  rc = check_list(name, (const void* const*)h_m, "m", h_sizes, n, 4);
+  if (rc) return rc;
+  rc = check_list(name, (const void* const*)h_v, "v", h_sizes, n, 4);
+  if (rc) return rc;
+  if (h_plow != nullptr) {
+    rc = check_list(name, (const void* const*)h_plow, "p_lowp", h_sizes, n, 2);
+    if (rc) return rc;
+  }
+  return launch_mt_adam(h_g, h_p, h_m, h_v, h_plow, h_sizes, n, g_dtype,
+                        h_plow ? plow_dtype : AXN_BF16, inv_scale, scan, *hp,
+                        (hipStream_t)stream);
+}
+
+int axn_mt_scale(void* const* h_g, const int64_t* h_sizes, int64_t n, int g_dtype,
+                 float inv_scale, const axn_scan_result* scan, int use_clip,
+                 void* stream) {
+  const char* name = "axn_mt_scale";
+  int rc = check_sizes(name, h_sizes, n);
+  if (rc) return rc;
+  REQUIRE(known_dtype(g_dtype), AXN_EINVAL, "%s: unknown gradient dtype %d", name, g_dtype);
+  REQUIRE(n == 0 || h_g != nullptr, AXN_EINVAL, "%s: null pointer array", name);
+  REQUIRE(!use_clip || scan != nullptr, AXN_EINVAL, "%s: clipping needs a scan result", name);
+  rc = check_list(name, (const void* const*)h_g, "g", h_sizes, n, g_dtype == AXN_F32 ? 4 : 2);
+  if (rc) return rc;
+  return launch_mt_scale(h_g, h_sizes, n, g_dtype, inv_scale, scan, use_clip,
+                         (hipStream_t)stream);
+}
+
+}  // extern "C"

@@ -1,0 +1,71 @@
+// Internal declarations shared by the kernel translation units and the C ABI.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+#include "axn.h"
+
+namespace axn {
+
+// Thread-local error text behind axn_last_error().
+void set_error(const char* fmt, ...);
+int hip_fail(hipError_t e, const char* what);
+
+#define AXN_HIP_TRY(expr)                                  \
+  do {                                                     \
+    hipError_t e__ = (expr);                               \
+    if (e__ != hipSuccess) return ::axn::hip_fail(e__, #expr); \
+  } while (0)
+
+// ---- bf16 GEMM ------------------------------------------------------------
+// C[M x N] (+)= A * B over a contraction of length Kc, bf16 operands, fp32
+// accumulate.  Each operand is either "K-major" (stored [rows][Kc], the
+// contraction index contiguous) or "MN-major" (stored [Kc][rows]).
+struct GemmArgs {
+  const uint16_t* A;
+  const uint16_t* B;
+  void* C;            // bf16 or fp32, row-major [M][N]
+  const float* bias;  // [N] or null
+  uint16_t* Z;        // optional pre-activation copy, bf16 [M][N], ld = ldc
+  int M, N, Kc;
+  int64_t lda, ldb, ldc;
+  int tiles_m, tiles_n;
+  int beta;  // 0: C = AB ; 1: C += AB
+};
+
+enum GemmLayout { GEMM_NT = 0, GEMM_NN = 1, GEMM_TN = 2 };
+// GEMM_NT: A K-major, B K-major   (forward  Y  = X  W^T)
+// GEMM_NN: A K-major, B MN-major  (dgrad    dX = dY W  )
+// GEMM_TN: A MN-major, B MN-major (wgrad    dW = dY^T X)
+
+int launch_gemm_bf16(GemmLayout layout, const GemmArgs& args, int epilogue,
+                     bool out_f32, hipStream_t stream);
+
+// ---- fp32 GEMM (full-precision layers) --------------------------------------
+int launch_gemm_f32(GemmLayout layout, const float* A, const float* B, float* C,
+                    const float* bias, float* Z, int M, int N, int Kc,
+                    int epilogue, int beta, hipStream_t stream);
+
+// ---- elementwise backward of the bias/GELU epilogue ----------------------
+size_t dgelu_dbias_workspace_bytes(int64_t M, int64_t N);
+int launch_dgelu_dbias(const void* dY, const void* Z, void* dZ, int dtype,
+                       float* dbias, int64_t M, int64_t N, int64_t ld, int beta,
+                       void* ws, size_t ws_bytes, hipStream_t stream);
+
+// ---- multi-tensor optimizer ------------------------------------------------
+size_t mt_scan_workspace_bytes(int64_t n, int64_t total);
+int launch_mt_scan(const void* const* h_g, const int64_t* h_sizes, int64_t n,
+                   int g_dtype, float inv_scale, float max_norm,
+                   axn_scan_result* result, void* ws, size_t ws_bytes,
+                   hipStream_t stream);
+int launch_mt_adam(const void* const* h_g, void* const* h_p, void* const* h_m,
+                   void* const* h_v, void* const* h_plow, const int64_t* h_sizes,
+                   int64_t n, int g_dtype, int plow_dtype, float inv_scale,
+                   const axn_scan_result* scan, const axn_adam_hparams& hp,
+                   hipStream_t stream);
+int launch_mt_scale(void* const* h_g, const int64_t* h_sizes, int64_t n,
+                    int g_dtype, float inv_scale, const axn_scan_result* scan,
+                    int use_clip, hipStream_t stream);
+
+}  // namespace axn

@@ -1,0 +1,669 @@
+// Mixed-precision optimizer step for gfx950 (MI355X): multi-tensor, HBM
+// streaming.  Three kernels share one addressing scheme:
+//   mt_scan   one read pass over the low-precision gradients: overflow check
+//             (axonn/inter_layer.py:435-445) + sum of squares of the unscaled
+//             gradients (axonn/intra_layer/gradient_normalization.py:18-34)
+//   mt_adam   one read-modify-write pass: unscale, clip, Adam on the fp32
+//             master weights and moments, low-precision copy of the weights
+//             (axonn/optim.py:157-190)
+//   mt_scale  in-place scaling of the gradients
+//             (axonn/inter_layer.py:458, gradient_normalization.py:88-93)
+//
+// Addressing.  The tensors of one launch (at most MT_MAX) travel in the kernel
+// argument block: pointers, sizes and a prefix sum of per-tensor chunk counts.
+// Workgroup b finds its tensor by binary search in that prefix sum (scalar
+// loads from the argument block) and owns MT_CHUNK consecutive elements of it.
+// Tensors are views into flat buffers at arbitrary element offsets
+// (axonn/utils.py:11-30), so each tensor starts with a scalar "head" of up to 7
+// elements after which every pointer of the tensor is 16-byte aligned; the
+// body is then moved as 16-byte vectors, 8 elements per lane per step.  A
+// tensor whose pointers cannot be aligned by one common head is processed with
+// scalar accesses.
+#include "axn_internal.h"
+
+#include <cmath>
+#include <vector>
+
+namespace axn {
+namespace {
+
+constexpr int MT_MAX = 64;         // tensors per launch
+constexpr int MT_THREADS = 256;    // threads per workgroup
+constexpr int MT_VEC = 8;          // elements per lane per step
+constexpr int MT_UNROLL = 4;       // steps per workgroup per tensor chunk pass
+constexpr int MT_CHUNK = MT_THREADS * MT_VEC * MT_UNROLL * 2;  // 16384 elements
+
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
+
+struct MtTable {
+  const void* g[MT_MAX];
+  void* p[MT_MAX];
+  void* m[MT_MAX];
+  void* v[MT_MAX];
+  void* plow[MT_MAX];
+  int64_t size[MT_MAX];
+  int32_t chunk_start[MT_MAX + 1];  // prefix sum of chunks per tensor
+  uint8_t head[MT_MAX];             // scalar elements before the aligned body
+  uint8_t vec_ok[MT_MAX];           // 0: scalar accesses only
+  int32_t n;
+};
+
+struct ScanPartial {
+  float sumsq;
+  float sum;
+  int32_t nonfinite;
+  int32_t pad;
+};
+
+__device__ __forceinline__ int find_tensor(const MtTable& t, int block) {
+  int lo = 0, hi = t.n;  // chunk_start[lo] <= block < chunk_start[hi]
+  while (hi - lo > 1) {
+    const int mid = (lo + hi) >> 1;
+    if (t.chunk_start[mid] <= block) lo = mid; else hi = mid;
+  }
+  return lo;
+}
+
+template <int DT> struct Lowp;
+template <> struct Lowp<AXN_BF16> {
+  typedef uint16_t raw;
+  __device__ static float to_float(raw x) { return __uint_as_float((uint32_t)x << 16); }
+  __device__ static raw from_float(float f) {
+    return __builtin_bit_cast(uint16_t, (__bf16)f);
+  }
+  __device__ static bool nonfinite(raw x) { return (x & 0x7F80u) == 0x7F80u; }
+};
+template <> struct Lowp<AXN_F16> {
+  typedef uint16_t raw;
+  __device__ static float to_float(raw x) { return (float)__builtin_bit_cast(_Float16, x); }
+  __device__ static raw from_float(float f) {
+    return __builtin_bit_cast(uint16_t, (_Float16)f);
+  }
+  __device__ static bool nonfinite(raw x) { return (x & 0x7C00u) == 0x7C00u; }
+};
+template <> struct Lowp<AXN_F32> {
+  typedef uint32_t raw;
+  __device__ static float to_float(raw x) { return __uint_as_float(x); }
+  __device__ static raw from_float(float f) { return __float_as_uint(f); }
+  __device__ static bool nonfinite(raw x) { return (x & 0x7F800000u) == 0x7F800000u; }
+};
+
+// 8 consecutive low-precision elements from a 16-byte aligned address.
+template <int DT>
+__device__ __forceinline__ void load8(const void* base, int64_t i,
+                                      typename Lowp<DT>::raw (&r)[8]) {
+  typedef typename Lowp<DT>::raw raw;
+  const raw* p = (const raw*)base + i;
+  if (sizeof(raw) == 2) {
+    const u32x4 w = __builtin_nontemporal_load((const u32x4*)p);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      r[2 * e] = (raw)(w[e] & 0xFFFFu);
+      r[2 * e + 1] = (raw)(w[e] >> 16);
+    }
+  } else {
+    const u32x4 w0 = __builtin_nontemporal_load((const u32x4*)p);
+    const u32x4 w1 = __builtin_nontemporal_load((const u32x4*)p + 1);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      r[e] = (raw)w0[e];
+      r[4 + e] = (raw)w1[e];
+    }
+  }
+}
+
+template <int DT>
+__device__ __forceinline__ void store8(void* base, int64_t i,
+                                       const typename Lowp<DT>::raw (&r)[8]) {
+  typedef typename Lowp<DT>::raw raw;
+  raw* p = (raw*)base + i;
+  if (sizeof(raw) == 2) {
+    u32x4 w;
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+      w[e] = (uint32_t)r[2 * e] | ((uint32_t)r[2 * e + 1] << 16);
+    __builtin_nontemporal_store(w, (u32x4*)p);
+  } else {
+    u32x4 w0, w1;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      w0[e] = (uint32_t)r[e];
+      w1[e] = (uint32_t)r[4 + e];
+    }
+    __builtin_nontemporal_store(w0, (u32x4*)p);
+    __builtin_nontemporal_store(w1, (u32x4*)p + 1);
+  }
+}
+
+__device__ __forceinline__ void loadf8(const float* p, float (&x)[8]) {
+  const f32x4 a = __builtin_nontemporal_load((const f32x4*)p);
+  const f32x4 b = __builtin_nontemporal_load((const f32x4*)p + 1);
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    x[e] = a[e];
+    x[4 + e] = b[e];
+  }
+}
+__device__ __forceinline__ void storef8(float* p, const float (&x)[8]) {
+  f32x4 a = {x[0], x[1], x[2], x[3]}, b = {x[4], x[5], x[6], x[7]};
+  __builtin_nontemporal_store(a, (f32x4*)p);
+  __builtin_nontemporal_store(b, (f32x4*)p + 1);
+}
+
+// Element range [begin, end) of tensor `t` owned by chunk `c`.  Chunk 0 also
+// owns the scalar head [0, head).
+struct Range {
+  int64_t begin, end;
+};
+__device__ __forceinline__ Range chunk_range(const MtTable& tab, int t, int c) {
+  const int64_t head = tab.head[t];
+  Range r;
+  r.begin = head + (int64_t)c * MT_CHUNK;
+  r.end = r.begin + MT_CHUNK;
+  if (r.end > tab.size[t]) r.end = tab.size[t];
+  if (r.begin > r.end) r.begin = r.end;
+  return r;
+}
+
+// ---------------------------------------------------------------- scan ------
+__device__ __forceinline__ float wave_sum(float x) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) x += __shfl_xor(x, o, 64);
+  return x;
+}
+__device__ __forceinline__ int wave_or(int x) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) x |= __shfl_xor(x, o, 64);
+  return x;
+}
+
+template <int DT>
+__global__ void __launch_bounds__(MT_THREADS)
+    mt_scan_kernel(const MtTable tab, float inv_scale, ScanPartial* partial,
+                   int block_base) {
+  typedef typename Lowp<DT>::raw raw;
+  const int t = find_tensor(tab, blockIdx.x);
+  const int c = blockIdx.x - tab.chunk_start[t];
+  const Range rg = chunk_range(tab, t, c);
+  const void* g = tab.g[t];
+  const int tid = threadIdx.x;
+
+  float sq = 0.f, sm = 0.f;
+  int bad = 0;
+  auto one = [&](raw x) {
+    bad |= Lowp<DT>::nonfinite(x) ? 1 : 0;
+    const float f = Lowp<DT>::to_float(x);
+    sm += f;
+    const float u = f * inv_scale;
+    sq += u * u;
+  };
+  if (tab.vec_ok[t]) {
+    if (c == 0 && tid < tab.head[t]) one(((const raw*)g)[tid]);
+    const int64_t nvec = (rg.end - rg.begin) / MT_VEC;
+    for (int64_t i = tid; i < nvec; i += MT_THREADS) {
+      raw r[8];
+      load8<DT>(g, rg.begin + i * MT_VEC, r);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) one(r[e]);
+    }
+    const int64_t tail = rg.begin + nvec * MT_VEC;
+    if (tail + tid < rg.end) one(((const raw*)g)[tail + tid]);
+  } else {
+    const int64_t b = (c == 0) ? 0 : rg.begin;
+    for (int64_t i = b + tid; i < rg.end; i += MT_THREADS) one(((const raw*)g)[i]);
+  }
+
+  __shared__ float s_sq[MT_THREADS / 64], s_sm[MT_THREADS / 64];
+  __shared__ int s_bad[MT_THREADS / 64];
+  sq = wave_sum(sq);
+  sm = wave_sum(sm);
+  bad = wave_or(bad);
+  if ((tid & 63) == 0) {
+    s_sq[tid >> 6] = sq;
+    s_sm[tid >> 6] = sm;
+    s_bad[tid >> 6] = bad;
+  }
+  __syncthreads();
+  if (tid == 0) {
+    ScanPartial p;
+    p.sumsq = (s_sq[0] + s_sq[1]) + (s_sq[2] + s_sq[3]);
+    p.sum = (s_sm[0] + s_sm[1]) + (s_sm[2] + s_sm[3]);
+    p.nonfinite = s_bad[0] | s_bad[1] | s_bad[2] | s_bad[3];
+    p.pad = 0;
+    partial[block_base + blockIdx.x] = p;
+  }
+}
+
+__device__ __forceinline__ double wave_sum_d(double x) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) x += __shfl_xor(x, o, 64);
+  return x;
+}
+
+// One workgroup of 1024 threads reduces the partials of one launch group in a
+// fixed order: wave w takes tensors w, w + 16, ...; lanes stride over that
+// tensor's chunks.  `first` initialises the result, later groups accumulate.
+__global__ void __launch_bounds__(1024)
+    mt_scan_finalize_kernel(const MtTable tab, const ScanPartial* partial,
+                            int block_base, double sum_limit, float max_norm,
+                            int first, axn_scan_result* out) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  __shared__ double s_sq[16];
+  __shared__ int s_bad[16];
+  double sq = 0.0;
+  int bad = 0;
+  for (int t = wave; t < tab.n; t += 16) {
+    double tsq = 0.0, tsm = 0.0;
+    int tbad = 0;
+    for (int b = tab.chunk_start[t] + lane; b < tab.chunk_start[t + 1]; b += 64) {
+      const ScanPartial p = partial[block_base + b];
+      tsq += (double)p.sumsq;
+      tsm += (double)p.sum;
+      tbad |= p.nonfinite;
+    }
+    tsq = wave_sum_d(tsq);
+    tsm = wave_sum_d(tsm);
+    tbad = wave_or(tbad);
+    // The tensor's sum, rounded to the gradient dtype, is non-finite.
+    if (!(fabs(tsm) < sum_limit)) tbad = 1;
+    sq += tsq;
+    bad |= tbad;
+  }
+  if (lane == 0) {
+    s_sq[wave] = sq;
+    s_bad[wave] = bad;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    double total = first ? 0.0 : out->sumsq;
+    int flag = first ? 0 : out->found_inf;
+    for (int w = 0; w < 16; ++w) {
+      total += s_sq[w];
+      flag |= s_bad[w];
+    }
+    const float norm = (float)sqrt(total);
+    float coef = 1.0f;
+    if (max_norm > 0.0f) {
+      coef = max_norm / (norm + 1e-6f);
+      if (coef > 1.0f) coef = 1.0f;  // a NaN coefficient stays NaN, as torch.clamp keeps it
+    }
+    out->sumsq = total;
+    out->total_norm = norm;
+    out->clip_coef = coef;
+    out->found_inf = flag;
+    out->reserved[0] = out->reserved[1] = out->reserved[2] = 0;
+  }
+}
+
+// ---------------------------------------------------------------- adam ------
+struct AdamScalars {
+  axn_adam_hparams hp;
+  float inv_scale;
+};
+
+__device__ __forceinline__ void adam_math(float g, float& p, float& m, float& v,
+                                          const AdamScalars& s, float gmul) {
+  g = g * s.inv_scale;
+  g = g * gmul;
+  if (s.hp.weight_decay != 0.0f) g = g + s.hp.weight_decay * p;
+  m = m + (g - m) * s.hp.one_minus_beta1;
+  v = v * s.hp.beta2 + s.hp.one_minus_beta2 * g * g;
+  const float denom = sqrtf(v) * s.hp.inv_sqrt_bc2 + s.hp.eps;
+  p = p - s.hp.lr_over_bc1 * (m / denom);
+}
+
+template <int GDT, int PDT, bool HAS_PLOW>
+__global__ void __launch_bounds__(MT_THREADS)
+    mt_adam_kernel(const MtTable tab, const AdamScalars s,
+                   const axn_scan_result* scan) {
+  typedef typename Lowp<GDT>::raw graw;
+  typedef typename Lowp<PDT>::raw praw;
+  float gmul = 1.0f;
+  if (scan != nullptr) {
+    if (scan->found_inf != 0) return;  // overflow: the whole step is skipped
+    gmul = scan->clip_coef;
+  }
+  const int t = find_tensor(tab, blockIdx.x);
+  const int c = blockIdx.x - tab.chunk_start[t];
+  const Range rg = chunk_range(tab, t, c);
+  const void* g = tab.g[t];
+  float* p = (float*)tab.p[t];
+  float* m = (float*)tab.m[t];
+  float* v = (float*)tab.v[t];
+  void* plow = tab.plow[t];
+  const int tid = threadIdx.x;
+
+  auto one = [&](int64_t i) {
+    float pp = p[i], mm = m[i], vv = v[i];
+    adam_math(Lowp<GDT>::to_float(((const graw*)g)[i]), pp, mm, vv, s, gmul);
+    p[i] = pp;
+    m[i] = mm;
+    v[i] = vv;
+    if (HAS_PLOW) ((praw*)plow)[i] = Lowp<PDT>::from_float(pp);
+  };
+
+  if (tab.vec_ok[t]) {
+    if (c == 0 && tid < tab.head[t]) one(tid);
+    const int64_t nvec = (rg.end - rg.begin) / MT_VEC;
+    int64_t i = tid;
+    // Main body: MT_UNROLL independent vectors per lane in flight.
+    for (; i + (MT_UNROLL - 1) * MT_THREADS < nvec; i += MT_UNROLL * MT_THREADS) {
+      graw gr[MT_UNROLL][8];
+      float pp[MT_UNROLL][8], mm[MT_UNROLL][8], vv[MT_UNROLL][8];
+#pragma unroll
+      for (int u = 0; u < MT_UNROLL; ++u) {
+        const int64_t e0 = rg.begin + (i + u * MT_THREADS) * MT_VEC;
+        load8<GDT>(g, e0, gr[u]);
+        loadf8(p + e0, pp[u]);
+        loadf8(m + e0, mm[u]);
+        loadf8(v + e0, vv[u]);
+      }
+#pragma unroll
+      for (int u = 0; u < MT_UNROLL; ++u) {
+        const int64_t e0 = rg.begin + (i + u * MT_THREADS) * MT_VEC;
+        praw pl[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          adam_math(Lowp<GDT>::to_float(gr[u][e]), pp[u][e], mm[u][e], vv[u][e], s, gmul);
+          if (HAS_PLOW) pl[e] = Lowp<PDT>::from_float(pp[u][e]);
+        }
+        storef8(p + e0, pp[u]);
+        storef8(m + e0, mm[u]);
+        storef8(v + e0, vv[u]);
+        if (HAS_PLOW) store8<PDT>(plow, e0, pl);
+      }
+    }
+    for (; i < nvec; i += MT_THREADS) {
+      const int64_t e0 = rg.begin + i * MT_VEC;
+      graw gr[8];
+      float pp[8], mm[8], vv[8];
+      praw pl[8];
+      load8<GDT>(g, e0, gr);
+      loadf8(p + e0, pp);
+      loadf8(m + e0, mm);
+      loadf8(v + e0, vv);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        adam_math(Lowp<GDT>::to_float(gr[e]), pp[e], mm[e], vv[e], s, gmul);
+        if (HAS_PLOW) pl[e] = Lowp<PDT>::from_float(pp[e]);
+      }
+      storef8(p + e0, pp);
+      storef8(m + e0, mm);
+      storef8(v + e0, vv);
+      if (HAS_PLOW) store8<PDT>(plow, e0, pl);
+    }
+    const int64_t tail = rg.begin + nvec * MT_VEC;
+    if (tail + tid < rg.end) one(tail + tid);
+  } else {
+    const int64_t b = (c == 0) ? 0 : rg.begin;
+    for (int64_t i = b + tid; i < rg.end; i += MT_THREADS) one(i);
+  }
+}
+
+// --------------------------------------------------------------- scale ------
+template <int DT>
+__global__ void __launch_bounds__(MT_THREADS)
+    mt_scale_kernel(const MtTable tab, float inv_scale,
+                    const axn_scan_result* scan, int use_clip) {
+  typedef typename Lowp<DT>::raw raw;
+  const float coef = use_clip ? scan->clip_coef : 1.0f;
+  const int t = find_tensor(tab, blockIdx.x);
+  const int c = blockIdx.x - tab.chunk_start[t];
+  const Range rg = chunk_range(tab, t, c);
+  void* g = const_cast<void*>(tab.g[t]);
+  const int tid = threadIdx.x;
+  // Two roundings, as the reference's separate div_ and mul_ passes make.
+  auto f = [&](raw x) -> raw {
+    raw y = Lowp<DT>::from_float(Lowp<DT>::to_float(x) * inv_scale);
+    if (use_clip) y = Lowp<DT>::from_float(Lowp<DT>::to_float(y) * coef);
+    return y;
+  };
+  if (tab.vec_ok[t]) {
+    if (c == 0 && tid < tab.head[t]) ((raw*)g)[tid] = f(((raw*)g)[tid]);
+    const int64_t nvec = (rg.end - rg.begin) / MT_VEC;
+    for (int64_t i = tid; i < nvec; i += MT_THREADS) {
+      raw r[8];
+      load8<DT>(g, rg.begin + i * MT_VEC, r);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) r[e] = f(r[e]);
+      store8<DT>(g, rg.begin + i * MT_VEC, r);
+    }
+    const int64_t tail = rg.begin + nvec * MT_VEC;
+    if (tail + tid < rg.end) ((raw*)g)[tail + tid] = f(((raw*)g)[tail + tid]);
+  } else {
+    const int64_t b = (c == 0) ? 0 : rg.begin;
+    for (int64_t i = b + tid; i < rg.end; i += MT_THREADS) ((raw*)g)[i] = f(((raw*)g)[i]);
+  }
+}
+
+// ------------------------------------------------------------- host side ----
+int dtype_size(int dt) { return dt == AXN_F32 ? 4 : 2; }
+
+// Number of leading scalar elements after which every given pointer of a
+// tensor is 16-byte aligned, or -1 when no common count exists.  The pointer
+// with the narrowest element decides the count; the others must agree.
+int common_head(const void* const* ptrs, const int* elem_sizes, int count) {
+  int best = 0;
+  for (int i = 0; i < count; ++i) {
+    if (ptrs[i] == nullptr) continue;
+    const uintptr_t a = (uintptr_t)ptrs[i];
+    const int es = elem_sizes[i];
+    if (a % es != 0) return -1;
+    const int h = (int)(((16 - a % 16) % 16) / es);
+    if (h > best) best = h;
+  }
+  for (int i = 0; i < count; ++i) {
+    if (ptrs[i] == nullptr) continue;
+    const uintptr_t a = (uintptr_t)ptrs[i] + (uintptr_t)best * elem_sizes[i];
+    if (a % 16 != 0) return -1;
+  }
+  return best;
+}
+
+struct Group {
+  MtTable tab;
+  int blocks;
+};
+
+// Splits the tensor list into launch groups and fills the argument tables.
+// `ptr_sets[k][i]` is pointer k of tensor i (k = 0 is always the gradient).
+int build_groups(const void* const* const* ptr_sets, const int* elem_sizes,
+                 int nsets, const int64_t* h_sizes, int64_t n,
+                 std::vector<Group>& out) {
+  out.clear();
+  Group cur;
+  cur.tab = MtTable();
+  cur.blocks = 0;
+  int k = 0;
+  auto flush = [&]() {
+    if (k == 0) return;
+    cur.tab.n = k;
+    cur.tab.chunk_start[k] = cur.blocks;
+    out.push_back(cur);
+    cur.tab = MtTable();
+    cur.blocks = 0;
+    k = 0;
+  };
+  for (int64_t i = 0; i < n; ++i) {
+    const int64_t sz = h_sizes[i];
+    if (sz == 0) continue;
+    const void* ptrs[5] = {nullptr, nullptr, nullptr, nullptr, nullptr};
+    for (int s = 0; s < nsets; ++s) ptrs[s] = ptr_sets[s] ? ptr_sets[s][i] : nullptr;
+    int head = common_head(ptrs, elem_sizes, nsets);
+    const bool vec_ok = head >= 0;
+    if (!vec_ok) head = 0;
+    if (head > sz) head = (int)sz;
+    const int64_t body = sz - head;
+    int64_t chunks = (body + MT_CHUNK - 1) / MT_CHUNK;
+    if (chunks == 0) chunks = 1;  // the head still needs a workgroup
+    if (chunks > 0x3fffffff) {
+      set_error("multi-tensor: tensor %lld has too many elements (%lld)",
+                (long long)i, (long long)sz);
+      return AXN_ELIMIT;
+    }
+    if (k == MT_MAX || (long long)cur.blocks + chunks > 0x7fffffffLL) flush();
+    cur.tab.g[k] = ptrs[0];
+    cur.tab.p[k] = const_cast<void*>(ptrs[1]);
+    cur.tab.m[k] = const_cast<void*>(ptrs[2]);
+    cur.tab.v[k] = const_cast<void*>(ptrs[3]);
+    cur.tab.plow[k] = const_cast<void*>(ptrs[4]);
+    cur.tab.size[k] = sz;
+    cur.tab.chunk_start[k] = cur.blocks;
+    cur.tab.head[k] = (uint8_t)head;
+    cur.tab.vec_ok[k] = vec_ok ? 1 : 0;
+    cur.blocks += (int)chunks;
+    ++k;
+  }
+  flush();
+  return AXN_OK;
+}
+
+double sum_limit_of(int dt) {
+  // Smallest magnitude that rounds (to nearest even) to infinity in the dtype.
+  switch (dt) {
+    case AXN_F16: return 65520.0;
+    case AXN_BF16: return 3.3961775292304601e38;   // 2^127 * (2 - 2^-8)
+    default: return 3.4028235677973366e38;         // 2^127 * (2 - 2^-24)
+  }
+}
+
+}  // namespace
+
+size_t mt_scan_workspace_bytes(int64_t n, int64_t total) {
+  if (n < 0 || total < 0) return 0;
+  // One partial per chunk; a tensor adds at most one ragged chunk.
+  const int64_t blocks = total / MT_CHUNK + 2 * n + 1;
+  return (size_t)blocks * sizeof(ScanPartial);
+}
+
+int launch_mt_scan(const void* const* h_g, const int64_t* h_sizes, int64_t n,
+                   int g_dtype, float inv_scale, float max_norm,
+                   axn_scan_result* result, void* ws, size_t ws_bytes,
+                   hipStream_t stream) {
+  const void* const* sets[1] = {h_g};
+  const int es[1] = {dtype_size(g_dtype)};
+  std::vector<Group> groups;
+  int rc = build_groups(sets, es, 1, h_sizes, n, groups);
+  if (rc != AXN_OK) return rc;
+  int64_t need = 0;
+  for (auto& gr : groups) need += gr.blocks;
+  if ((size_t)need * sizeof(ScanPartial) > ws_bytes) {
+    set_error("mt_scan: workspace too small (%zu bytes given, %zu needed)",
+              ws_bytes, (size_t)need * sizeof(ScanPartial));
+    return AXN_EINVAL;
+  }
+  ScanPartial* partial = (ScanPartial*)ws;
+  if (groups.empty()) {
+    // Nothing to scan: norm 0, no overflow.
+    MtTable empty = MtTable();
+    empty.n = 0;
+    hipLaunchKernelGGL(mt_scan_finalize_kernel, dim3(1), dim3(1024), 0, stream,
+                       empty, partial, 0, sum_limit_of(g_dtype), max_norm, 1, result);
+    AXN_HIP_TRY(hipGetLastError());
+    return AXN_OK;
+  }
+  int base = 0;
+  bool first = true;
+  for (auto& gr : groups) {
+    switch (g_dtype) {
+      case AXN_BF16:
+        hipLaunchKernelGGL(mt_scan_kernel<AXN_BF16>, dim3(gr.blocks), dim3(MT_THREADS),
+                           0, stream, gr.tab, inv_scale, partial, base);
+        break;
+      case AXN_F16:
+        hipLaunchKernelGGL(mt_scan_kernel<AXN_F16>, dim3(gr.blocks), dim3(MT_THREADS),
+                           0, stream, gr.tab, inv_scale, partial, base);
+        break;
+      default:
+        hipLaunchKernelGGL(mt_scan_kernel<AXN_F32>, dim3(gr.blocks), dim3(MT_THREADS),
+                           0, stream, gr.tab, inv_scale, partial, base);
+        break;
+    }
+    AXN_HIP_TRY(hipGetLastError());
+    hipLaunchKernelGGL(mt_scan_finalize_kernel, dim3(1), dim3(1024), 0, stream,
+                       gr.tab, partial, base, sum_limit_of(g_dtype), max_norm,
+                       first ? 1 : 0, result);
+    AXN_HIP_TRY(hipGetLastError());
+    base += gr.blocks;
+    first = false;
+  }
+  return AXN_OK;
+}
+
+template <int GDT>
+int adam_dispatch(const Group& gr, const AdamScalars& s, int plow_dtype,
+                  bool has_plow, const axn_scan_result* scan, hipStream_t stream) {
+  const dim3 grid(gr.blocks), block(MT_THREADS);
+  if (!has_plow) {
+    hipLaunchKernelGGL((mt_adam_kernel<GDT, AXN_BF16, false>), grid, block, 0,
+                       stream, gr.tab, s, scan);
+  } else if (plow_dtype == AXN_BF16) {
+    hipLaunchKernelGGL((mt_adam_kernel<GDT, AXN_BF16, true>), grid, block, 0,
+                       stream, gr.tab, s, scan);
+  } else {
+    hipLaunchKernelGGL((mt_adam_kernel<GDT, AXN_F16, true>), grid, block, 0,
+                       stream, gr.tab, s, scan);
+  }
+  AXN_HIP_TRY(hipGetLastError());
+  return AXN_OK;
+}
+
+int launch_mt_adam(const void* const* h_g, void* const* h_p, void* const* h_m,
+                   void* const* h_v, void* const* h_plow, const int64_t* h_sizes,
+                   int64_t n, int g_dtype, int plow_dtype, float inv_scale,
+                   const axn_scan_result* scan, const axn_adam_hparams& hp,
+                   hipStream_t stream) {
+  const void* const* sets[5] = {h_g, (const void* const*)h_p, (const void* const*)h_m,
+                                (const void* const*)h_v, (const void* const*)h_plow};
+  const int es[5] = {dtype_size(g_dtype), 4, 4, 4, dtype_size(plow_dtype)};
+  std::vector<Group> groups;
+  int rc = build_groups(sets, es, 5, h_sizes, n, groups);
+  if (rc != AXN_OK) return rc;
+  AdamScalars s;
+  s.hp = hp;
+  s.inv_scale = inv_scale;
+  const bool has_plow = h_plow != nullptr;
+  for (auto& gr : groups) {
+    switch (g_dtype) {
+      case AXN_BF16: rc = adam_dispatch<AXN_BF16>(gr, s, plow_dtype, has_plow, scan, stream); break;
+      case AXN_F16: rc = adam_dispatch<AXN_F16>(gr, s, plow_dtype, has_plow, scan, stream); break;
+      default: rc = adam_dispatch<AXN_F32>(gr, s, plow_dtype, has_plow, scan, stream); break;
+    }
+    if (rc != AXN_OK) return rc;
+  }
+  return AXN_OK;
+}
+
+int launch_mt_scale(void* const* h_g, const int64_t* h_sizes, int64_t n,
+                    int g_dtype, float inv_scale, const axn_scan_result* scan,
+                    int use_clip, hipStream_t stream) {
+  const void* const* sets[1] = {(const void* const*)h_g};
+  const int es[1] = {dtype_size(g_dtype)};
+  std::vector<Group> groups;
+  int rc = build_groups(sets, es, 1, h_sizes, n, groups);
+  if (rc != AXN_OK) return rc;
+  for (auto& gr : groups) {
+    const dim3 grid(gr.blocks), block(MT_THREADS);
+    switch (g_dtype) {
+      case AXN_BF16:
+        hipLaunchKernelGGL(mt_scale_kernel<AXN_BF16>, grid, block, 0, stream,
+                           gr.tab, inv_scale, scan, use_clip);
+        break;
+      case AXN_F16:
+        hipLaunchKernelGGL(mt_scale_kernel<AXN_F16>, grid, block, 0, stream,
+                           gr.tab, inv_scale, scan, use_clip);
+        break;
+      default:
+        hipLaunchKernelGGL(mt_scale_kernel<AXN_F32>, grid, block, 0, stream,
+                           gr.tab, inv_scale, scan, use_clip);
+        break;
+    }
+    AXN_HIP_TRY(hipGetLastError());
+  }
+  return AXN_OK;
+}
+
+}  // namespace axn

@@ -1,0 +1,210 @@
+/*
+ * axn.h - C ABI of libaxn_gfx950.so: the per-GPU training hot path of AxoNN's
+ * tensor-parallel Linear layer and mixed-precision optimizer step, as
+ * hand-written gfx950 (MI355X, CDNA4) kernels.
+ *
+ * The reference (axonn-ai/axonn) is pure Python and has no FFI of its own; its seam
+ * is the torch.autograd.Function / torch.optim.Optimizer protocol.  Each entry
+ * point below replaces the torch call(s) the reference makes at the cited
+ * file:line (paths relative to the reference checkout).
+ *
+ * Conventions
+ *   - Every pointer is a DEVICE pointer unless the parameter name starts with
+ *     "h_" (host array).  The library never frees or retains caller memory.
+ *   - Every call is asynchronous on the hipStream_t passed as `stream`
+ *     (void*; NULL = the default stream).  No call synchronises the device.
+ *   - Return value: AXN_OK (0) or a negative axn_status.  axn_last_error()
+ *     returns a thread-local description of the last failure on this thread.
+ *   - Argument validation happens before any HIP call, so bad-argument
+ *     behaviour is testable on a host without a GPU.
+ *   - Matrices are row-major.  "ld*" are row strides in ELEMENTS.
+ *   - bf16 = bfloat16 stored as uint16_t, fp32 accumulate everywhere.
+ */
+#ifndef AXN_H_
+#define AXN_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define AXN_ABI_VERSION 1
+
+#if defined(__GNUC__)
+#define AXN_API __attribute__((visibility("default")))
+#else
+#define AXN_API
+#endif
+
+typedef enum axn_status {
+  AXN_OK = 0,
+  AXN_EINVAL = -1, /* null pointer, negative size, unknown enum value      */
+  AXN_EALIGN = -2, /* pointer or leading dimension not aligned as required */
+  AXN_ESHAPE = -3, /* shape not supported by the kernels                   */
+  AXN_EHIP = -4,   /* a HIP runtime call failed (message has the detail)   */
+  AXN_ELIMIT = -5  /* size exceeds a documented limit of the entry point   */
+} axn_status;
+
+typedef enum axn_dtype {
+  AXN_BF16 = 0,
+  AXN_F16 = 1,
+  AXN_F32 = 2
+} axn_dtype;
+
+/* Epilogue fused into the forward GEMM. */
+typedef enum axn_epilogue {
+  AXN_EPI_NONE = 0,      /* Y = X W^T                                 */
+  AXN_EPI_BIAS = 1,      /* Y = X W^T + b                             */
+  AXN_EPI_BIAS_GELU = 2, /* Z = X W^T + b ; Y = gelu(Z) (exact erf)   */
+  AXN_EPI_GELU = 3       /* Z = X W^T     ; Y = gelu(Z)               */
+} axn_epilogue;
+
+AXN_API int axn_abi_version(void);
+AXN_API const char* axn_last_error(void);
+
+/* ------------------------------------------------------------------------
+ * Linear layer: the three shard GEMMs.
+ * M = tokens, K = local in_features, N = local out_features.
+ * Requirements (else AXN_ESHAPE / AXN_EALIGN): M,N,K >= 1; N % 8 == 0 and
+ * K % 8 == 0; all pointers 16-byte aligned; every ld a multiple of 8.
+ * ------------------------------------------------------------------------ */
+
+/* Forward.  Replaces `input_.matmul(weight.t())`
+ * (axonn/intra_layer/fully_connected.py:118) and the separate broadcast
+ * `x + bias` (fully_connected.py:348); the GELU the reference's callers place
+ * after the layer (docs/user_guide.rst:120) can be fused as well.
+ *   X [M,K] bf16, W [N,K] bf16, bias [N] fp32 or NULL,
+ *   Y [M,N] bf16, Zsave [M,N] bf16 or NULL (pre-activation, saved for
+ *   axn_dgelu_dbias when a GELU epilogue is used; same ld as Y). */
+AXN_API int axn_gemm_fwd(const void* X, const void* W, const float* bias, void* Y,
+                 void* Zsave, int64_t M, int64_t N, int64_t K, int64_t ldx,
+                 int64_t ldw, int64_t ldy, int epilogue, void* stream);
+
+/* Input gradient.  Replaces `grad_output.matmul(weight)`
+ * (fully_connected.py:140 and :186).
+ *   dY [M,N] bf16, W [N,K] bf16, dX [M,K] bf16. */
+AXN_API int axn_gemm_dgrad(const void* dY, const void* W, void* dX, int64_t M,
+                   int64_t N, int64_t K, int64_t lddy, int64_t ldw,
+                   int64_t lddx, void* stream);
+
+/* Weight gradient.  Replaces
+ * `grad_output.reshape(-1,N).t().mm(input_.view(-1,K))`
+ * (fully_connected.py:147-151 and :171-175) and, with beta = 1, the
+ * accumulation `param.grad.add_(grad)` across micro-batches
+ * (axonn/intra_layer/overlap_communication.py:42-45 / autograd AccumulateGrad).
+ *   dY [M,N] bf16, X [M,K] bf16, dW [N,K] of dw_dtype (AXN_BF16 or AXN_F32),
+ *   dW = beta * dW + dY^T X  with beta in {0, 1}. */
+AXN_API int axn_gemm_wgrad(const void* dY, const void* X, void* dW, int64_t M,
+                   int64_t N, int64_t K, int64_t lddy, int64_t ldx,
+                   int64_t lddw, int beta, int dw_dtype, void* stream);
+
+/* Backward of the fused bias/GELU epilogue, one pass over [M,N]:
+ *   dZ = dY * gelu'(Z)   (Z = NULL: dZ is not written, dbias = colsum(dY))
+ *   dbias[n] = beta * dbias[n] + sum_m dZ[m,n]        (dbias NULL: skipped)
+ * Replaces what autograd derives from `x + bias` (fully_connected.py:348)
+ * and from the caller's nn.GELU.  dY, Z, dZ are of `dtype` (AXN_BF16 or
+ * AXN_F32), row stride ld; dbias is fp32.  N % 8 == 0, pointers 16-byte
+ * aligned, ld % 8 == 0.  Deterministic: column partial sums go through
+ * `workspace` (axn_dgelu_dbias_workspace_bytes, needed only when dbias is
+ * given) and are reduced in a fixed order.  dZ may alias dY. */
+AXN_API int axn_dgelu_dbias(const void* dY, const void* Z, void* dZ, int dtype,
+                    float* dbias, int64_t M, int64_t N, int64_t ld, int beta,
+                    void* workspace, size_t workspace_bytes, void* stream);
+AXN_API size_t axn_dgelu_dbias_workspace_bytes(int64_t M, int64_t N);
+
+/* fp32 variants of the three GEMMs for full-precision layers (the reference's
+ * own tests run the layer in fp32: axonn/tests/test_intra_layer_fc.py:25).
+ * Same argument meaning as above with fp32 operands and results; bias fp32.
+ * Any M,N,K >= 1, pointers 4-byte aligned. */
+AXN_API int axn_gemm_fwd_f32(const float* X, const float* W, const float* bias,
+                     float* Y, float* Zsave, int64_t M, int64_t N, int64_t K,
+                     int epilogue, void* stream);
+AXN_API int axn_gemm_dgrad_f32(const float* dY, const float* W, float* dX, int64_t M,
+                       int64_t N, int64_t K, void* stream);
+AXN_API int axn_gemm_wgrad_f32(const float* dY, const float* X, float* dW, int64_t M,
+                       int64_t N, int64_t K, int beta, void* stream);
+
+/* ------------------------------------------------------------------------
+ * Mixed-precision optimizer step over a list of tensors (multi-tensor).
+ * The tensor list is given as host arrays of device pointers and element
+ * counts; tensors may be views into one flat buffer at arbitrary element
+ * offsets (axonn/utils.py:11-30), so only natural alignment is required.
+ * ------------------------------------------------------------------------ */
+
+/* Device-resident result of the gradient scan, consumed by axn_mt_adam and
+ * axn_mt_scale without a host round trip.  32 bytes. */
+typedef struct axn_scan_result {
+  double sumsq;       /* sum over all tensors of (g * inv_scale)^2            */
+  float total_norm;   /* sqrt(sumsq)                                          */
+  float clip_coef;    /* min(1, max_norm / (total_norm + 1e-6)); 1 if no clip */
+  int32_t found_inf;  /* 1 if the overflow check fired, else 0                */
+  int32_t reserved[3];
+} axn_scan_result;
+
+/* Scratch bytes axn_mt_scan needs for `n` tensors of `total` elements. */
+AXN_API size_t axn_mt_scan_workspace_bytes(int64_t n, int64_t total);
+
+/* One read pass over the gradients.  Replaces, fused:
+ *   - the overflow test `s = tensor.sum(); isinf(s) + isnan(s) > 0` applied
+ *     per tensor to the scaled low-precision gradients
+ *     (axonn/inter_layer.py:435-445 called from :455, and optim.py:161):
+ *     found_inf = OR over tensors of [the tensor's sum, rounded to g_dtype,
+ *     is non-finite]; any inf/nan element makes its tensor's sum non-finite;
+ *   - the global gradient 2-norm of the unscaled gradients and the clip
+ *     coefficient (axonn/intra_layer/gradient_normalization.py:18-34, :86-87).
+ *   h_g[n]: device pointers to gradients of g_dtype (BF16, F16 or F32);
+ *   h_sizes[n]: element counts; inv_scale = 1 / loss_scale;
+ *   max_norm <= 0 disables clipping (clip_coef = 1).
+ *   result: device axn_scan_result, fully overwritten. */
+AXN_API int axn_mt_scan(const void* const* h_g, const int64_t* h_sizes, int64_t n,
+                int g_dtype, float inv_scale, float max_norm,
+                axn_scan_result* result, void* workspace,
+                size_t workspace_bytes, void* stream);
+
+/* Scalar hyper-parameters of one Adam step.  The bias corrections are
+ * computed by the caller in double precision, as torch does
+ * (torch/optim/adam.py::_single_tensor_adam, reached from
+ * axonn/optim.py:168-182). */
+typedef struct axn_adam_hparams {
+  float lr_over_bc1;     /* lr / (1 - beta1^t)            */
+  float inv_sqrt_bc2;    /* 1 / sqrt(1 - beta2^t)         */
+  float beta1;
+  float one_minus_beta1;
+  float beta2;
+  float one_minus_beta2;
+  float eps;
+  float weight_decay;    /* L2 form: g += weight_decay * p */
+} axn_adam_hparams;
+
+/* One streaming pass: for every element
+ *   g  = float(g_lowp) * inv_scale * clip_coef          (optim.py:157-160,
+ *                                      gradient_normalization.py:88-93)
+ *   g += weight_decay * p
+ *   m += (g - m) * (1 - beta1);  v = v * beta2 + (1 - beta2) * g * g
+ *   p -= lr_over_bc1 * m / (sqrt(v) * inv_sqrt_bc2 + eps)       (optim.py:168-182)
+ *   p_lowp = round_to_nearest_even(p)                            (optim.py:183-185)
+ * `scan` may be NULL (no overflow gate, clip_coef = 1); otherwise, when
+ * scan->found_inf != 0 NOTHING is written (the whole step is skipped on the
+ * device, axonn/inter_layer.py:428-430), and scan->clip_coef is applied.
+ *   h_g/h_p/h_m/h_v/h_plow[n]: device pointers; h_plow may be NULL (no
+ *   low-precision copy) ; p, m, v are fp32. */
+AXN_API int axn_mt_adam(const void* const* h_g, void* const* h_p, void* const* h_m,
+                void* const* h_v, void* const* h_plow, const int64_t* h_sizes,
+                int64_t n, int g_dtype, int plow_dtype, float inv_scale,
+                const axn_scan_result* scan, const axn_adam_hparams* hp,
+                void* stream);
+
+/* In-place g = g * inv_scale * (use_clip ? scan->clip_coef : 1) on every
+ * tensor, in g_dtype.  Replaces `p.grad.div_(loss_scale)`
+ * (axonn/inter_layer.py:458) and the clipping `g.mul_(clip_coef_clamped)`
+ * (gradient_normalization.py:88-93).  `scan` may be NULL when use_clip = 0. */
+AXN_API int axn_mt_scale(void* const* h_g, const int64_t* h_sizes, int64_t n,
+                 int g_dtype, float inv_scale, const axn_scan_result* scan,
+                 int use_clip, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* AXN_H_ */
