@@ -243,7 +243,7 @@ size_t axn_mt_scan_workspace_bytes(int64_t n, int64_t total) {
 }
 
 int axn_mt_scan(const void* const* h_g, const int64_t* h_sizes, int64_t n,
-                int g_dtype, float inv_scale, float max_norm,
+                int g_dtype, float inv_scale, float max_norm, int accumulate,
                 axn_scan_result* result, void* workspace, size_t workspace_bytes,
                 void* stream) {
   const char* name = "axn_mt_scan";
@@ -258,7 +258,8 @@ int axn_mt_scan(const void* const* h_g, const int64_t* h_sizes, int64_t n,
           "%s: workspace must be 16-byte aligned", name);
   rc = check_list(name, h_g, "g", h_sizes, n, g_dtype == AXN_F32 ? 4 : 2);
   if (rc) return rc;
-  return launch_mt_scan(h_g, h_sizes, n, g_dtype, inv_scale, max_norm, result,
+  REQUIRE(accumulate == 0 || accumulate == 1, AXN_EINVAL, "%s: accumulate must be 0 or 1", name);
+  return launch_mt_scan(h_g, h_sizes, n, g_dtype, inv_scale, max_norm, accumulate, result,
                         workspace, workspace_bytes, (hipStream_t)stream);
 }
 

@@ -56,7 +56,7 @@ int launch_dgelu_dbias(const void* dY, const void* Z, void* dZ, int dtype,
 // ---- multi-tensor optimizer ------------------------------------------------
 size_t mt_scan_workspace_bytes(int64_t n, int64_t total);
 int launch_mt_scan(const void* const* h_g, const int64_t* h_sizes, int64_t n,
-                   int g_dtype, float inv_scale, float max_norm,
+                   int g_dtype, float inv_scale, float max_norm, int accumulate,
                    axn_scan_result* result, void* ws, size_t ws_bytes,
                    hipStream_t stream);
 int launch_mt_adam(const void* const* h_g, void* const* h_p, void* const* h_m,

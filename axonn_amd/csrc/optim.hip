@@ -313,6 +313,10 @@ __device__ __forceinline__ void adam_math(float g, float& p, float& m, float& v,
   v = v * s.hp.beta2 + s.hp.one_minus_beta2 * g * g;
   const float denom = sqrtf(v) * s.hp.inv_sqrt_bc2 + s.hp.eps;
   p = p - s.hp.lr_over_bc1 * (m / denom);
+  // The low-precision copy must be the rounding of the fp32 value that is
+  // stored, not of the unrounded expression: keep the compiler from folding
+  // the conversion into the last multiply-add (a mixed-precision FMA rounds once).
+  asm volatile("" : "+v"(p));
 }
 
 template <int GDT, int PDT, bool HAS_PLOW>
@@ -540,7 +544,7 @@ size_t mt_scan_workspace_bytes(int64_t n, int64_t total) {
 }
 
 int launch_mt_scan(const void* const* h_g, const int64_t* h_sizes, int64_t n,
-                   int g_dtype, float inv_scale, float max_norm,
+                   int g_dtype, float inv_scale, float max_norm, int accumulate,
                    axn_scan_result* result, void* ws, size_t ws_bytes,
                    hipStream_t stream) {
   const void* const* sets[1] = {h_g};
@@ -561,12 +565,13 @@ int launch_mt_scan(const void* const* h_g, const int64_t* h_sizes, int64_t n,
     MtTable empty = MtTable();
     empty.n = 0;
     hipLaunchKernelGGL(mt_scan_finalize_kernel, dim3(1), dim3(1024), 0, stream,
-                       empty, partial, 0, sum_limit_of(g_dtype), max_norm, 1, result);
+                       empty, partial, 0, sum_limit_of(g_dtype), max_norm,
+                       accumulate ? 0 : 1, result);
     AXN_HIP_TRY(hipGetLastError());
     return AXN_OK;
   }
   int base = 0;
-  bool first = true;
+  bool first = !accumulate;
   for (auto& gr : groups) {
     switch (g_dtype) {
       case AXN_BF16:

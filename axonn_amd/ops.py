@@ -1,0 +1,295 @@
+"""Tensor-level wrappers over the C ABI of libaxn_gfx950.so.
+
+Each function checks dtypes and devices, allocates the outputs with torch,
+passes raw pointers, sizes and torch's current HIP stream to the library and
+returns.  None of the arithmetic happens here, and nothing here falls back to a
+torch op: tensors that are not on a GPU are rejected.
+"""
+
+import torch
+
+from . import _native as nv
+
+EPILOGUES = {
+    (False, None): nv.EPI_NONE,
+    (True, None): nv.EPI_BIAS,
+    (True, "gelu"): nv.EPI_BIAS_GELU,
+    (False, "gelu"): nv.EPI_GELU,
+}
+
+
+def _require_gpu(*tensors):
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise RuntimeError(
+                "axonn_amd kernels run on the GPU only; got a tensor on %s" % t.device
+            )
+
+
+def _rows(t):
+    """A 2-D tensor usable by the kernels: unit stride along the last dimension.
+    Returns (tensor, leading dimension)."""
+    if t.dim() != 2:
+        raise ValueError("expected a 2-D tensor, got shape %s" % (tuple(t.shape),))
+    if t.stride(1) != 1 or (t.shape[0] > 1 and t.stride(0) < t.shape[1]):
+        t = t.contiguous()
+    ld = t.stride(0) if t.shape[0] > 1 else t.shape[1]
+    return t, ld
+
+
+def _bf16_ok(t, ld):
+    return t.data_ptr() % 16 == 0 and ld % 8 == 0
+
+
+def _prep_bf16(t):
+    t, ld = _rows(t)
+    if not _bf16_ok(t, ld):
+        t = t.contiguous().clone()
+        ld = t.shape[1]
+    return t, ld
+
+
+# ------------------------------------------------------------------ GEMMs ----
+def gemm_fwd(x, w, bias=None, activation=None, save_z=False):
+    """Y = act(X W^T + b).  x [M,K], w [N,K]; bf16 or fp32 (both the same).
+    Returns (y, z) with z the saved pre-activation (None unless activation and
+    save_z)."""
+    _require_gpu(x, w, bias)
+    if x.dtype != w.dtype:
+        raise TypeError("input is %s but weight is %s" % (x.dtype, w.dtype))
+    epi = EPILOGUES[(bias is not None, activation)]
+    M, K = x.shape
+    N = w.shape[0]
+    if w.shape[1] != K:
+        raise ValueError("weight is %s, input has %d features" % (tuple(w.shape), K))
+    if bias is not None:
+        bias = bias.float().contiguous()
+        if bias.numel() != N:
+            raise ValueError("bias has %d elements, expected %d" % (bias.numel(), N))
+    want_z = activation is not None and save_z
+    if x.dtype == torch.bfloat16:
+        x, ldx = _prep_bf16(x)
+        w, ldw = _prep_bf16(w)
+        y = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
+        z = torch.empty_like(y) if want_z else None
+        nv.call("axn_gemm_fwd", nv.ptr(x), nv.ptr(w), nv.ptr(bias), nv.ptr(y), nv.ptr(z),
+                M, N, K, ldx, ldw, N, epi, nv.current_stream())
+    elif x.dtype == torch.float32:
+        x, w = x.contiguous(), w.contiguous()
+        y = torch.empty((M, N), dtype=torch.float32, device=x.device)
+        z = torch.empty_like(y) if want_z else None
+        nv.call("axn_gemm_fwd_f32", nv.ptr(x), nv.ptr(w), nv.ptr(bias), nv.ptr(y), nv.ptr(z),
+                M, N, K, epi, nv.current_stream())
+    else:
+        raise TypeError("the Linear kernels take bf16 or fp32 operands, got %s" % x.dtype)
+    return y, z
+
+
+def gemm_dgrad(dy, w):
+    """dX = dY W.  dy [M,N], w [N,K]."""
+    _require_gpu(dy, w)
+    if dy.dtype != w.dtype:
+        raise TypeError("grad_output is %s but weight is %s" % (dy.dtype, w.dtype))
+    M, N = dy.shape
+    K = w.shape[1]
+    if dy.dtype == torch.bfloat16:
+        dy, lddy = _prep_bf16(dy)
+        w, ldw = _prep_bf16(w)
+        dx = torch.empty((M, K), dtype=torch.bfloat16, device=dy.device)
+        nv.call("axn_gemm_dgrad", nv.ptr(dy), nv.ptr(w), nv.ptr(dx), M, N, K, lddy, ldw, K,
+                nv.current_stream())
+    elif dy.dtype == torch.float32:
+        dy, w = dy.contiguous(), w.contiguous()
+        dx = torch.empty((M, K), dtype=torch.float32, device=dy.device)
+        nv.call("axn_gemm_dgrad_f32", nv.ptr(dy), nv.ptr(w), nv.ptr(dx), M, N, K,
+                nv.current_stream())
+    else:
+        raise TypeError("the Linear kernels take bf16 or fp32 operands, got %s" % dy.dtype)
+    return dx
+
+
+def gemm_wgrad(dy, x, out=None, accumulate=False, out_dtype=None):
+    """dW = dY^T X, optionally accumulated into `out` (dW += ...).  dy [M,N],
+    x [M,K]; the result is [N,K] in `out_dtype` (bf16 or fp32 for bf16 operands)."""
+    _require_gpu(dy, x, out)
+    if dy.dtype != x.dtype:
+        raise TypeError("grad_output is %s but input is %s" % (dy.dtype, x.dtype))
+    M, N = dy.shape
+    K = x.shape[1]
+    if out is not None:
+        if out.numel() != N * K or not out.is_contiguous():
+            raise ValueError("`out` must be a contiguous tensor of %d elements" % (N * K))
+        out_dtype = out.dtype
+    elif accumulate:
+        raise ValueError("accumulate=True needs `out`")
+    if out_dtype is None:
+        out_dtype = dy.dtype
+    if dy.dtype == torch.bfloat16:
+        if out_dtype not in (torch.bfloat16, torch.float32):
+            raise TypeError("dW must be bf16 or fp32, got %s" % out_dtype)
+        dy, lddy = _prep_bf16(dy)
+        x, ldx = _prep_bf16(x)
+        if out is None:
+            out = torch.empty((N, K), dtype=out_dtype, device=dy.device)
+        nv.call("axn_gemm_wgrad", nv.ptr(dy), nv.ptr(x), nv.ptr(out), M, N, K, lddy, ldx, K,
+                1 if accumulate else 0, nv.dtype_code(out_dtype), nv.current_stream())
+    elif dy.dtype == torch.float32:
+        if out_dtype != torch.float32:
+            raise TypeError("fp32 operands give an fp32 dW, got %s" % out_dtype)
+        dy, x = dy.contiguous(), x.contiguous()
+        if out is None:
+            out = torch.empty((N, K), dtype=torch.float32, device=dy.device)
+        nv.call("axn_gemm_wgrad_f32", nv.ptr(dy), nv.ptr(x), nv.ptr(out), M, N, K,
+                1 if accumulate else 0, nv.current_stream())
+    else:
+        raise TypeError("the Linear kernels take bf16 or fp32 operands, got %s" % dy.dtype)
+    return out
+
+
+def dgelu_dbias(dy, z=None, want_dbias=True, dbias_out=None, accumulate=False):
+    """dZ = dY * gelu'(Z) (when z is given) and dbias = column sums of dZ (fp32).
+    Returns (dz, dbias); dz is dy itself when z is None."""
+    _require_gpu(dy, z, dbias_out)
+    if dy.dtype not in (torch.bfloat16, torch.float32):
+        raise TypeError("bf16 or fp32 expected, got %s" % dy.dtype)
+    dy, ld = _rows(dy)
+    if dy.data_ptr() % 16 or ld % 8:
+        dy = dy.contiguous().clone()
+        ld = dy.shape[1]
+    M, N = dy.shape
+    dz = None
+    if z is not None:
+        if z.dtype != dy.dtype or z.shape != dy.shape:
+            raise ValueError("z must match dy in dtype and shape")
+        if not z.is_contiguous() or ld != N:
+            z = z.contiguous()
+            dy = dy.contiguous()
+            ld = N
+        dz = torch.empty_like(dy)
+    dbias = None
+    ws, ws_bytes = None, 0
+    if want_dbias:
+        dbias = dbias_out if dbias_out is not None else torch.empty(N, dtype=torch.float32, device=dy.device)
+        if dbias.dtype != torch.float32 or dbias.numel() != N:
+            raise ValueError("dbias must be fp32 with %d elements" % N)
+        ws_bytes = nv.load().axn_dgelu_dbias_workspace_bytes(M, N)
+        ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=dy.device)
+    elif z is None:
+        return dy, None
+    nv.call("axn_dgelu_dbias", nv.ptr(dy), nv.ptr(z), nv.ptr(dz), nv.dtype_code(dy.dtype),
+            nv.ptr(dbias), M, N, ld, 1 if (accumulate and dbias_out is not None) else 0,
+            nv.ptr(ws), ws_bytes, nv.current_stream())
+    return (dz if dz is not None else dy), dbias
+
+
+# ---------------------------------------------------------- multi-tensor -----
+class ScanResult:
+    """Device-resident axn_scan_result (32 bytes) with typed views."""
+
+    def __init__(self, device):
+        self.buf = torch.zeros(8, dtype=torch.float32, device=device)
+
+    @property
+    def sumsq(self):
+        return self.buf.view(torch.float64)[0]
+
+    @property
+    def total_norm(self):
+        return self.buf[2]
+
+    @property
+    def clip_coef(self):
+        return self.buf[3]
+
+    @property
+    def found_inf(self):
+        return self.buf.view(torch.int32)[4]
+
+    def ptr(self):
+        return nv.ptr(self.buf)
+
+
+def _check_list(tensors, dtype=None):
+    for t in tensors:
+        _require_gpu(t)
+        if not t.is_contiguous():
+            raise ValueError("multi-tensor kernels need contiguous tensors")
+        if dtype is not None and t.dtype != dtype:
+            raise TypeError("expected %s, got %s" % (dtype, t.dtype))
+
+
+def mt_scan(grads, inv_scale=1.0, max_norm=0.0, result=None, accumulate=False):
+    """Overflow flag, sum of squares, 2-norm and clip coefficient of a list of
+    gradients of ONE dtype, left on the device in a ScanResult."""
+    if len(grads) == 0:
+        raise ValueError("empty gradient list")
+    dt = grads[0].dtype
+    _check_list(grads, dt)
+    device = grads[0].device
+    if result is None:
+        result = ScanResult(device)
+        accumulate = False
+    total = sum(g.numel() for g in grads)
+    ws_bytes = nv.load().axn_mt_scan_workspace_bytes(len(grads), total)
+    ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=device)
+    nv.call("axn_mt_scan", nv.ptr_array(grads), nv.size_array(grads), len(grads),
+            nv.dtype_code(dt), float(inv_scale), float(max_norm), 1 if accumulate else 0,
+            result.ptr(), nv.ptr(ws), ws_bytes, nv.current_stream())
+    return result
+
+
+def mt_adam(grads, params32, exp_avg, exp_avg_sq, params_lowp, hparams, inv_scale=1.0,
+            scan=None):
+    """One fused Adam pass over the lists; see axn_mt_adam in include/axn.h."""
+    n = len(grads)
+    if not (len(params32) == len(exp_avg) == len(exp_avg_sq) == n):
+        raise ValueError("list lengths differ")
+    if n == 0:
+        return
+    gdt = grads[0].dtype
+    _check_list(grads, gdt)
+    _check_list(params32, torch.float32)
+    _check_list(exp_avg, torch.float32)
+    _check_list(exp_avg_sq, torch.float32)
+    plow_arr, pdt = None, nv.BF16
+    if params_lowp is not None:
+        if len(params_lowp) != n:
+            raise ValueError("list lengths differ")
+        _check_list(params_lowp, params_lowp[0].dtype)
+        pdt = nv.dtype_code(params_lowp[0].dtype)
+        plow_arr = nv.ptr_array(params_lowp)
+    for g, p in zip(grads, params32):
+        if g.numel() != p.numel():
+            raise ValueError("gradient and parameter sizes differ")
+    nv.call("axn_mt_adam", nv.ptr_array(grads), nv.ptr_array(params32), nv.ptr_array(exp_avg),
+            nv.ptr_array(exp_avg_sq), plow_arr, nv.size_array(grads), n, nv.dtype_code(gdt),
+            pdt, float(inv_scale), scan.ptr() if scan is not None else None,
+            hparams, nv.current_stream())
+
+
+def mt_scale(grads, inv_scale=1.0, scan=None, use_clip=False):
+    """In-place g *= inv_scale (* clip coefficient) on a list of ONE dtype."""
+    if len(grads) == 0:
+        return
+    dt = grads[0].dtype
+    _check_list(grads, dt)
+    nv.call("axn_mt_scale", nv.ptr_array(grads), nv.size_array(grads), len(grads),
+            nv.dtype_code(dt), float(inv_scale), scan.ptr() if scan is not None else None,
+            1 if use_clip else 0, nv.current_stream())
+
+
+def adam_hparams(step, lr, beta1, beta2, eps, weight_decay):
+    """Host-side scalars of Adam step number `step` (1-based); bias corrections
+    in Python doubles as torch computes them."""
+    bc1 = 1.0 - beta1 ** step
+    bc2 = 1.0 - beta2 ** step
+    return nv.AdamHParams(
+        lr_over_bc1=lr / bc1,
+        inv_sqrt_bc2=1.0 / (bc2 ** 0.5),
+        beta1=beta1,
+        one_minus_beta1=1.0 - beta1,
+        beta2=beta2,
+        one_minus_beta2=1.0 - beta2,
+        eps=eps,
+        weight_decay=weight_decay,
+    )

@@ -157,9 +157,12 @@ AXN_API size_t axn_mt_scan_workspace_bytes(int64_t n, int64_t total);
  *   h_g[n]: device pointers to gradients of g_dtype (BF16, F16 or F32);
  *   h_sizes[n]: element counts; inv_scale = 1 / loss_scale;
  *   max_norm <= 0 disables clipping (clip_coef = 1).
- *   result: device axn_scan_result, fully overwritten. */
+ *   result: device axn_scan_result; overwritten when accumulate = 0; with
+ *   accumulate = 1 the new sum of squares and flag are combined with what
+ *   `result` already holds (a gradient list of several dtypes takes one call
+ *   per dtype on the same stream) and norm and coefficient are recomputed. */
 AXN_API int axn_mt_scan(const void* const* h_g, const int64_t* h_sizes, int64_t n,
-                int g_dtype, float inv_scale, float max_norm,
+                int g_dtype, float inv_scale, float max_norm, int accumulate,
                 axn_scan_result* result, void* workspace,
                 size_t workspace_bytes, void* stream);
 

@@ -1,0 +1,125 @@
+"""The C-ABI shared library: it loads, exports every symbol include/axn.h
+declares, and rejects bad arguments with the documented codes before touching
+the GPU (so all of this runs on a host without one)."""
+
+import ctypes
+import os
+import re
+
+import pytest
+
+from axonn_amd import _native as nv
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "axn.h")).read()
+    return sorted(set(re.findall(r"AXN_API\s+[\w\s\*]+?\b(axn_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_declares_the_expected_entry_points():
+    names = declared_symbols()
+    assert len(names) >= 14
+    assert set(names) == set(nv.SYMBOLS), "binding table and header disagree"
+
+
+def test_library_loads_and_exports_every_declared_symbol():
+    lib = ctypes.CDLL(nv.lib_path())
+    for name in declared_symbols():
+        assert hasattr(lib, name), "libaxn_gfx950.so does not export %s" % name
+    assert nv.load().axn_abi_version() == nv.ABI_VERSION
+
+
+def test_library_is_a_gfx950_code_object():
+    blob = open(nv.lib_path(), "rb").read()
+    assert b"gfx950" in blob
+
+
+def test_workspace_queries():
+    lib = nv.load()
+    assert lib.axn_mt_scan_workspace_bytes(64, 1_300_000_000) >= (1_300_000_000 // 16384) * 16
+    assert lib.axn_mt_scan_workspace_bytes(-1, 5) == 0
+    assert lib.axn_dgelu_dbias_workspace_bytes(8192, 5120) == 64 * 5120 * 4
+    assert lib.axn_dgelu_dbias_workspace_bytes(0, 8) == 0
+
+
+def _err():
+    return nv.load().axn_last_error().decode()
+
+
+A = ctypes.c_void_p(0x1000)  # never dereferenced: validation fails first
+
+
+def test_gemm_argument_errors():
+    lib = nv.load()
+    f = lib.axn_gemm_fwd
+    assert f(None, A, None, A, None, 8, 8, 8, 8, 8, 8, 0, None) == nv.AXN_EINVAL
+    assert "null" in _err()
+    assert f(A, A, None, A, None, 0, 8, 8, 8, 8, 8, 0, None) == nv.AXN_EINVAL
+    assert f(A, A, None, A, None, 8, 12, 8, 8, 8, 16, 0, None) == nv.AXN_ESHAPE
+    assert "multiples of 8" in _err()
+    assert f(A, A, None, A, None, 8, 8, 8, 4, 8, 8, 0, None) == nv.AXN_EINVAL  # ld < row
+    assert f(A, A, None, A, None, 8, 8, 8, 12, 8, 8, 0, None) == nv.AXN_EALIGN  # ld % 8
+    assert f(ctypes.c_void_p(0x1004), A, None, A, None, 8, 8, 8, 8, 8, 8, 0, None) == nv.AXN_EALIGN
+    assert f(A, A, None, A, None, 8, 8, 8, 8, 8, 8, 7, None) == nv.AXN_EINVAL  # epilogue
+    assert f(A, A, None, A, None, 8, 8, 8, 8, 8, 8, nv.EPI_BIAS, None) == nv.AXN_EINVAL
+    assert "bias" in _err()
+    assert f(A, A, None, A, None, 2 ** 31, 8, 8, 8, 8, 8, 0, None) == nv.AXN_ELIMIT
+    assert lib.axn_gemm_dgrad(A, A, None, 8, 8, 8, 8, 8, 8, None) == nv.AXN_EINVAL
+    assert lib.axn_gemm_wgrad(A, A, A, 8, 8, 8, 8, 8, 8, 2, nv.BF16, None) == nv.AXN_EINVAL
+    assert lib.axn_gemm_wgrad(A, A, A, 8, 8, 8, 8, 8, 8, 0, nv.F16, None) == nv.AXN_EINVAL
+    assert lib.axn_gemm_fwd_f32(A, None, None, A, None, 4, 4, 4, 0, None) == nv.AXN_EINVAL
+    assert lib.axn_gemm_wgrad_f32(A, A, A, 4, 4, 4, 3, None) == nv.AXN_EINVAL
+    assert lib.axn_gemm_dgrad_f32(ctypes.c_void_p(0x1002), A, A, 4, 4, 4, None) == nv.AXN_EALIGN
+
+
+def test_elementwise_argument_errors():
+    lib = nv.load()
+    f = lib.axn_dgelu_dbias
+    assert f(None, None, None, nv.BF16, A, 8, 8, 8, 0, A, 1024, None) == nv.AXN_EINVAL
+    assert f(A, A, None, nv.BF16, A, 8, 8, 8, 0, A, 1024, None) == nv.AXN_EINVAL  # Z without dZ
+    assert f(A, None, None, nv.BF16, None, 8, 8, 8, 0, A, 1024, None) == nv.AXN_EINVAL  # nothing to do
+    assert f(A, None, None, nv.F16, A, 8, 8, 8, 0, A, 1024, None) == nv.AXN_EINVAL
+    assert f(A, None, None, nv.BF16, A, 8, 12, 16, 0, A, 1024, None) == nv.AXN_ESHAPE
+    assert f(A, None, None, nv.BF16, A, 8, 8, 8, 0, A, 4, None) == nv.AXN_EINVAL  # workspace too small
+    assert "workspace" in _err()
+
+
+def test_multi_tensor_argument_errors():
+    lib = nv.load()
+    ptrs = (ctypes.c_void_p * 2)(0x1000, 0x2001)
+    sizes = (ctypes.c_int64 * 2)(4, 4)
+    res = ctypes.c_void_p(0x3000)
+    assert lib.axn_mt_scan(ptrs, sizes, 2, nv.BF16, 1.0, 0.0, 0, res, A, 4096, None) == nv.AXN_EALIGN
+    assert "g[1]" in _err()
+    sizes[1] = -1
+    assert lib.axn_mt_scan(ptrs, sizes, 2, nv.BF16, 1.0, 0.0, 0, res, A, 4096, None) == nv.AXN_EINVAL
+    sizes[1] = 0  # empty tensors may carry any pointer
+    assert lib.axn_mt_scan(ptrs, sizes, 2, 9, 1.0, 0.0, 0, res, A, 4096, None) == nv.AXN_EINVAL
+    assert lib.axn_mt_scan(ptrs, sizes, 2, nv.BF16, 1.0, 0.0, 0, None, A, 4096, None) == nv.AXN_EINVAL
+    assert lib.axn_mt_scan(ptrs, sizes, 2, nv.BF16, 1.0, 0.0, 5, res, A, 4096, None) == nv.AXN_EINVAL
+    assert lib.axn_mt_scan(ptrs, sizes, 2, nv.BF16, 1.0, 0.0, 0, res, A, 0, None) == nv.AXN_EINVAL
+    assert "workspace" in _err()
+    hp = nv.AdamHParams()
+    assert lib.axn_mt_adam(ptrs, ptrs, ptrs, ptrs, None, sizes, 2, nv.BF16, nv.BF16, 1.0, None,
+                           None, None) == nv.AXN_EINVAL
+    assert lib.axn_mt_adam(ptrs, None, ptrs, ptrs, None, sizes, 2, nv.BF16, nv.BF16, 1.0, None,
+                           hp, None) == nv.AXN_EINVAL
+    assert lib.axn_mt_adam(ptrs, ptrs, ptrs, ptrs, ptrs, sizes, 2, nv.BF16, nv.F32, 1.0, None,
+                           hp, None) == nv.AXN_EINVAL
+    assert lib.axn_mt_scale(ptrs, sizes, 2, nv.BF16, 1.0, None, 1, None) == nv.AXN_EINVAL
+    assert "scan" in _err()
+    assert lib.axn_mt_scale(ptrs, sizes, -1, nv.BF16, 1.0, None, 0, None) == nv.AXN_EINVAL
+
+
+def test_adam_hparams_struct_layout():
+    assert ctypes.sizeof(nv.AdamHParams) == 32
+    assert nv.SCAN_RESULT_BYTES == 32
+
+
+def test_missing_library_fails_loudly(monkeypatch):
+    monkeypatch.setattr(nv, "_lib", None)
+    monkeypatch.setattr(nv, "_LIB_PATH", "/nonexistent/libaxn_gfx950.so")
+    with pytest.raises(ImportError, match="not built"):
+        nv.load()

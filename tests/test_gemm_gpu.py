@@ -1,0 +1,226 @@
+"""Parity of the GEMM kernels (through the C ABI) with the CPU oracle.
+
+Tolerance (bf16 operands, fp32 accumulate): normwise relative error <= 1e-2
+against the oracle evaluated in float64 on the same bf16-rounded inputs.  What is
+actually left is the final rounding to bf16 (about 2e-3 normwise); with an fp32
+result only fp32 accumulation error remains (<= 1e-5).
+"""
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import linear as ol
+
+pytestmark = pytest.mark.gpu
+
+BF16_TOL = 1e-2
+F32_TOL = 1e-5
+
+
+def rel(a, b):
+    a, b = np.asarray(a, np.float64), np.asarray(b, np.float64)
+    return float(np.linalg.norm(a - b) / max(np.linalg.norm(b), 1e-300))
+
+
+def bf16_inputs(M, N, K, seed, x_std=1.0, w_std=0.02, g_std=1e-3):
+    g = torch.Generator().manual_seed(seed)
+    X = (torch.randn(M, K, generator=g) * x_std).bfloat16()
+    W = (torch.randn(N, K, generator=g) * w_std).bfloat16()
+    dY = (torch.randn(M, N, generator=g) * g_std).bfloat16()
+    return X, W, dY
+
+
+def np64(t):
+    return t.float().cpu().numpy().astype(np.float64)
+
+
+SHAPES = [
+    (32, 64, 64), (16, 128, 128), (2, 256, 256),       # the reference's test shapes
+    (256, 256, 64), (128, 128, 64), (256, 512, 320),   # exact tiles, 1 and 5 contraction steps
+    (100, 72, 40), (33, 8, 8), (1, 8, 16), (257, 264, 72), (130, 136, 520),  # ragged
+    (512, 1024, 1024),
+]
+
+
+@pytest.mark.parametrize("M,N,K", SHAPES)
+def test_three_gemms_match_oracle(M, N, K):
+    from axonn_amd import ops
+
+    X, W, dY = bf16_inputs(M, N, K, seed=M * 7 + N * 3 + K)
+    yo, _ = ol.linear_forward(np64(X), np64(W).reshape(-1), (N, K))
+    bw = ol.linear_backward(np64(X), np64(W).reshape(-1), (N, K), np64(dY))
+    Xd, Wd, dYd = X.cuda(), W.cuda(), dY.cuda()
+    y, _ = ops.gemm_fwd(Xd, Wd)
+    dx = ops.gemm_dgrad(dYd, Wd)
+    dw = ops.gemm_wgrad(dYd, Xd)
+    dw32 = ops.gemm_wgrad(dYd, Xd, out_dtype=torch.float32)
+    assert y.dtype == torch.bfloat16 and y.shape == (M, N)
+    assert rel(np64(y), yo) < BF16_TOL
+    assert rel(np64(dx), bw["dx"]) < BF16_TOL
+    assert rel(np64(dw), bw["dw"].reshape(N, K)) < BF16_TOL
+    assert rel(np64(dw32), bw["dw"].reshape(N, K)) < F32_TOL
+
+
+@pytest.mark.parametrize("M,N,K", [(64, 64, 64), (300, 136, 96), (256, 256, 128)])
+@pytest.mark.parametrize("epilogue", ["bias", "bias_gelu", "gelu"])
+def test_fused_epilogues_match_oracle(M, N, K, epilogue):
+    from axonn_amd import ops
+
+    X, W, _ = bf16_inputs(M, N, K, seed=11, w_std=0.2)
+    b = torch.randn(N, generator=torch.Generator().manual_seed(5)) * 0.5
+    bias = b if "bias" in epilogue else None
+    act = "gelu" if "gelu" in epilogue else None
+    yo, zo = ol.linear_forward(np64(X), np64(W).reshape(-1), (N, K),
+                               bias=None if bias is None else b.double().numpy(), activation=act)
+    y, z = ops.gemm_fwd(X.cuda(), W.cuda(), bias=None if bias is None else b.cuda(),
+                        activation=act, save_z=True)
+    assert rel(np64(y), yo) < BF16_TOL
+    if act:
+        assert rel(np64(z), zo) < BF16_TOL
+    else:
+        assert z is None
+
+
+def test_dgelu_dbias_matches_oracle():
+    from axonn_amd import ops
+
+    g = torch.Generator().manual_seed(3)
+    M, N = 333, 520
+    dY = torch.randn(M, N, generator=g).bfloat16()
+    Z = (torch.randn(M, N, generator=g) * 2).bfloat16()
+    dz, db = ops.dgelu_dbias(dY.cuda(), Z.cuda(), want_dbias=True)
+    want = np64(dY) * ol.dgelu(np64(Z))
+    assert rel(np64(dz), want) < BF16_TOL
+    # dbias is the column sum of the rounded dZ the weight-gradient kernel reads
+    assert rel(db.cpu().numpy(), np64(dz).sum(0)) < 1e-6
+    assert rel(db.cpu().numpy(), want.sum(0)) < BF16_TOL
+    _, db2 = ops.dgelu_dbias(dY.cuda(), None, want_dbias=True)
+    assert rel(db2.cpu().numpy(), np64(dY).sum(0)) < 1e-6
+    # fp32 variant
+    dz32, db32 = ops.dgelu_dbias(dY.float().cuda(), Z.float().cuda(), want_dbias=True)
+    assert rel(dz32.cpu().numpy(), want) < 1e-6 and rel(db32.cpu().numpy(), want.sum(0)) < 1e-5
+
+
+def test_wgrad_accumulates_over_micro_batches():
+    """dW += dY^T X over 4 micro-batches equals the weight gradient of the
+    concatenated batch (overlap_communication.py:38-47 semantics, in fp32 and in
+    the parameter's bf16)."""
+    from axonn_amd import ops
+
+    N, K, M = 136, 72, 96
+    xs, gs = [], []
+    for mb in range(4):
+        X, _, dY = bf16_inputs(M, N, K, seed=mb)
+        xs.append(X)
+        gs.append(dY)
+    want = ol.linear_backward(np.concatenate([np64(x) for x in xs]), np.zeros(N * K), (N, K),
+                              np.concatenate([np64(g) for g in gs]))["dw"].reshape(N, K)
+    acc32 = torch.zeros(N, K, device="cuda")
+    acc16 = None
+    ref16 = None
+    for x, g in zip(xs, gs):
+        ops.gemm_wgrad(g.cuda(), x.cuda(), out=acc32, accumulate=True)
+        if acc16 is None:
+            acc16 = ops.gemm_wgrad(g.cuda(), x.cuda())
+        else:
+            ops.gemm_wgrad(g.cuda(), x.cuda(), out=acc16, accumulate=True)
+        part = ol.linear_backward(np64(x), np.zeros(N * K), (N, K), np64(g))["dw"]
+        ref16 = ol.accumulate(ref16, part, "bf16")
+    assert rel(acc32.cpu().numpy(), want) < F32_TOL
+    assert rel(np64(acc16), want) < BF16_TOL
+    assert rel(np64(acc16), ref16.reshape(N, K)) < BF16_TOL
+
+
+def test_strided_operands_and_leading_dimensions():
+    """Row-strided views (ld > row length) go to the kernels without a copy."""
+    from axonn_amd import ops
+
+    big = torch.randn(64, 256, generator=torch.Generator().manual_seed(1)).bfloat16().cuda()
+    X = big[:, 64:192]  # 64 x 128 view, ld 256, 16-byte aligned start
+    W = (torch.randn(72, 128, generator=torch.Generator().manual_seed(2)) * 0.1).bfloat16().cuda()
+    y, _ = ops.gemm_fwd(X, W)
+    yo, _ = ol.linear_forward(np64(X), np64(W).reshape(-1), (72, 128))
+    assert rel(np64(y), yo) < BF16_TOL
+    Xo = big[:, 3:131]  # misaligned start: the wrapper copies
+    y2, _ = ops.gemm_fwd(Xo, W)
+    yo2, _ = ol.linear_forward(np64(Xo), np64(W).reshape(-1), (72, 128))
+    assert rel(np64(y2), yo2) < BF16_TOL
+
+
+def test_unsupported_shapes_raise():
+    from axonn_amd import _native as nv
+    from axonn_amd import ops
+
+    X = torch.zeros(8, 12, dtype=torch.bfloat16, device="cuda")
+    W = torch.zeros(16, 12, dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(nv.AxnError, match="multiples of 8") as e:
+        ops.gemm_fwd(X, W)
+    assert e.value.code == nv.AXN_ESHAPE
+    with pytest.raises(TypeError):
+        ops.gemm_fwd(X.half(), W.half())
+    with pytest.raises(TypeError):
+        ops.gemm_fwd(X, W.float())
+
+
+@pytest.mark.parametrize("M,N,K", [(5, 7, 3), (64, 48, 40), (130, 70, 257)])
+def test_fp32_gemms_match_oracle(M, N, K):
+    from axonn_amd import ops
+
+    g = torch.Generator().manual_seed(M + N + K)
+    X, W, dY = torch.randn(M, K, generator=g), torch.randn(N, K, generator=g) * 0.1, torch.randn(M, N, generator=g)
+    b = torch.randn(N, generator=g)
+    yo, zo = ol.linear_forward(X.double().numpy(), W.double().numpy().reshape(-1), (N, K),
+                               bias=b.double().numpy(), activation="gelu")
+    bw = ol.linear_backward(X.double().numpy(), W.double().numpy().reshape(-1), (N, K), dY.double().numpy())
+    y, z = ops.gemm_fwd(X.cuda(), W.cuda(), bias=b.cuda(), activation="gelu", save_z=True)
+    assert rel(y.cpu().numpy(), yo) < F32_TOL and rel(z.cpu().numpy(), zo) < F32_TOL
+    assert rel(ops.gemm_dgrad(dY.cuda(), W.cuda()).cpu().numpy(), bw["dx"]) < F32_TOL
+    dw = ops.gemm_wgrad(dY.cuda(), X.cuda())
+    assert rel(dw.cpu().numpy(), bw["dw"].reshape(N, K)) < F32_TOL
+    ops.gemm_wgrad(dY.cuda(), X.cuda(), out=dw, accumulate=True)
+    assert rel(dw.cpu().numpy(), 2 * bw["dw"].reshape(N, K)) < F32_TOL
+
+
+# ---- full benchmark shapes: size-independent properties + sampled oracle ------
+FULL = {
+    "qkv": (4096, 6144, 4096), "o": (4096, 4096, 4096), "gate_up": (4096, 14336, 4096),
+    "down": (4096, 4096, 14336), "mlp_shard": (8192, 5120, 2560), "skinny": (512, 8192, 3584),
+}
+
+
+@pytest.mark.parametrize("name", sorted(FULL))
+def test_full_size_shapes_sampled_oracle_and_properties(name):
+    from axonn_amd import ops
+
+    M, N, K = FULL[name]
+    g = torch.Generator(device="cuda").manual_seed(0)
+    X = torch.randn(M, K, generator=g, device="cuda").bfloat16()
+    W = (torch.randn(N, K, generator=g, device="cuda") * 0.02).bfloat16()
+    dY = (torch.randn(M, N, generator=g, device="cuda") * 1e-3).bfloat16()
+    y, _ = ops.gemm_fwd(X, W)
+    dx = ops.gemm_dgrad(dY, W)
+    dw = ops.gemm_wgrad(dY, X, out_dtype=torch.float32)
+    # (a) oracle on a sample of rows / columns of each result
+    rs = np.random.default_rng(1)
+    rows = np.sort(rs.choice(M, 48, replace=False))
+    nrows = np.sort(rs.choice(N, 48, replace=False))
+    ti, tn = torch.from_numpy(rows).cuda(), torch.from_numpy(nrows).cuda()
+    Wn, Xn, dYn = np64(W), np64(X[ti]), np64(dY[ti])
+    yo, _ = ol.linear_forward(Xn, Wn.reshape(-1), (N, K))
+    assert rel(np64(y[ti]), yo) < BF16_TOL
+    assert rel(np64(dx[ti]), dYn @ Wn) < BF16_TOL
+    dwo = np64(dY[:, tn]).T @ np64(X)   # rows `nrows` of dW
+    assert rel(dw[tn].cpu().numpy(), dwo) < 1e-4
+    # (b) linearity in the input: f(2x) = 2 f(x) exactly (powers of two commute with rounding)
+    y2, _ = ops.gemm_fwd(X * 2, W)
+    assert torch.equal(y2, y * 2)
+    # (c) <dY, X W^T> = <dY W, X> = <dY^T X, W>: the three kernels agree with each other
+    a = float((dY.double() * y.double()).sum())
+    yd = float((dx.double() * X.double()).sum())
+    wd = float((dw.double() * W.double()).sum())
+    scale = float(dY.double().norm() * y.double().norm())
+    assert abs(a - yd) < 1e-3 * scale and abs(a - wd) < 1e-3 * scale
+    # (d) determinism: the same call gives the same bits
+    y3, _ = ops.gemm_fwd(X, W)
+    assert torch.equal(y3, y)

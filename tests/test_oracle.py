@@ -1,0 +1,384 @@
+"""Pins the CPU oracle (oracle/) before it is trusted as the checker.
+
+The reference holds no golden vectors and no optimizer tests; its layer tests
+assert equality with torch.nn.Linear and torch.nn.utils.clip_grad_norm_
+(axonn/tests/test_intra_layer_fc.py:77, :167-199).  So every oracle function is
+pinned here against (a) the torch library routine the reference delegates to,
+(b) closed forms / invariants, (c) brute force on tiny inputs - chosen so that
+a dropped term, a wrong sign, a transposed operand or a wrong rounding fails.
+"""
+
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import linear as ol
+from oracle import optim as oo
+from oracle import torch_cpu as ot
+
+REF_SHAPES = [(32, 64), (16, 128), (2, 256)]  # test_intra_layer_fc.py:18
+
+
+# ------------------------------------------------------------------ bf16 -----
+def test_bf16_rounding_matches_torch_bitwise():
+    rng = np.random.default_rng(0)
+    x = (rng.standard_normal(20000) * np.logspace(-30, 30, 20000)).astype(np.float32)
+    special = np.array([0.0, -0.0, np.inf, -np.inf, 1.00390625, 1.01171875, 1.005859375,
+                        3.39e38, 3.4e38, 1e-40, -1e-45, 65504.0], dtype=np.float32)
+    x = np.concatenate([x, special])
+    want = torch.from_numpy(x).bfloat16().view(torch.int16).numpy().view(np.uint16)
+    assert np.array_equal(ol.bf16_bits(x), want)
+    assert ol.bf16_bits(np.array([np.nan], dtype=np.float32))[0] == 0x7FC0
+
+
+def test_bf16_ties_to_even_by_hand():
+    # 1 + 2^-8 is exactly half way between 1.0 (even mantissa) and 1 + 2^-7
+    assert ol.bf16_round(np.float32(1.0 + 2.0 ** -8)) == 1.0
+    # 1 + 3 * 2^-8 is half way between 1 + 2^-7 (odd) and 1 + 2^-6 (even)
+    assert ol.bf16_round(np.float32(1.0 + 3 * 2.0 ** -8)) == 1.0 + 2.0 ** -6
+    assert np.isinf(ol.bf16_round(np.float32(3.4e38)))
+
+
+# ------------------------------------------------------------------ GELU -----
+def test_gelu_against_math_erf_and_torch():
+    z = np.linspace(-6, 6, 241)
+    brute = np.array([0.5 * v * (1.0 + math.erf(v / math.sqrt(2.0))) for v in z])
+    assert np.allclose(ol.gelu(z), brute, rtol=0, atol=1e-15)
+    t = torch.nn.functional.gelu(torch.from_numpy(z)).numpy()
+    assert np.allclose(ol.gelu(z), t, rtol=1e-12, atol=1e-15)
+    # special values: gelu(0) = 0, gelu(z) -> z for large z, -> 0 for very negative z
+    assert ol.gelu(0.0) == 0.0
+    assert abs(ol.gelu(10.0) - 10.0) < 1e-12 and abs(ol.gelu(-10.0)) < 1e-12
+
+
+def test_dgelu_against_autograd_and_finite_differences():
+    z = np.linspace(-5, 5, 101)
+    zt = torch.from_numpy(z).requires_grad_(True)
+    torch.nn.functional.gelu(zt).sum().backward()
+    assert np.allclose(ol.dgelu(z), zt.grad.numpy(), rtol=1e-12, atol=1e-14)
+    h = 1e-6
+    fd = (ol.gelu(z + h) - ol.gelu(z - h)) / (2 * h)
+    assert np.allclose(ol.dgelu(z), fd, atol=1e-8)
+    assert ol.dgelu(0.0) == 0.5
+
+
+# ----------------------------------------------------------------- layer -----
+@pytest.mark.parametrize("B,H", REF_SHAPES)
+@pytest.mark.parametrize("bias", [False, True])
+def test_linear_matches_torch_nn_linear(B, H, bias):
+    """The reference's own assertion (test_intra_layer_fc.py:55-77, :157-199)."""
+    torch.manual_seed(42)
+    X = (torch.randn(B, H) * 0.01).double().requires_grad_(True)
+    dY = (torch.randn(B, H) * 0.01).double()
+    layer = torch.nn.Linear(H, H, bias=bias).double()
+    Y = layer(X)
+    Y.backward(dY)
+    w_flat = ol.extract_local_params_from_full_params(layer.weight.detach().numpy())
+    assert w_flat.ndim == 1 and w_flat.size == H * H
+    b = layer.bias.detach().numpy() if bias else None
+    y, _ = ol.linear_forward(X.detach().numpy(), w_flat, (H, H), bias=b)
+    bw = ol.linear_backward(X.detach().numpy(), w_flat, (H, H), dY.numpy(), has_bias=bias)
+    assert np.allclose(y, Y.detach().numpy(), rtol=1e-12, atol=1e-15)
+    assert np.allclose(bw["dx"], X.grad.numpy(), rtol=1e-12, atol=1e-15)
+    assert bw["dw"].ndim == 1  # the reference returns the weight gradient flattened
+    assert np.allclose(bw["dw"].reshape(H, H), layer.weight.grad.numpy(), rtol=1e-12, atol=1e-15)
+    if bias:
+        assert np.allclose(bw["db"], layer.bias.grad.numpy(), rtol=1e-12, atol=1e-15)
+
+
+def test_linear_brute_force_non_square():
+    """Triple loops on a tiny non-square case: catches a transposed operand."""
+    rng = np.random.default_rng(1)
+    M, K, N = 3, 5, 4
+    x, w, g = rng.standard_normal((M, K)), rng.standard_normal((N, K)), rng.standard_normal((M, N))
+    y = np.zeros((M, N))
+    dx = np.zeros((M, K))
+    dw = np.zeros((N, K))
+    for i in range(M):
+        for j in range(N):
+            for k in range(K):
+                y[i, j] += x[i, k] * w[j, k]
+                dx[i, k] += g[i, j] * w[j, k]
+                dw[j, k] += g[i, j] * x[i, k]
+    yo, _ = ol.linear_forward(x, w.reshape(-1), (N, K))
+    bw = ol.linear_backward(x, w.reshape(-1), (N, K), g)
+    assert np.allclose(yo, y) and np.allclose(bw["dx"], dx)
+    assert np.allclose(bw["dw"].reshape(N, K), dw)
+
+
+def test_linear_3d_input_and_skip_bias_add():
+    rng = np.random.default_rng(2)
+    x = rng.standard_normal((2, 3, 8))
+    w = rng.standard_normal((6, 8))
+    b = rng.standard_normal(6)
+    y, _ = ol.linear_forward(x, w.reshape(-1), (6, 8), bias=b)
+    want = torch.nn.functional.linear(torch.from_numpy(x), torch.from_numpy(w), torch.from_numpy(b))
+    assert y.shape == (2, 3, 6) and np.allclose(y, want.numpy())
+    (y2, b2), _ = ol.linear_forward(x, w.reshape(-1), (6, 8), bias=b, skip_bias_add=True)
+    assert np.allclose(y2 + b2, y)
+
+
+def test_fused_gelu_layer_against_autograd():
+    torch.manual_seed(5)
+    X = torch.randn(7, 12).double().requires_grad_(True)
+    lin = torch.nn.Linear(12, 9).double()
+    dY = torch.randn(7, 9).double()
+    Z = lin(X)
+    Y = torch.nn.functional.gelu(Z)
+    Y.backward(dY)
+    w = lin.weight.detach().numpy().reshape(-1)
+    y, z = ol.linear_forward(X.detach().numpy(), w, (9, 12), bias=lin.bias.detach().numpy(),
+                             activation="gelu")
+    bw = ol.linear_backward(X.detach().numpy(), w, (9, 12), dY.numpy(), z=z, activation="gelu",
+                            has_bias=True)
+    assert np.allclose(z, Z.detach().numpy()) and np.allclose(y, Y.detach().numpy())
+    assert np.allclose(bw["dx"], X.grad.numpy())
+    assert np.allclose(bw["dw"].reshape(9, 12), lin.weight.grad.numpy())
+    assert np.allclose(bw["db"], lin.bias.grad.numpy())
+
+
+def test_linearity_and_microbatch_additivity():
+    rng = np.random.default_rng(3)
+    x1, x2 = rng.standard_normal((4, 6)), rng.standard_normal((4, 6))
+    g1, g2 = rng.standard_normal((4, 5)), rng.standard_normal((4, 5))
+    w = rng.standard_normal(30)
+    y1, _ = ol.linear_forward(x1, w, (5, 6))
+    y2, _ = ol.linear_forward(x2, w, (5, 6))
+    y12, _ = ol.linear_forward(2 * x1 - 3 * x2, w, (5, 6))
+    assert np.allclose(y12, 2 * y1 - 3 * y2)
+    # dW over a concatenated batch is the sum of the per-micro-batch dW
+    d1 = ol.linear_backward(x1, w, (5, 6), g1)["dw"]
+    d2 = ol.linear_backward(x2, w, (5, 6), g2)["dw"]
+    dcat = ol.linear_backward(np.concatenate([x1, x2]), w, (5, 6), np.concatenate([g1, g2]))["dw"]
+    assert np.allclose(dcat, d1 + d2)
+
+
+def test_accumulate_rounds_in_param_dtype():
+    """overlap_communication.py:38-47: first assignment, then add_ in the
+    parameter's dtype."""
+    g1 = np.array([1.0, 1.0 + 2.0 ** -9])
+    acc = ol.accumulate(None, g1, "bf16")
+    want = torch.tensor(g1).to(torch.bfloat16)
+    assert np.array_equal(acc, want.double().numpy())
+    g2 = np.array([2.0 ** -9, 3.0])
+    acc2 = ol.accumulate(acc, g2, "bf16")
+    want2 = want.clone().add_(torch.tensor(g2).to(torch.bfloat16))
+    assert np.array_equal(acc2, want2.double().numpy())
+
+
+def test_default_init_bound_is_kaiming_uniform_a_sqrt5():
+    torch.manual_seed(0)
+    K = 1024
+    w = torch.nn.init.kaiming_uniform_(torch.empty(4096, K), a=math.sqrt(5))
+    b = ol.default_init_bound(K)
+    assert b == 1.0 / math.sqrt(K)
+    assert float(w.abs().max()) <= b and float(w.abs().max()) > 0.999 * b
+    assert abs(float(w.var()) - b * b / 3.0) < 0.02 * b * b / 3.0
+
+
+# ----------------------------------------------------------- overflow check --
+def test_check_nan_brute_force():
+    for dt in ("f32", "f16", "bf16"):
+        assert not oo.check_nan(np.array([1.0, -2.0, 3.0]), dt)
+        assert oo.check_nan(np.array([1.0, np.inf]), dt)
+        assert oo.check_nan(np.array([-np.inf, 1.0]), dt)
+        assert oo.check_nan(np.array([np.inf, -np.inf]), dt)  # inf - inf = nan
+        assert oo.check_nan(np.array([0.0, np.nan]), dt)
+    # the fp16 corner: finite elements whose sum leaves the fp16 range
+    x = np.full(4, 30000.0)
+    assert not oo.any_nonfinite(x)
+    assert oo.check_nan(x, "f16") and not oo.check_nan(x, "f32")
+    # and it is what torch's sum does
+    assert ot.check_nan(torch.full((4,), 30000.0, dtype=torch.float16))
+    assert not ot.check_nan(torch.full((2,), 30000.0, dtype=torch.float16))
+    assert not oo.check_nan(np.full(2, 30000.0), "f16")
+
+
+def test_check_nan_equals_elementwise_when_sum_in_range():
+    rng = np.random.default_rng(4)
+    for trial in range(50):
+        x = rng.standard_normal(64) * 100
+        if trial % 3 == 0:
+            x[rng.integers(64)] = rng.choice([np.inf, -np.inf, np.nan])
+        assert oo.check_nan(x, "bf16") == oo.any_nonfinite(x)
+        t = torch.tensor(x, dtype=torch.bfloat16)
+        assert ot.check_nan(t) == oo.check_nan(t.double().numpy(), "bf16")
+
+
+def test_unscale_is_exact_for_power_of_two_scales():
+    rng = np.random.default_rng(5)
+    g = ol.round_to(rng.standard_normal(100) * 40.0, "f16")
+    overflow, (u,) = oo.unscale_gradients([g], "f16", 2.0 ** 16)
+    assert not overflow
+    t = torch.tensor(g, dtype=torch.float16)
+    t.div_(2.0 ** 16)
+    assert np.array_equal(u, t.double().numpy())
+    # unscaling happens even when an overflow is found (inter_layer.py:455-458)
+    g[3] = np.inf
+    overflow, (u,) = oo.unscale_gradients([g], "f16", 2.0 ** 16)
+    assert overflow and np.isinf(u[3]) and u[0] == g[0] / 2.0 ** 16
+
+
+# ------------------------------------------------------------- loss scaler ---
+def test_loss_scaler_state_machine_table():
+    s = oo.LossScaler()
+    assert (s.loss_scale, s.max_scale, s.min_scale, s.scaling_window) == (65536.0, 2.0 ** 24, 1024.0, 200)
+    assert oo.sync_scale(s, True) is True and s.loss_scale == 32768.0 and s.no_overflow_iters == 0
+    for i in range(199):
+        assert oo.sync_scale(s, False) is False
+        assert s.loss_scale == 32768.0 and s.no_overflow_iters == i + 1
+    assert oo.sync_scale(s, False) is False  # the 200th clean step doubles
+    assert s.loss_scale == 65536.0 and s.no_overflow_iters == 0
+    s = oo.LossScaler(loss_scale=1024.0)
+    oo.sync_scale(s, True)
+    assert s.loss_scale == 1024.0  # floor
+    s = oo.LossScaler(loss_scale=2.0 ** 24, no_overflow_iters=199)
+    oo.sync_scale(s, False)
+    assert s.loss_scale == 2.0 ** 24  # cap
+    s = oo.LossScaler(no_overflow_iters=150)
+    oo.sync_scale(s, True)
+    assert s.no_overflow_iters == 0  # overflow resets the window
+
+
+# ------------------------------------------------------------ norm / clip ----
+@pytest.mark.parametrize("max_norm", [1e-3, 1.0, 100.0])
+def test_clip_matches_torch_clip_grad_norm(max_norm):
+    torch.manual_seed(6)
+    params = [torch.nn.Parameter(torch.zeros(n)) for n in (5, 17, 64)]
+    for p in params:
+        p.grad = torch.randn_like(p) * 0.3
+    grads = [p.grad.clone().double().numpy() for p in params]
+    total = torch.nn.utils.clip_grad_norm_(params, max_norm, foreach=False)
+    t, clipped = oo.clip_grad_norm_(grads, max_norm, "f32")
+    assert abs(t - float(total)) <= 1e-6 * float(total)
+    for c, p in zip(clipped, params):
+        assert np.allclose(c, p.grad.double().numpy(), rtol=2e-7, atol=0)
+    # closed form
+    flat = np.concatenate(grads)
+    assert abs(t - math.sqrt(float(np.sum(flat ** 2)))) < 1e-6 * t
+    assert oo.clip_coef(2.0, 1.0) == 1.0 / (2.0 + 1e-6) and oo.clip_coef(0.5, 1.0) == 1.0
+
+
+def test_norm_of_norms_equals_flat_norm():
+    rng = np.random.default_rng(7)
+    ts = [rng.standard_normal(n) for n in (3, 40, 7)]
+    assert abs(oo.get_total_norm(ts) - np.linalg.norm(np.concatenate(ts))) < 1e-12
+    assert oo.get_total_norm([]) == 0.0
+
+
+# ------------------------------------------------------------------ Adam -----
+@pytest.mark.parametrize("wd", [0.0, 0.01])
+def test_adam_matches_torch_optim_adam_over_steps(wd):
+    torch.manual_seed(8)
+    p = torch.nn.Parameter(torch.randn(257) * 0.02)
+    opt = torch.optim.Adam([p], lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=wd,
+                           foreach=False)
+    po = p.detach().numpy().copy()
+    mo = np.zeros_like(po)
+    vo = np.zeros_like(po)
+    for step in range(1, 6):
+        g = torch.randn(257) * 1e-3
+        p.grad = g.clone()
+        opt.step()
+        po, mo, vo = oo.adam_update(po, g.numpy(), mo, vo, step, weight_decay=wd)
+        st = opt.state[p]
+        # same float32 operation order as torch: agreement to one ulp of p
+        # (torch's CPU kernels may fuse a multiply-add where numpy does not)
+        ref = p.detach().numpy()
+        assert np.max(np.abs(po - ref)) <= 2.0 ** -23 * np.max(np.abs(ref))
+        assert np.max(np.abs(po - ref)) / np.max(np.abs(ref)) <= 1e-6
+        assert np.allclose(mo, st["exp_avg"].numpy(), rtol=3e-7, atol=1e-10)
+        assert np.allclose(vo, st["exp_avg_sq"].numpy(), rtol=3e-7, atol=1e-15)
+
+
+def test_adam_step_one_closed_form_and_f64():
+    rng = np.random.default_rng(9)
+    p = (rng.standard_normal(100) * 0.02).astype(np.float32)
+    g = (rng.standard_normal(100) * 1e-3).astype(np.float32)
+    z = np.zeros(100, dtype=np.float32)
+    p1, m1, v1 = oo.adam_update(p, g, z, z, 1)
+    # step 1: m = (1-b1) g, v = (1-b2) g^2, update = -lr * g / (|g| + eps)
+    assert np.allclose(m1, 0.1 * g, rtol=1e-6)
+    assert np.allclose(v1, 0.001 * g * g, rtol=1e-5)
+    want = p.astype(np.float64) - 1e-3 * g.astype(np.float64) / (np.abs(g.astype(np.float64)) + 1e-8)
+    assert np.allclose(p1, want, rtol=1e-6)
+    p64, m64, v64 = oo.adam_update_f64(p, g, z, z, 1)
+    assert np.allclose(p1, p64, rtol=1e-6) and np.allclose(m1, m64, rtol=1e-6)
+    # sign: a positive gradient decreases the parameter
+    assert np.all(np.sign(p1.astype(np.float64) - p) == -np.sign(g))
+
+
+def test_bias_corrections_are_python_doubles():
+    bc1, bc2 = oo.bias_corrections(3, 0.9, 0.999)
+    assert bc1 == 1.0 - 0.9 ** 3 and bc2 == 1.0 - 0.999 ** 3
+
+
+def test_mixed_precision_step_matches_torch_pipeline():
+    torch.manual_seed(10)
+    sizes = [33, 7, 129]
+    scale = 65536.0
+    p32 = [torch.randn(n) * 0.02 for n in sizes]
+    m = [torch.zeros(n) for n in sizes]
+    v = [torch.zeros(n) for n in sizes]
+    g = [(torch.randn(n) * 1e-3 * scale).bfloat16() for n in sizes]
+    res = oo.mixed_precision_step(
+        [t.float().numpy() for t in g], [t.numpy().copy() for t in p32],
+        [t.numpy().copy() for t in m], [t.numpy().copy() for t in v],
+        step=1, loss_scale=scale, max_norm=0.01)
+    tp = [t.clone() for t in p32]
+    tm = [t.clone() for t in m]
+    tv = [t.clone() for t in v]
+    tres = ot.optimizer_step(g, tp, tm, tv, 1, scale, max_norm=0.01)
+    assert res["overflow"] is False and tres["overflow"] is False
+    assert abs(res["total_norm"] - tres["total_norm"]) < 1e-6 * tres["total_norm"]
+    assert res["clip_coef"] < 1.0
+    for a, b in zip(res["p"], tp):
+        assert np.allclose(a, b.numpy(), rtol=1e-6, atol=0)
+    for a, b in zip(res["p_low"], tres["p_low"]):
+        assert np.array_equal(a, b.float().numpy())
+    # overflow: nothing changes
+    g[1][3] = float("inf")
+    res = oo.mixed_precision_step(
+        [t.float().numpy() for t in g], [t.numpy() for t in p32], [t.numpy() for t in m],
+        [t.numpy() for t in v], step=1, loss_scale=scale, max_norm=0.01)
+    assert res["overflow"] is True and res["p_low"] is None
+    for a, b in zip(res["p"], p32):
+        assert np.array_equal(a, b.numpy())
+
+
+def test_coalesce_layout():
+    a, b, c = np.arange(3.0), np.arange(4.0).reshape(2, 2) + 10, np.array([99.0])
+    flat, views = oo.coalesce([a, b, c])
+    assert np.array_equal(flat, [0, 1, 2, 10, 11, 12, 13, 99])
+    views[1][1, 0] = -1.0  # views alias the flat buffer
+    assert flat[5] == -1.0
+    t = torch._utils._flatten_dense_tensors([torch.tensor(a), torch.tensor(b) * 0 + torch.tensor(b), torch.tensor(c)])
+    assert t.numel() == flat.size
+    assert oo.group_offsets([3, 4, 1]) == [0, 3, 7, 8]
+
+
+def test_torch_cpu_mlp_step_matches_numpy_oracle():
+    """The 2-layer MLP configuration, small: the two independent restatements
+    agree on loss gradient and on the Adam-updated weights."""
+    torch.manual_seed(0)
+    B, D, Hd = 8, 16, 32
+    w1 = torch.nn.init.kaiming_uniform_(torch.empty(Hd, D), a=math.sqrt(5))
+    w2 = torch.nn.init.kaiming_uniform_(torch.empty(D, Hd), a=math.sqrt(5))
+    b1, b2 = torch.zeros(Hd), torch.zeros(D)
+    x, tgt = torch.randn(B, D), torch.randn(B, D)
+    res = ot.mlp_step(x, tgt, w1, b1, w2, b2)
+    # numpy oracle, float64
+    h, z1 = ol.linear_forward(x.numpy(), w1.numpy().reshape(-1), (Hd, D), bias=b1.numpy(),
+                              activation="gelu")
+    y, _ = ol.linear_forward(h, w2.numpy().reshape(-1), (D, Hd), bias=b2.numpy())
+    dy = 2.0 * (y - tgt.numpy()) / y.size
+    bw2 = ol.linear_backward(h, w2.numpy().reshape(-1), (D, Hd), dy, has_bias=True)
+    bw1 = ol.linear_backward(x.numpy(), w1.numpy().reshape(-1), (Hd, D), bw2["dx"], z=z1,
+                             activation="gelu", has_bias=True)
+    assert np.allclose(bw1["dw"].reshape(Hd, D), res["grads"][0].numpy(), rtol=1e-4, atol=1e-7)
+    assert np.allclose(bw1["db"], res["grads"][1].numpy(), rtol=1e-4, atol=1e-7)
+    assert np.allclose(bw2["dw"].reshape(D, Hd), res["grads"][2].numpy(), rtol=1e-4, atol=1e-7)
+    p1, _, _ = oo.adam_update(w1.numpy(), res["grads"][0].numpy(), 0 * w1.numpy(), 0 * w1.numpy(), 1)
+    assert np.allclose(p1, res["params"][0].numpy(), rtol=1e-6, atol=0)
