@@ -1,0 +1,376 @@
+#!/usr/bin/env python3
+"""Benchmark of the hot path on ONE MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A step is one forward + backward pass over the Llama-3-8B-shaped Linear set
+(4096 tokens; QKV 4096->6144, O 4096->4096, gate and up 4096->14336, down
+14336->4096; bf16 operands, fp32 accumulate, no bias): 15 GEMM launches through
+the C ABI of libaxn_gfx950.so on operands already resident in HBM.  `value` is
+the aggregate TFLOP/s over the set (algorithmic 6 M N K per layer).
+
+The same run also times, outside the main timed region and reported in extra
+keys of the one JSON line:
+  adam      the mixed-precision Adam step (scan + update) on 1.3e9 parameters in
+            64 ragged tensors, GB/s at 30 algorithmic bytes per element, and the
+            overflow (skip) variant
+  shapes    the 12B-style MLP shard with fused bias + GELU and the skinny
+            decode-like shard
+  cpu_baseline  the torch-CPU restatement of the same layer math on the host cores
+
+Every GEMM launch of the timed region is bracketed by HIP events on the launch
+stream; `roofline` reports the kernel with the largest share of the time.
+"""
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_BF16_TFLOPS = 2516.6   # MI355X dense bf16 MFMA
+PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
+
+LLAMA_SET = [  # (name, M, N, K), gate and up are two layers of one shape
+    ("qkv", 4096, 6144, 4096),
+    ("o", 4096, 4096, 4096),
+    ("gate", 4096, 14336, 4096),
+    ("up", 4096, 14336, 4096),
+    ("down", 4096, 4096, 14336),
+]
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-adam", action="store_true")
+    ap.add_argument("--no-extra-shapes", action="store_true")
+    ap.add_argument("--adam-elements", type=float, default=1.3e9)
+    return ap.parse_args()
+
+
+class Layer:
+    def __init__(self, name, M, N, K, seed, torch, bias=False):
+        g = torch.Generator(device="cuda").manual_seed(seed)
+        self.name, self.M, self.N, self.K = name, M, N, K
+        self.X = torch.randn(M, K, generator=g, device="cuda").bfloat16()
+        self.W = (torch.randn(N, K, generator=g, device="cuda") * 0.02).bfloat16()
+        self.dY = (torch.randn(M, N, generator=g, device="cuda") * 1e-3).bfloat16()
+        self.bias = (torch.randn(N, generator=g, device="cuda") * 0.1) if bias else None
+        self.Y = torch.empty(M, N, dtype=torch.bfloat16, device="cuda")
+        self.Z = torch.empty(M, N, dtype=torch.bfloat16, device="cuda") if bias else None
+        self.dZ = torch.empty(M, N, dtype=torch.bfloat16, device="cuda") if bias else None
+        self.dX = torch.empty(M, K, dtype=torch.bfloat16, device="cuda")
+        self.dW = torch.zeros(N, K, dtype=torch.bfloat16, device="cuda")
+        self.db = torch.zeros(N, device="cuda") if bias else None
+        self.flops = 6.0 * M * N * K
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py measures the per-GPU hot path on ONE GPU; --gpus %d is not supported "
+              "(nothing in this build uses a second GPU)" % args.gpus, file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    from axonn_amd import _native as nv
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(2)
+    lib = nv.load()
+    torch.cuda.set_device(0)
+    stream = nv.current_stream()
+
+    def fwd(L, epi=nv.EPI_NONE):
+        nv.check(lib.axn_gemm_fwd(L.X.data_ptr(), L.W.data_ptr(),
+                                  None if L.bias is None else L.bias.data_ptr(), L.Y.data_ptr(),
+                                  None if L.Z is None else L.Z.data_ptr(),
+                                  L.M, L.N, L.K, L.K, L.K, L.N, epi, stream))
+
+    def dgrad(L, dY=None):
+        nv.check(lib.axn_gemm_dgrad((dY if dY is not None else L.dY).data_ptr(), L.W.data_ptr(),
+                                    L.dX.data_ptr(), L.M, L.N, L.K, L.N, L.K, L.K, stream))
+
+    def wgrad(L, beta=0, dY=None):
+        nv.check(lib.axn_gemm_wgrad((dY if dY is not None else L.dY).data_ptr(), L.X.data_ptr(),
+                                    L.dW.data_ptr(), L.M, L.N, L.K, L.N, L.K, L.K, beta, nv.BF16,
+                                    stream))
+
+    layers = [Layer(n, M, N, K, i, torch) for i, (n, M, N, K) in enumerate(LLAMA_SET)]
+    total_flops = sum(L.flops for L in layers)
+
+    def ev():
+        return torch.cuda.Event(enable_timing=True)
+
+    spans = {"fwd": [], "dgrad": [], "wgrad": []}  # (start, end, flops) per launch
+
+    def timed(kind, fn, L):
+        s, e = ev(), ev()
+        s.record()
+        fn(L)
+        e.record()
+        spans[kind].append((s, e, L.flops / 3.0))
+
+    def step(record):
+        for L in layers:
+            timed("fwd", fwd, L) if record else fwd(L)
+        for L in reversed(layers):
+            timed("dgrad", dgrad, L) if record else dgrad(L)
+            timed("wgrad", wgrad, L) if record else wgrad(L)
+
+    for _ in range(args.warmup):
+        step(False)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step(True)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed / args.steps * 1e3
+    value = total_flops / (elapsed / args.steps) / 1e12
+
+    kinds = {}
+    for kind, lst in spans.items():
+        tot_ms = sum(s.elapsed_time(e) for s, e, _ in lst)
+        tot_fl = sum(f for _, _, f in lst)
+        kinds[kind] = {
+            "launches": len(lst), "avg_us": tot_ms / len(lst) * 1e3,
+            "tflops": tot_fl / (tot_ms * 1e-3) / 1e12, "total_ms": tot_ms,
+        }
+    dom = max(kinds, key=lambda k: kinds[k]["total_ms"])
+    kernel_names = {"fwd": "gemm_bf16_kernel<A K-major, B K-major> (Y = X W^T)",
+                    "dgrad": "gemm_bf16_kernel<A K-major, B MN-major> (dX = dY W)",
+                    "wgrad": "gemm_bf16_kernel<A MN-major, B MN-major> (dW = dY^T X)"}
+    roofline = {
+        "bound": "mfma", "kernel": kernel_names[dom],
+        "achieved": round(kinds[dom]["tflops"], 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+        "frac": round(kinds[dom]["tflops"] / PEAK_BF16_TFLOPS, 4),
+        "avg_launch_us": round(kinds[dom]["avg_us"], 1),
+        "flops_per_launch": kinds[dom]["tflops"] * 1e12 * kinds[dom]["avg_us"] * 1e-6,
+        "traffic": None,
+        "per_kernel": {k: {"avg_us": round(v["avg_us"], 1), "tflops": round(v["tflops"], 1),
+                           "frac": round(v["tflops"] / PEAK_BF16_TFLOPS, 4)}
+                       for k, v in kinds.items()},
+    }
+    del layers
+    torch.cuda.empty_cache()
+
+    def time_loop(fn, n, w=3):
+        for _ in range(w):
+            fn()
+        torch.cuda.synchronize()
+        s, e = ev(), ev()
+        s.record()
+        for _ in range(n):
+            fn()
+        e.record()
+        torch.cuda.synchronize()
+        return s.elapsed_time(e) / n * 1e-3
+
+    shapes = {}
+    if not args.no_extra_shapes:
+        # 12B-style MLP shard: bias + GELU fused, dW accumulated over 4 micro-batches
+        L = Layer("mlp_shard", 8192, 5120, 2560, 10, torch, bias=True)
+        ws_bytes = lib.axn_dgelu_dbias_workspace_bytes(L.M, L.N)
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device="cuda")
+
+        def mlp_shard_step():
+            for mb in range(4):
+                fwd(L, nv.EPI_BIAS_GELU)
+                nv.check(lib.axn_dgelu_dbias(L.dY.data_ptr(), L.Z.data_ptr(), L.dZ.data_ptr(),
+                                             nv.BF16, L.db.data_ptr(), L.M, L.N, L.N,
+                                             1 if mb else 0, ws.data_ptr(), ws_bytes, stream))
+                dgrad(L, L.dZ)
+                wgrad(L, 1 if mb else 0, L.dZ)
+
+        t = time_loop(mlp_shard_step, max(args.steps // 4, 3)) / 4
+        shapes["mlp_shard_8192x5120x2560_bias_gelu"] = {
+            "us_per_microbatch": round(t * 1e6, 1), "tflops": round(L.flops / t / 1e12, 1),
+            "frac_mfma": round(L.flops / t / 1e12 / PEAK_BF16_TFLOPS, 4)}
+        del L, ws
+        L = Layer("skinny", 512, 8192, 3584, 11, torch)
+
+        def skinny_step():
+            fwd(L)
+            dgrad(L)
+            wgrad(L)
+
+        t = time_loop(skinny_step, max(args.steps, 10))
+        nbytes = 6.0 * (L.M * L.K + L.N * L.K + L.M * L.N)
+        shapes["skinny_512x8192x3584"] = {
+            "us": round(t * 1e6, 1), "tflops": round(L.flops / t / 1e12, 1),
+            "frac_mfma": round(L.flops / t / 1e12 / PEAK_BF16_TFLOPS, 4),
+            "gbs": round(nbytes / t / 1e9, 1), "frac_hbm": round(nbytes / t / 1e9 / PEAK_HBM_GBS, 4)}
+        del L
+        torch.cuda.empty_cache()
+
+    adam = None
+    if not args.no_adam:
+        adam = bench_adam(args, torch, nv, lib, stream, time_loop)
+
+    cpu = None
+    if not args.no_cpu_baseline:
+        cpu = cpu_baseline(torch)
+        if adam is not None:
+            adam["cpu_baseline"] = cpu_adam_baseline(torch)
+
+    out = {
+        "metric": "Linear fwd+bwd TFLOP/s on the Llama-3-8B-shaped set (Adam step GB/s under 'adam')",
+        "value": round(value, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {
+            "workload": "llama3-8b-shaped Linear set, 4096 tokens: qkv 4096->6144, o 4096->4096, "
+                        "gate+up 4096->14336 (x2), down 14336->4096; fwd+bwd, bf16 in/out, fp32 "
+                        "accumulate, no bias; X~N(0,1), W~N(0,0.02), dY~N(0,1e-3)",
+            "flops_per_step": total_flops, "frac_of_mfma_peak": round(value / PEAK_BF16_TFLOPS, 4),
+        },
+        "roofline": roofline,
+        "cpu_baseline": cpu,
+        "adam": adam,
+        "shapes": shapes,
+    }
+    print(json.dumps(out))
+
+
+def adam_sizes(total, n=64, seed=0):
+    """64 ragged sizes: seeded fractions of the total clipped to [1e5, 6e7] (scaled
+    with the total), remainder onto the largest, sizes left odd on purpose."""
+    import numpy as np
+
+    scale = total / 1.3e9
+    frac = np.random.default_rng(seed).random(n)
+    sizes = np.clip((frac / frac.sum() * total).astype(np.int64), int(1e5 * scale), int(6e7 * scale))
+    sizes = sizes | 1
+    sizes[np.argmax(sizes)] += int(total) - int(sizes.sum())
+    return [int(s) for s in sizes]
+
+
+def bench_adam(args, torch, nv, lib, stream, time_loop):
+    import ctypes
+
+    total = int(args.adam_elements)
+    sizes = adam_sizes(total)
+    total = sum(sizes)
+    g = torch.Generator(device="cuda").manual_seed(1)
+    P = torch.empty(total, device="cuda").normal_(0, 0.02, generator=g)
+    G = torch.empty(total, dtype=torch.bfloat16, device="cuda")
+    chunk = 1 << 26
+    for o in range(0, total, chunk):  # bf16(N(0, 1e-3) * 65536) without a 5 GB fp32 temporary
+        n = min(chunk, total - o)
+        G[o:o + n] = (torch.randn(n, generator=g, device="cuda") * (1e-3 * 65536.0)).bfloat16()
+    M = torch.zeros(total, device="cuda")
+    V = torch.zeros(total, device="cuda")
+    PL = torch.empty(total, dtype=torch.bfloat16, device="cuda")
+
+    def arr(t):
+        a = (ctypes.c_void_p * len(sizes))()
+        off = 0
+        for i, n in enumerate(sizes):
+            a[i] = t.data_ptr() + off * t.element_size()
+            off += n
+        return a
+
+    ag, ap, am, av, apl = arr(G), arr(P), arr(M), arr(V), arr(PL)
+    asz = (ctypes.c_int64 * len(sizes))(*sizes)
+    ws_bytes = lib.axn_mt_scan_workspace_bytes(len(sizes), total)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device="cuda")
+    res = torch.zeros(8, dtype=torch.float32, device="cuda")
+    inv = 1.0 / 65536.0
+    state = {"t": 0}
+
+    def hp(t):
+        bc1, bc2 = 1 - 0.9 ** t, 1 - 0.999 ** t
+        return nv.AdamHParams(1e-3 / bc1, 1.0 / bc2 ** 0.5, 0.9, 1 - 0.9, 0.999, 1 - 0.999, 1e-8, 0.0)
+
+    def scan():
+        nv.check(lib.axn_mt_scan(ag, asz, len(sizes), nv.BF16, inv, 1.0, 0, res.data_ptr(),
+                                 ws.data_ptr(), ws_bytes, stream))
+
+    def update():
+        state["t"] += 1
+        nv.check(lib.axn_mt_adam(ag, ap, am, av, apl, asz, len(sizes), nv.BF16, nv.BF16, inv,
+                                 res.data_ptr(), hp(state["t"]), stream))
+
+    def full():
+        scan()
+        update()
+
+    n = max(min(args.steps, 10), 3)
+    t_full = time_loop(full, n, 2)
+    t_scan = time_loop(scan, n, 1)
+    t_upd = time_loop(update, n, 1)
+    found = int(res.view(torch.int32)[4].item())
+    # overflow variant: one +inf in tensor 17 -> scan only, every write skipped
+    off17 = sum(sizes[:17]) + 5
+    saved = G[off17].clone()
+    G[off17] = float("inf")
+    t_skip = time_loop(full, n, 1)
+    found_skip = int(res.view(torch.int32)[4].item())
+    G[off17] = saved
+    out = {
+        "elements": total, "tensors": len(sizes), "bytes_per_element": 30,
+        "ms_per_step": round(t_full * 1e3, 4),
+        "value": round(30.0 * total / t_full / 1e9, 1), "unit": "GB/s",
+        "roofline": {"bound": "hbm", "kernel": "mt_adam_kernel + mt_scan_kernel",
+                     "achieved": round(30.0 * total / t_full / 1e9, 1), "peak": PEAK_HBM_GBS,
+                     "unit": "GB/s", "frac": round(30.0 * total / t_full / 1e9 / PEAK_HBM_GBS, 4),
+                     "traffic": None},
+        "scan_ms": round(t_scan * 1e3, 4), "scan_gbs": round(2.0 * total / t_scan / 1e9, 1),
+        "update_ms": round(t_upd * 1e3, 4), "update_gbs": round(28.0 * total / t_upd / 1e9, 1),
+        "found_inf": found,
+        "skip_variant": {"ms_per_step": round(t_skip * 1e3, 4), "found_inf": found_skip,
+                         "gbs_at_2B_per_element": round(2.0 * total / t_skip / 1e9, 1)},
+    }
+    del P, G, M, V, PL, ws
+    torch.cuda.empty_cache()
+    return out
+
+
+def cpu_baseline(torch):
+    """The torch-CPU restatement of the layer math (oracle/torch_cpu.py) on the
+    host cores: fp32 fwd+bwd of the O-projection and QKV shapes, a bounded sample
+    of the step's 5 layers."""
+    from oracle import torch_cpu as ot
+
+    cores = torch.get_num_threads()
+    sample = [(4096, 4096, 4096), (4096, 6144, 4096)]
+    secs, flops = ot.time_linear_set(sample, reps=1)
+    return {"value": round(flops / secs / 1e12, 4), "unit": "TFLOP/s", "cores": cores,
+            "kind": "port",
+            "sample": "fp32 torch-CPU fwd+bwd of the o (4096x4096x4096) and qkv (4096x6144x4096) "
+                      "layers, 1 warm-up + 1 timed pass each (%.1f s)" % secs}
+
+
+def cpu_adam_baseline(torch):
+    from oracle import torch_cpu as ot
+
+    n = 1 << 24
+    g = torch.Generator().manual_seed(0)
+    p = torch.randn(n, generator=g) * 0.02
+    gr = (torch.randn(n, generator=g) * 1e-3 * 65536.0).bfloat16()
+    m, v = torch.zeros(n), torch.zeros(n)
+    ot.optimizer_step([gr], [p], [m], [v], 1, 65536.0, max_norm=1.0)
+    t0 = time.perf_counter()
+    reps = 3
+    for i in range(reps):
+        ot.optimizer_step([gr], [p], [m], [v], i + 2, 65536.0, max_norm=1.0)
+    secs = (time.perf_counter() - t0) / reps
+    return {"value": round(30.0 * n / secs / 1e9, 2), "unit": "GB/s",
+            "cores": torch.get_num_threads(), "kind": "port",
+            "sample": "torch-CPU unscale + overflow check + clip + Adam + bf16 cast on %d elements "
+                      "(1/77 of the workload), %d timed steps" % (n, reps)}
+
+
+if __name__ == "__main__":
+    main()
