@@ -12,7 +12,7 @@
 // Addressing.  The tensors of one launch (at most MT_MAX) travel in the kernel
 // argument block: pointers, sizes and a prefix sum of per-tensor chunk counts.
 // Workgroup b finds its tensor by binary search in that prefix sum (scalar
-// loads from the argument block) and owns MT_CHUNK consecutive elements of it.
+// loads from the argument block) and owns one chunk of consecutive elements of it.
 // Tensors are views into flat buffers at arbitrary element offsets
 // (axonn/utils.py:11-30), so each tensor starts with a scalar "head" of up to 7
 // elements after which every pointer of the tensor is 16-byte aligned; the
@@ -27,11 +27,44 @@
 namespace axn {
 namespace {
 
+#ifndef AXN_SCAN_CHUNK
+#define AXN_SCAN_CHUNK 65536
+#endif
+#ifndef AXN_ADAM_CHUNK
+#define AXN_ADAM_CHUNK 4096
+#endif
+#ifndef AXN_ADAM_UNROLL
+#define AXN_ADAM_UNROLL 1
+#endif
+#ifndef AXN_ADAM_NT_G
+#define AXN_ADAM_NT_G 1
+#endif
+#ifndef AXN_ADAM_NT_STORE
+#define AXN_ADAM_NT_STORE 1
+#endif
+
 constexpr int MT_MAX = 64;         // tensors per launch
 constexpr int MT_THREADS = 256;    // threads per workgroup
 constexpr int MT_VEC = 8;          // elements per lane per step
-constexpr int MT_UNROLL = 4;       // steps per workgroup per tensor chunk pass
-constexpr int MT_CHUNK = MT_THREADS * MT_VEC * MT_UNROLL * 2;  // 16384 elements
+// Elements per workgroup.  The read-only scan streams best in long runs with
+// non-temporal loads; the read-modify-write update does best with short runs,
+// cached loads, high occupancy (one vector per lane in flight) and
+// non-temporal stores.  Both measured on MI355X.
+constexpr int SCAN_CHUNK = AXN_SCAN_CHUNK;
+constexpr int ADAM_CHUNK = AXN_ADAM_CHUNK;
+constexpr int SCALE_CHUNK = 16384;
+constexpr int ADAM_UNROLL = AXN_ADAM_UNROLL;  // independent vectors per lane in flight
+
+// Memory access policies, compile-time per call site.
+template <bool NT, typename T>
+__device__ __forceinline__ T ld(const T* p) {
+  if (NT) return __builtin_nontemporal_load(p);
+  return *p;
+}
+template <bool NT, typename T>
+__device__ __forceinline__ void st(T v, T* p) {
+  if (NT) __builtin_nontemporal_store(v, p); else *p = v;
+}
 
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
@@ -49,6 +82,7 @@ struct MtTable {
   uint8_t head[MT_MAX];             // scalar elements before the aligned body
   uint8_t vec_ok[MT_MAX];           // 0: scalar accesses only
   int32_t n;
+  int32_t chunk;                    // elements per workgroup (multiple of MT_VEC)
 };
 
 struct ScanPartial {
@@ -92,21 +126,21 @@ template <> struct Lowp<AXN_F32> {
 };
 
 // 8 consecutive low-precision elements from a 16-byte aligned address.
-template <int DT>
+template <int DT, bool NT>
 __device__ __forceinline__ void load8(const void* base, int64_t i,
                                       typename Lowp<DT>::raw (&r)[8]) {
   typedef typename Lowp<DT>::raw raw;
   const raw* p = (const raw*)base + i;
   if (sizeof(raw) == 2) {
-    const u32x4 w = __builtin_nontemporal_load((const u32x4*)p);
+    const u32x4 w = ld<NT>((const u32x4*)p);
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
       r[2 * e] = (raw)(w[e] & 0xFFFFu);
       r[2 * e + 1] = (raw)(w[e] >> 16);
     }
   } else {
-    const u32x4 w0 = __builtin_nontemporal_load((const u32x4*)p);
-    const u32x4 w1 = __builtin_nontemporal_load((const u32x4*)p + 1);
+    const u32x4 w0 = ld<NT>((const u32x4*)p);
+    const u32x4 w1 = ld<NT>((const u32x4*)p + 1);
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
       r[e] = (raw)w0[e];
@@ -115,7 +149,7 @@ __device__ __forceinline__ void load8(const void* base, int64_t i,
   }
 }
 
-template <int DT>
+template <int DT, bool NT>
 __device__ __forceinline__ void store8(void* base, int64_t i,
                                        const typename Lowp<DT>::raw (&r)[8]) {
   typedef typename Lowp<DT>::raw raw;
@@ -125,7 +159,7 @@ __device__ __forceinline__ void store8(void* base, int64_t i,
 #pragma unroll
     for (int e = 0; e < 4; ++e)
       w[e] = (uint32_t)r[2 * e] | ((uint32_t)r[2 * e + 1] << 16);
-    __builtin_nontemporal_store(w, (u32x4*)p);
+    st<NT>(w, (u32x4*)p);
   } else {
     u32x4 w0, w1;
 #pragma unroll
@@ -133,24 +167,26 @@ __device__ __forceinline__ void store8(void* base, int64_t i,
       w0[e] = (uint32_t)r[e];
       w1[e] = (uint32_t)r[4 + e];
     }
-    __builtin_nontemporal_store(w0, (u32x4*)p);
-    __builtin_nontemporal_store(w1, (u32x4*)p + 1);
+    st<NT>(w0, (u32x4*)p);
+    st<NT>(w1, (u32x4*)p + 1);
   }
 }
 
+template <bool NT>
 __device__ __forceinline__ void loadf8(const float* p, float (&x)[8]) {
-  const f32x4 a = __builtin_nontemporal_load((const f32x4*)p);
-  const f32x4 b = __builtin_nontemporal_load((const f32x4*)p + 1);
+  const f32x4 a = ld<NT>((const f32x4*)p);
+  const f32x4 b = ld<NT>((const f32x4*)p + 1);
 #pragma unroll
   for (int e = 0; e < 4; ++e) {
     x[e] = a[e];
     x[4 + e] = b[e];
   }
 }
+template <bool NT>
 __device__ __forceinline__ void storef8(float* p, const float (&x)[8]) {
   f32x4 a = {x[0], x[1], x[2], x[3]}, b = {x[4], x[5], x[6], x[7]};
-  __builtin_nontemporal_store(a, (f32x4*)p);
-  __builtin_nontemporal_store(b, (f32x4*)p + 1);
+  st<NT>(a, (f32x4*)p);
+  st<NT>(b, (f32x4*)p + 1);
 }
 
 // Element range [begin, end) of tensor `t` owned by chunk `c`.  Chunk 0 also
@@ -161,8 +197,8 @@ struct Range {
 __device__ __forceinline__ Range chunk_range(const MtTable& tab, int t, int c) {
   const int64_t head = tab.head[t];
   Range r;
-  r.begin = head + (int64_t)c * MT_CHUNK;
-  r.end = r.begin + MT_CHUNK;
+  r.begin = head + (int64_t)c * tab.chunk;
+  r.end = r.begin + tab.chunk;
   if (r.end > tab.size[t]) r.end = tab.size[t];
   if (r.begin > r.end) r.begin = r.end;
   return r;
@@ -205,7 +241,7 @@ __global__ void __launch_bounds__(MT_THREADS)
     const int64_t nvec = (rg.end - rg.begin) / MT_VEC;
     for (int64_t i = tid; i < nvec; i += MT_THREADS) {
       raw r[8];
-      load8<DT>(g, rg.begin + i * MT_VEC, r);
+      load8<DT, true>(g, rg.begin + i * MT_VEC, r);
 #pragma unroll
       for (int e = 0; e < 8; ++e) one(r[e]);
     }
@@ -229,9 +265,15 @@ __global__ void __launch_bounds__(MT_THREADS)
   __syncthreads();
   if (tid == 0) {
     ScanPartial p;
-    p.sumsq = (s_sq[0] + s_sq[1]) + (s_sq[2] + s_sq[3]);
-    p.sum = (s_sm[0] + s_sm[1]) + (s_sm[2] + s_sm[3]);
-    p.nonfinite = s_bad[0] | s_bad[1] | s_bad[2] | s_bad[3];
+    p.sumsq = 0.f;
+    p.sum = 0.f;
+    p.nonfinite = 0;
+#pragma unroll
+    for (int w = 0; w < MT_THREADS / 64; ++w) {  // fixed order: deterministic
+      p.sumsq += s_sq[w];
+      p.sum += s_sm[w];
+      p.nonfinite |= s_bad[w];
+    }
     p.pad = 0;
     partial[block_base + blockIdx.x] = p;
   }
@@ -353,20 +395,20 @@ __global__ void __launch_bounds__(MT_THREADS)
     if (c == 0 && tid < tab.head[t]) one(tid);
     const int64_t nvec = (rg.end - rg.begin) / MT_VEC;
     int64_t i = tid;
-    // Main body: MT_UNROLL independent vectors per lane in flight.
-    for (; i + (MT_UNROLL - 1) * MT_THREADS < nvec; i += MT_UNROLL * MT_THREADS) {
-      graw gr[MT_UNROLL][8];
-      float pp[MT_UNROLL][8], mm[MT_UNROLL][8], vv[MT_UNROLL][8];
+    // Main body: ADAM_UNROLL independent vectors per lane in flight.
+    for (; i + (ADAM_UNROLL - 1) * MT_THREADS < nvec; i += ADAM_UNROLL * MT_THREADS) {
+      graw gr[ADAM_UNROLL][8];
+      float pp[ADAM_UNROLL][8], mm[ADAM_UNROLL][8], vv[ADAM_UNROLL][8];
 #pragma unroll
-      for (int u = 0; u < MT_UNROLL; ++u) {
+      for (int u = 0; u < ADAM_UNROLL; ++u) {
         const int64_t e0 = rg.begin + (i + u * MT_THREADS) * MT_VEC;
-        load8<GDT>(g, e0, gr[u]);
-        loadf8(p + e0, pp[u]);
-        loadf8(m + e0, mm[u]);
-        loadf8(v + e0, vv[u]);
+        load8<GDT, AXN_ADAM_NT_G != 0>(g, e0, gr[u]);
+        loadf8<false>(p + e0, pp[u]);
+        loadf8<false>(m + e0, mm[u]);
+        loadf8<false>(v + e0, vv[u]);
       }
 #pragma unroll
-      for (int u = 0; u < MT_UNROLL; ++u) {
+      for (int u = 0; u < ADAM_UNROLL; ++u) {
         const int64_t e0 = rg.begin + (i + u * MT_THREADS) * MT_VEC;
         praw pl[8];
 #pragma unroll
@@ -374,10 +416,10 @@ __global__ void __launch_bounds__(MT_THREADS)
           adam_math(Lowp<GDT>::to_float(gr[u][e]), pp[u][e], mm[u][e], vv[u][e], s, gmul);
           if (HAS_PLOW) pl[e] = Lowp<PDT>::from_float(pp[u][e]);
         }
-        storef8(p + e0, pp[u]);
-        storef8(m + e0, mm[u]);
-        storef8(v + e0, vv[u]);
-        if (HAS_PLOW) store8<PDT>(plow, e0, pl);
+        storef8<AXN_ADAM_NT_STORE != 0>(p + e0, pp[u]);
+        storef8<AXN_ADAM_NT_STORE != 0>(m + e0, mm[u]);
+        storef8<AXN_ADAM_NT_STORE != 0>(v + e0, vv[u]);
+        if (HAS_PLOW) store8<PDT, AXN_ADAM_NT_STORE != 0>(plow, e0, pl);
       }
     }
     for (; i < nvec; i += MT_THREADS) {
@@ -385,19 +427,19 @@ __global__ void __launch_bounds__(MT_THREADS)
       graw gr[8];
       float pp[8], mm[8], vv[8];
       praw pl[8];
-      load8<GDT>(g, e0, gr);
-      loadf8(p + e0, pp);
-      loadf8(m + e0, mm);
-      loadf8(v + e0, vv);
+      load8<GDT, AXN_ADAM_NT_G != 0>(g, e0, gr);
+      loadf8<false>(p + e0, pp);
+      loadf8<false>(m + e0, mm);
+      loadf8<false>(v + e0, vv);
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
         adam_math(Lowp<GDT>::to_float(gr[e]), pp[e], mm[e], vv[e], s, gmul);
         if (HAS_PLOW) pl[e] = Lowp<PDT>::from_float(pp[e]);
       }
-      storef8(p + e0, pp);
-      storef8(m + e0, mm);
-      storef8(v + e0, vv);
-      if (HAS_PLOW) store8<PDT>(plow, e0, pl);
+      storef8<AXN_ADAM_NT_STORE != 0>(p + e0, pp);
+      storef8<AXN_ADAM_NT_STORE != 0>(m + e0, mm);
+      storef8<AXN_ADAM_NT_STORE != 0>(v + e0, vv);
+      if (HAS_PLOW) store8<PDT, AXN_ADAM_NT_STORE != 0>(plow, e0, pl);
     }
     const int64_t tail = rg.begin + nvec * MT_VEC;
     if (tail + tid < rg.end) one(tail + tid);
@@ -430,10 +472,10 @@ __global__ void __launch_bounds__(MT_THREADS)
     const int64_t nvec = (rg.end - rg.begin) / MT_VEC;
     for (int64_t i = tid; i < nvec; i += MT_THREADS) {
       raw r[8];
-      load8<DT>(g, rg.begin + i * MT_VEC, r);
+      load8<DT, false>(g, rg.begin + i * MT_VEC, r);
 #pragma unroll
       for (int e = 0; e < 8; ++e) r[e] = f(r[e]);
-      store8<DT>(g, rg.begin + i * MT_VEC, r);
+      store8<DT, true>(g, rg.begin + i * MT_VEC, r);
     }
     const int64_t tail = rg.begin + nvec * MT_VEC;
     if (tail + tid < rg.end) ((raw*)g)[tail + tid] = f(((raw*)g)[tail + tid]);
@@ -475,7 +517,7 @@ struct Group {
 // Splits the tensor list into launch groups and fills the argument tables.
 // `ptr_sets[k][i]` is pointer k of tensor i (k = 0 is always the gradient).
 int build_groups(const void* const* const* ptr_sets, const int* elem_sizes,
-                 int nsets, const int64_t* h_sizes, int64_t n,
+                 int nsets, const int64_t* h_sizes, int64_t n, int chunk,
                  std::vector<Group>& out) {
   out.clear();
   Group cur;
@@ -485,6 +527,7 @@ int build_groups(const void* const* const* ptr_sets, const int* elem_sizes,
   auto flush = [&]() {
     if (k == 0) return;
     cur.tab.n = k;
+    cur.tab.chunk = chunk;
     cur.tab.chunk_start[k] = cur.blocks;
     out.push_back(cur);
     cur.tab = MtTable();
@@ -501,7 +544,7 @@ int build_groups(const void* const* const* ptr_sets, const int* elem_sizes,
     if (!vec_ok) head = 0;
     if (head > sz) head = (int)sz;
     const int64_t body = sz - head;
-    int64_t chunks = (body + MT_CHUNK - 1) / MT_CHUNK;
+    int64_t chunks = (body + chunk - 1) / chunk;
     if (chunks == 0) chunks = 1;  // the head still needs a workgroup
     if (chunks > 0x3fffffff) {
       set_error("multi-tensor: tensor %lld has too many elements (%lld)",
@@ -539,7 +582,7 @@ double sum_limit_of(int dt) {
 size_t mt_scan_workspace_bytes(int64_t n, int64_t total) {
   if (n < 0 || total < 0) return 0;
   // One partial per chunk; a tensor adds at most one ragged chunk.
-  const int64_t blocks = total / MT_CHUNK + 2 * n + 1;
+  const int64_t blocks = total / SCAN_CHUNK + 2 * n + 1;
   return (size_t)blocks * sizeof(ScanPartial);
 }
 
@@ -550,7 +593,7 @@ int launch_mt_scan(const void* const* h_g, const int64_t* h_sizes, int64_t n,
   const void* const* sets[1] = {h_g};
   const int es[1] = {dtype_size(g_dtype)};
   std::vector<Group> groups;
-  int rc = build_groups(sets, es, 1, h_sizes, n, groups);
+  int rc = build_groups(sets, es, 1, h_sizes, n, SCAN_CHUNK, groups);
   if (rc != AXN_OK) return rc;
   int64_t need = 0;
   for (auto& gr : groups) need += gr.blocks;
@@ -564,6 +607,7 @@ int launch_mt_scan(const void* const* h_g, const int64_t* h_sizes, int64_t n,
     // Nothing to scan: norm 0, no overflow.
     MtTable empty = MtTable();
     empty.n = 0;
+    empty.chunk = SCAN_CHUNK;
     hipLaunchKernelGGL(mt_scan_finalize_kernel, dim3(1), dim3(1024), 0, stream,
                        empty, partial, 0, sum_limit_of(g_dtype), max_norm,
                        accumulate ? 0 : 1, result);
@@ -625,7 +669,7 @@ int launch_mt_adam(const void* const* h_g, void* const* h_p, void* const* h_m,
                                 (const void* const*)h_v, (const void* const*)h_plow};
   const int es[5] = {dtype_size(g_dtype), 4, 4, 4, dtype_size(plow_dtype)};
   std::vector<Group> groups;
-  int rc = build_groups(sets, es, 5, h_sizes, n, groups);
+  int rc = build_groups(sets, es, 5, h_sizes, n, ADAM_CHUNK, groups);
   if (rc != AXN_OK) return rc;
   AdamScalars s;
   s.hp = hp;
@@ -648,7 +692,7 @@ int launch_mt_scale(void* const* h_g, const int64_t* h_sizes, int64_t n,
   const void* const* sets[1] = {(const void* const*)h_g};
   const int es[1] = {dtype_size(g_dtype)};
   std::vector<Group> groups;
-  int rc = build_groups(sets, es, 1, h_sizes, n, groups);
+  int rc = build_groups(sets, es, 1, h_sizes, n, SCALE_CHUNK, groups);
   if (rc != AXN_OK) return rc;
   for (auto& gr : groups) {
     const dim3 grid(gr.blocks), block(MT_THREADS);
