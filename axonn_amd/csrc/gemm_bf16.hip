@@ -3,13 +3,12 @@
 //   forward  Y  = X  W^T   (axonn/intra_layer/fully_connected.py:118)
 //   dgrad    dX = dY W     (fully_connected.py:140)
 //   wgrad    dW = dY^T X   (fully_connected.py:147-151)
-// as one templated kernel over the operand storage orders.
+// templated over the operand storage orders.
 //
-// Structure
+// Common to both kernels in this file
 //   * v_mfma_f32_32x32x16_bf16, fp32 accumulate in registers.
 //   * A workgroup owns a BM x BN output tile and walks the contraction in
-//     steps of 64; operand tiles are staged global -> VGPR -> LDS, double
-//     buffered, one workgroup barrier per step.
+//     steps of 64 through double-buffered LDS tiles.
 //   * LDS layouts are chosen per storage order so that fragment reads are free
 //     of bank conflicts on the 64-bank LDS:
 //       K-major  tile [rows][64]   : 16-byte chunk c of row r lives at chunk
@@ -25,6 +24,24 @@
 //     contiguous bytes and a row segment of 128 bytes is written by 8 lanes.
 //   * Workgroup ids are remapped so that each of the 8 XCDs (private L2 each)
 //     works on a compact block of neighbouring tiles.
+//
+// gemm_bf16_pingpong_kernel (whole 256 x 256 tiles, contraction % 64 == 0)
+//   8 waves, two per SIMD.  Operand tiles go global -> LDS directly
+//   (global_load_lds, 16 bytes per lane, no registers, no ds_write) into a ring
+//   of four 32-deep stages.  Every wave alternates between a memory cluster
+//   (the 12 fragment reads of one stage into registers) and a compute cluster
+//   (16 MFMAs on registers, with the wave's 4 copies of a stage three ahead
+//   issued between them).  The two waves of a SIMD run one cluster apart, so
+//   the matrix pipe always has a wave whose operands are already in registers
+//   while the other one waits on LDS, and the copies of all 8 waves trickle out
+//   evenly instead of in bursts that block instruction issue.
+//
+// gemm_bf16_kernel (any shape with N % 8 == 0 and K % 8 == 0)
+//   Operand tiles are staged global -> VGPR -> LDS with bounds checks, one
+//   barrier per step; used for ragged shapes and for problems too small to fill
+//   the chip with 256 x 256 tiles.
+#include <utility>
+
 #include "axn_internal.h"
 
 namespace axn {
@@ -33,6 +50,7 @@ namespace {
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
 typedef __attribute__((ext_vector_type(4))) short s16x4;
+typedef __attribute__((ext_vector_type(8))) short s16x8;
 typedef __attribute__((ext_vector_type(16))) float f32x16;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
@@ -42,6 +60,16 @@ constexpr int NUM_XCD = 8;      // MI355X: 8 accelerator dies, round-robin dispa
 constexpr int EPI_LD = 68;      // floats per row of the epilogue staging buffer
 
 #define LDS_PTR(T, p) ((__attribute__((address_space(3))) T*)(p))
+
+template <int... I, class F>
+__device__ __forceinline__ void static_for_impl(std::integer_sequence<int, I...>, F&& f) {
+  (f(std::integral_constant<int, I>{}), ...);
+}
+// Calls f(integral_constant<int, 0>) ... f(integral_constant<int, N - 1>).
+template <int N, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+  static_for_impl(std::make_integer_sequence<int, N>{}, f);
+}
 
 __device__ __forceinline__ float gelu_exact(float z) {
   return 0.5f * z * (1.0f + erff(z * 0.70710678118654752440f));
@@ -148,93 +176,28 @@ struct OperandTile {
       s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(s16x4, lds + off));
       s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
           LDS_PTR(s16x4, lds + off + 4 * (ROWS * 2)));
-      typedef __attribute__((ext_vector_type(8))) short s16x8;
       s16x8 v = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
       return __builtin_bit_cast(bf16x8, v);
     }
   }
 };
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, bool A_KMAJOR, bool B_KMAJOR,
-          int EPI, bool OUT_F32, bool EDGE>
-__global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
-    gemm_bf16_kernel(const GemmArgs g) {
-  constexpr int NT = WAVES_M * WAVES_N * 64;
-  constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N;
-  constexpr int FM = WTM / 32, FN = WTN / 32;
-  static_assert(WTM % 32 == 0 && WTN % 32 == 0, "wave tile must be 32-aligned");
-  using TA = OperandTile<BM, A_KMAJOR, NT, EDGE>;
-  using TB = OperandTile<BN, B_KMAJOR, NT, EDGE>;
-  constexpr int STAGE = TA::BYTES + TB::BYTES;
-
-  extern __shared__ __attribute__((aligned(16))) char lds[];
-
-  const int tid = threadIdx.x;
-  const int lane = tid & 63;
-  const int wave = tid >> 6;
-  const int wm = wave / WAVES_N, wn = wave % WAVES_N;
-
-  int tm, tn;
-  tile_of_workgroup(blockIdx.x, g.tiles_m, g.tiles_n, tm, tn);
-  const int m0 = tm * BM, n0 = tn * BN;
-
-  f32x16 acc[FM][FN];
-#pragma unroll
-  for (int i = 0; i < FM; ++i)
-#pragma unroll
-    for (int j = 0; j < FN; ++j)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
-
-  u32x4 ra[TA::PER_THREAD], rb[TB::PER_THREAD];
-  const int KT = (g.Kc + BK - 1) / BK;
-
-  TA::load(ra, g.A, g.lda, m0, g.M, 0, g.Kc, tid);
-  TB::load(rb, g.B, g.ldb, n0, g.N, 0, g.Kc, tid);
-  TA::store(ra, lds, tid);
-  TB::store(rb, lds + TA::BYTES, tid);
-  __syncthreads();
-
-  for (int kt = 0; kt < KT; ++kt) {
-    const char* sA = lds + (kt & 1) * STAGE;
-    const char* sB = sA + TA::BYTES;
-    const bool more = kt + 1 < KT;
-    if (more) {
-      TA::load(ra, g.A, g.lda, m0, g.M, (kt + 1) * BK, g.Kc, tid);
-      TB::load(rb, g.B, g.ldb, n0, g.N, (kt + 1) * BK, g.Kc, tid);
-    }
-#pragma unroll
-    for (int kk = 0; kk < BK / 16; ++kk) {
-      bf16x8 fa[FM], fb[FN];
-#pragma unroll
-      for (int i = 0; i < FM; ++i) fa[i] = TA::frag(sA, wm * WTM + i * 32, kk, lane);
-#pragma unroll
-      for (int j = 0; j < FN; ++j) fb[j] = TB::frag(sB, wn * WTN + j * 32, kk, lane);
-#pragma unroll
-      for (int i = 0; i < FM; ++i)
-#pragma unroll
-        for (int j = 0; j < FN; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[j], fa[i],
-                                                              acc[i][j], 0, 0, 0);
-    }
-    if (more) {
-      char* nA = lds + ((kt + 1) & 1) * STAGE;
-      TA::store(ra, nA, tid);
-      TB::store(rb, nA + TA::BYTES, tid);
-    }
-    __syncthreads();
-  }
-
-  // ---- epilogue -----------------------------------------------------------
-  // With the operands swapped, lane l register r of acc[i][j] is the output
-  // element  row = l % 32,  col = 8 * (r / 4) + 4 * (l / 32) + r % 4  of the
-  // 32 x 32 block (i, j) of this wave's tile.
+// Writes a wave's accumulators to C with the fused epilogue.  With the operands
+// swapped, lane l register r of acc[i][j] is the output element
+//   row = l % 32,  col = 8 * (r / 4) + 4 * (l / 32) + r % 4
+// of the 32 x 32 block (i, j) of the wave's tile.  Blocks are transposed through
+// a per-wave LDS buffer (32 rows x 64 fp32 columns, padded) so that every lane
+// then owns 8 consecutive columns of one row.  The caller must have made sure
+// that no wave still reads operand tiles from LDS.
+template <int FM, int FN, int EPI, bool OUT_F32, bool EDGE>
+__device__ __forceinline__ void store_tile(const f32x16 (&acc)[FM][FN], const GemmArgs& g,
+                                           char* lds, int wave, int lane, int row0,
+                                           int col0) {
+  constexpr int WTN = FN * 32;
   constexpr int EPC = (WTN < 64) ? WTN : 64;  // columns per staging pass
   constexpr int JP = EPC / 32;                // fragments per pass
   constexpr int LPR = EPC / 8;                // lanes per row on read-back
   constexpr int RPI = 64 / LPR;               // rows per read-back iteration
-  static_assert(32 * EPI_LD * 4 * WAVES_M * WAVES_N <= 2 * STAGE,
-                "epilogue staging must fit in the operand buffers");
   float* E = (float*)lds + wave * (32 * EPI_LD);
 
 #pragma unroll
@@ -257,8 +220,8 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
         const f32x4 v0 = *(const f32x4*)&E[r * EPI_LD + c];
         const f32x4 v1 = *(const f32x4*)&E[r * EPI_LD + c + 4];
         float v[8] = {v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
-        const int row = m0 + wm * WTM + i * 32 + r;
-        const int col = n0 + wn * WTN + jp * EPC + c;
+        const int row = row0 + i * 32 + r;
+        const int col = col0 + jp * EPC + c;
         if (EDGE && (row >= g.M || col >= g.N)) continue;
         const int64_t o = (int64_t)row * g.ldc + col;
         if (EPI == AXN_EPI_BIAS || EPI == AXN_EPI_BIAS_GELU) {
@@ -306,6 +269,358 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
   }
 }
 
+// ---------------------------------------------------------------------------
+// Ping-pong kernel.
+// ---------------------------------------------------------------------------
+template <int IMM>
+__device__ __forceinline__ bf16x8 lds_read_b128(uint32_t addr) {
+  bf16x8 v;
+  asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(IMM));
+  return v;
+}
+template <int IMM>
+__device__ __forceinline__ s16x4 lds_read_tr16_b64(uint32_t addr) {
+  s16x4 v;
+  asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(IMM));
+  return v;
+}
+
+// One operand of the ping-pong kernel: a 256-row x 32-deep tile (16 KiB), copied
+// by all 8 waves (2 copies each) and read as 32-row MFMA fragments.  The reads
+// are inline assembly: the compiler neither waits for them nor orders them
+// behind outstanding copies.
+//   K-major  tile [256][32]  : 64-byte rows, 16-byte chunk c of row r lives at
+//                              chunk c ^ ((r >> 2) & 3)
+//   MN-major tile [32][256]  : 512-byte rows, 64-byte chunk c of contraction row
+//                              k lives at chunk c ^ (k & 3)
+template <bool KMAJOR, int FR /* fragments per wave */>
+struct PingPongOperand {
+  static constexpr int ROWS = 256;
+  static constexpr int PK = 32;                  // contraction depth of a stage
+  static constexpr int BYTES = ROWS * PK * 2;    // 16 KiB
+  static constexpr int DMA_N = BYTES / 1024 / 8; // 2 copies per wave
+  static constexpr int NADDR = KMAJOR ? 2 : FR;  // address registers for the reads
+
+  // Source pointer of this lane for copy 0 of the tile at contraction offset 0,
+  // and the uniform element stride from copy i to copy i + 1.  Lane l of copy i
+  // lands at tile + (8 i + wave) * 1024 + 16 l, so the LDS swizzle is applied here.
+  __device__ __forceinline__ static const uint16_t* dma_base(const uint16_t* base, int64_t ld,
+                                                             int row0, int wave, int lane,
+                                                             int64_t& istride) {
+    if (KMAJOR) {
+      const int row = wave * 16 + (lane >> 2);        // + 128 i
+      const int c = (lane & 3) ^ ((row >> 2) & 3);    // 128 i does not change the swizzle
+      istride = 128 * ld;
+      return base + (int64_t)(row0 + row) * ld + c * 8;
+    } else {
+      const int k = wave * 2 + (lane >> 5);           // + 16 i
+      const int p16 = lane & 31;
+      const int c64 = (p16 >> 2) ^ (k & 3);           // 16 i does not change k & 3
+      istride = 16 * ld;
+      return base + (int64_t)k * ld + row0 + (c64 * 4 + (p16 & 3)) * 8;
+    }
+  }
+
+  template <int I>
+  __device__ __forceinline__ static void dma_one(const uint16_t* p, int64_t istride,
+                                                 char* lds_tile, int wave) {
+    static_assert(I >= 0 && I < DMA_N, "copy index");
+    __builtin_amdgcn_global_load_lds(
+        (const __attribute__((address_space(1))) void*)(p + I * istride),
+        LDS_PTR(void, lds_tile + (8 * I + wave) * 1024), 16, 0, 0);
+  }
+
+  // Per-lane LDS addresses (relative to the tile) the fragment reads start from.
+  __device__ __forceinline__ static void read_bases(uint32_t (&a)[NADDR], int wrow0, int lane) {
+    if (KMAJOR) {
+      const int r = wrow0 + (lane & 31);
+      const int swz = ((lane & 31) >> 2) & 3;
+#pragma unroll
+      for (int kk = 0; kk < 2; ++kk)
+        a[kk] = (uint32_t)(r * 64 + (((kk * 2 + (lane >> 5)) ^ swz) << 4));
+    } else {
+      const int kq = (lane & 15) >> 2;
+      const int k = 8 * (lane >> 5) + kq;
+#pragma unroll
+      for (int i = 0; i < FR; ++i) {
+        const int colbyte = (wrow0 + i * 32 + 16 * ((lane >> 4) & 1) + 4 * (lane & 3)) * 2;
+        a[i] = (uint32_t)(k * (ROWS * 2) + ((((colbyte >> 6) ^ kq) << 6) | (colbyte & 63)));
+      }
+    }
+  }
+
+  // All fragments of one stage: f[kk][i], 16 contraction elements x 32 rows each.
+  __device__ __forceinline__ static void read_all(bf16x8 (&f)[2][FR], const uint32_t (&a)[NADDR]) {
+    static_for<2>([&](auto kk_) {
+      constexpr int kk = decltype(kk_)::value;
+      static_for<FR>([&](auto i_) {
+        constexpr int i = decltype(i_)::value;
+        if constexpr (KMAJOR) {
+          f[kk][i] = lds_read_b128<i * 32 * 64>(a[kk]);
+        } else {
+          const s16x4 lo = lds_read_tr16_b64<kk * 16 * ROWS * 2>(a[i]);
+          const s16x4 hi = lds_read_tr16_b64<(kk * 16 + 4) * ROWS * 2>(a[i]);
+          f[kk][i] = __builtin_bit_cast(
+              bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+        }
+      });
+    });
+  }
+};
+
+// Schedule of the ping-pong kernel.  Stages of 256 x 256 x 32 (32 KiB) form a
+// ring of 4 in LDS.  Wave iteration i handles stage-tile i:
+//   memory cluster  : read the 12 fragments of tile i into registers, wait
+//   compute cluster : 16 MFMAs; between them this wave's 4 copies of tile i + 3
+// Group 0 (waves 0-3) runs its memory cluster in global cluster 2i and its
+// compute cluster in 2i + 1; group 1 (waves 4-7) one cluster later.  Tile i + 3
+// goes to the stage of tile i - 1, whose last reader (group 1, cluster 2i - 1)
+// finished before either group's compute cluster i starts; it is first read in
+// cluster 2i + 6, so every copy has at least three clusters to land.
+template <bool A_KMAJOR, bool B_KMAJOR, int EPI, bool OUT_F32>
+__global__ void __launch_bounds__(512) gemm_bf16_pingpong_kernel(const GemmArgs g) {
+  constexpr int BM = 256, BN = 256, WTM = 128, WTN = 64, FM = 4, FN = 2, KK = 2;
+  constexpr int PK = 32, NSTAGE = 4;
+  using OA = PingPongOperand<A_KMAJOR, FM>;
+  using OB = PingPongOperand<B_KMAJOR, FN>;
+  constexpr int STAGE = OA::BYTES + OB::BYTES;  // 32 KiB
+  static_assert(OA::DMA_N == 2 && OB::DMA_N == 2, "copy interleave below");
+
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: scalar branches
+  const int group = wave >> 2;  // 0: waves 0-3, 1: waves 4-7; one of each per SIMD
+  const int wm = group, wn = wave & 3;
+
+  int tm, tn;
+  tile_of_workgroup(blockIdx.x, g.tiles_m, g.tiles_n, tm, tn);
+  const int m0 = tm * BM, n0 = tn * BN;
+
+  f32x16 acc[FM][FN];
+#pragma unroll
+  for (int i = 0; i < FM; ++i)
+#pragma unroll
+    for (int j = 0; j < FN; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+  const int KT = g.Kc / PK;
+  int64_t a_is, b_is;
+  const uint16_t* pa = OA::dma_base(g.A, g.lda, m0, wave, lane, a_is);
+  const uint16_t* pb = OB::dma_base(g.B, g.ldb, n0, wave, lane, b_is);
+  const int64_t a_step = A_KMAJOR ? (int64_t)PK : (int64_t)PK * g.lda;
+  const int64_t b_step = B_KMAJOR ? (int64_t)PK : (int64_t)PK * g.ldb;
+
+  const uint32_t lds0 = (uint32_t)(uintptr_t)LDS_PTR(char, lds);
+  uint32_t ra0[OA::NADDR], rb0[OB::NADDR];
+  OA::read_bases(ra0, wm * WTM, lane);
+  OB::read_bases(rb0, wn * WTN, lane);
+#pragma unroll
+  for (int i = 0; i < OA::NADDR; ++i) ra0[i] += lds0;
+#pragma unroll
+  for (int i = 0; i < OB::NADDR; ++i) rb0[i] += lds0 + OA::BYTES;
+
+  // Tiles 0, 1, 2 up front; pa/pb then point at tile 3.
+#pragma unroll
+  for (int t = 0; t < NSTAGE - 1; ++t) {
+    if (t < KT) {
+      char* st = lds + t * STAGE;
+      OA::template dma_one<0>(pa, a_is, st, wave);
+      OA::template dma_one<1>(pa, a_is, st, wave);
+      OB::template dma_one<0>(pb, b_is, st + OA::BYTES, wave);
+      OB::template dma_one<1>(pb, b_is, st + OA::BYTES, wave);
+    }
+    pa += a_step;
+    pb += b_step;
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __builtin_amdgcn_s_barrier();
+  // Group 1 runs one cluster behind group 0 from here on.
+  if (group == 1) __builtin_amdgcn_s_barrier();
+
+#ifdef AXN_EXP_NOBARRIER
+#define AXN_LOOP_BARRIER()
+#else
+#define AXN_LOOP_BARRIER() __builtin_amdgcn_s_barrier()
+#endif
+  bf16x8 fa[KK][FM], fb[KK][FN];
+  // One wave iteration.  COPY: this wave's four copies of tile kt + 3 are issued
+  // between the MFMAs (steady state); otherwise the ring is draining.
+  // Copy completion: a wave's copies complete in order.  At the end of its memory
+  // cluster kt a wave has at most the copies of tiles kt + 1 (issued in compute
+  // cluster kt - 2) and kt + 2 (compute cluster kt - 1) in flight; tile kt + 1 is
+  // first read (by group 0) in the cluster after group 1's memory cluster kt, so
+  // both groups wait there until only the 4 copies of tile kt + 2 are left.
+  auto iteration = [&](int kt, auto copy_) {
+    constexpr bool COPY = decltype(copy_)::value;
+    const uint32_t cur = (uint32_t)(kt & (NSTAGE - 1)) * STAGE;
+    // ---- memory cluster ------------------------------------------------------
+    uint32_t ra[OA::NADDR], rb[OB::NADDR];
+#pragma unroll
+    for (int i = 0; i < OA::NADDR; ++i) ra[i] = ra0[i] + cur;
+#pragma unroll
+    for (int i = 0; i < OB::NADDR; ++i) rb[i] = rb0[i] + cur;
+#ifdef AXN_EXP_NOREAD
+    if (kt == 0) {
+      OA::read_all(fa, ra);
+      OB::read_all(fb, rb);
+    }
+#else
+    OA::read_all(fa, ra);
+    OB::read_all(fb, rb);
+#endif
+    // All 12 fragments flow through the wait, so no MFMA can move above it.
+    asm volatile("s_waitcnt lgkmcnt(0)"
+                 : "+v"(fa[0][0]), "+v"(fa[0][1]), "+v"(fa[0][2]), "+v"(fa[0][3]),
+                   "+v"(fa[1][0]), "+v"(fa[1][1]), "+v"(fa[1][2]), "+v"(fa[1][3]),
+                   "+v"(fb[0][0]), "+v"(fb[0][1]), "+v"(fb[1][0]), "+v"(fb[1][1]));
+    if (COPY) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
+    AXN_LOOP_BARRIER();
+    __builtin_amdgcn_sched_barrier(0);
+    // ---- compute cluster -----------------------------------------------------
+    char* dst = lds + (uint32_t)((kt + NSTAGE - 1) & (NSTAGE - 1)) * STAGE;
+    __builtin_amdgcn_s_setprio(1);
+    auto mfma4 = [&](int kk, int i0) {  // 4 MFMAs: rows i0, i0 + 1 x both column fragments
+#pragma unroll
+      for (int i = i0; i < i0 + 2; ++i)
+#pragma unroll
+        for (int j = 0; j < FN; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[kk][j], fa[kk][i],
+                                                              acc[i][j], 0, 0, 0);
+    };
+    mfma4(0, 0);
+    if (COPY) OA::template dma_one<0>(pa, a_is, dst, wave);
+    __builtin_amdgcn_sched_barrier(0);
+    mfma4(0, 2);
+    if (COPY) OB::template dma_one<0>(pb, b_is, dst + OA::BYTES, wave);
+    __builtin_amdgcn_sched_barrier(0);
+    mfma4(1, 0);
+    if (COPY) OA::template dma_one<1>(pa, a_is, dst, wave);
+    __builtin_amdgcn_sched_barrier(0);
+    mfma4(1, 2);
+    if (COPY) OB::template dma_one<1>(pb, b_is, dst + OA::BYTES, wave);
+    __builtin_amdgcn_s_setprio(0);
+    __builtin_amdgcn_sched_barrier(0);
+#ifndef AXN_EXP_SAMETILE
+    if (COPY) {
+      pa += a_step;
+      pb += b_step;
+    }
+#endif
+    AXN_LOOP_BARRIER();
+    __builtin_amdgcn_sched_barrier(0);
+  };
+#ifdef AXN_EXP_NODMA
+  const int steady = 0;
+#else
+  const int steady = KT - (NSTAGE - 1) > 0 ? KT - (NSTAGE - 1) : 0;
+#endif
+  for (int kt = 0; kt < steady; ++kt) iteration(kt, std::true_type{});
+  for (int kt = steady; kt < KT; ++kt) iteration(kt, std::false_type{});
+  if (group == 0) __builtin_amdgcn_s_barrier();  // group 1 is one barrier ahead in count
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+
+  store_tile<FM, FN, EPI, OUT_F32, false>(acc, g, lds, wave, lane, m0 + wm * WTM, n0 + wn * WTN);
+}
+
+// ---------------------------------------------------------------------------
+// Register-staged kernel.
+// ---------------------------------------------------------------------------
+template <int BM, int BN, int WAVES_M, int WAVES_N, bool A_KMAJOR, bool B_KMAJOR,
+          int EPI, bool OUT_F32, bool EDGE>
+__global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
+    gemm_bf16_kernel(const GemmArgs g) {
+  constexpr int NT = WAVES_M * WAVES_N * 64;
+  constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N;
+  constexpr int FM = WTM / 32, FN = WTN / 32;
+  static_assert(WTM % 32 == 0 && WTN % 32 == 0, "wave tile must be 32-aligned");
+  using TA = OperandTile<BM, A_KMAJOR, NT, EDGE>;
+  using TB = OperandTile<BN, B_KMAJOR, NT, EDGE>;
+  constexpr int STAGE = TA::BYTES + TB::BYTES;
+  static_assert(32 * EPI_LD * 4 * WAVES_M * WAVES_N <= 2 * STAGE,
+                "epilogue staging must fit in the operand buffers");
+
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+
+  int tm, tn;
+  tile_of_workgroup(blockIdx.x, g.tiles_m, g.tiles_n, tm, tn);
+  const int m0 = tm * BM, n0 = tn * BN;
+
+  f32x16 acc[FM][FN];
+#pragma unroll
+  for (int i = 0; i < FM; ++i)
+#pragma unroll
+    for (int j = 0; j < FN; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+  u32x4 ra[TA::PER_THREAD], rb[TB::PER_THREAD];
+  const int KT = (g.Kc + BK - 1) / BK;
+  constexpr int KK = BK / 16;  // MFMA steps per staged tile
+
+  TA::load(ra, g.A, g.lda, m0, g.M, 0, g.Kc, tid);
+  TB::load(rb, g.B, g.ldb, n0, g.N, 0, g.Kc, tid);
+  TA::store(ra, lds, tid);
+  TB::store(rb, lds + TA::BYTES, tid);
+  __syncthreads();
+
+  // Fragments are double buffered in registers: while the MFMAs of step kk
+  // run, the ds_reads of step kk + 1 are in flight.
+  bf16x8 fa[2][FM], fb[2][FN];
+  auto read_frags = [&](int buf, const char* sA, const char* sB, int kk) {
+#pragma unroll
+    for (int i = 0; i < FM; ++i) fa[buf][i] = TA::frag(sA, wm * WTM + i * 32, kk, lane);
+#pragma unroll
+    for (int j = 0; j < FN; ++j) fb[buf][j] = TB::frag(sB, wn * WTN + j * 32, kk, lane);
+  };
+  auto mfma_step = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < FM; ++i)
+#pragma unroll
+      for (int j = 0; j < FN; ++j)
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[buf][j], fa[buf][i],
+                                                            acc[i][j], 0, 0, 0);
+  };
+
+  read_frags(0, lds, lds + TA::BYTES, 0);
+  for (int kt = 0; kt < KT; ++kt) {
+    const char* sA = lds + (kt & 1) * STAGE;
+    const char* sB = sA + TA::BYTES;
+    char* nA = lds + ((kt + 1) & 1) * STAGE;
+    const bool more = kt + 1 < KT;
+    if (more) {
+      TA::load(ra, g.A, g.lda, m0, g.M, (kt + 1) * BK, g.Kc, tid);
+      TB::load(rb, g.B, g.ldb, n0, g.N, (kt + 1) * BK, g.Kc, tid);
+    }
+#pragma unroll
+    for (int kk = 0; kk < KK - 1; ++kk) {
+      read_frags((kk + 1) & 1, sA, sB, kk + 1);
+      mfma_step(kk & 1);
+    }
+    // Last step of this tile: every read of the current buffer has been issued,
+    // so the next tile can go to the other buffer while the MFMAs run.
+    if (more) {
+      TA::store(ra, nA, tid);
+      TB::store(rb, nA + TA::BYTES, tid);
+    }
+    mfma_step((KK - 1) & 1);
+    __syncthreads();
+    if (more) read_frags(0, nA, nA + TA::BYTES, 0);
+  }
+
+  store_tile<FM, FN, EPI, OUT_F32, EDGE>(acc, g, lds, wave, lane, m0 + wm * WTM, n0 + wn * WTN);
+}
+
 template <int BM, int BN, int WAVES_M, int WAVES_N, bool AK, bool BKM, int EPI,
           bool OUT_F32, bool EDGE>
 int launch_cfg(const GemmArgs& in, hipStream_t stream) {
@@ -315,13 +630,8 @@ int launch_cfg(const GemmArgs& in, hipStream_t stream) {
   constexpr int NT = WAVES_M * WAVES_N * 64;
   constexpr size_t lds = 2 * (size_t)(BM + BN) * BK * 2;
   auto kern = gemm_bf16_kernel<BM, BN, WAVES_M, WAVES_N, AK, BKM, EPI, OUT_F32, EDGE>;
-  static thread_local bool attr_set = false;
-  if (!attr_set) {
-    AXN_HIP_TRY(hipFuncSetAttribute((const void*)kern,
-                                    hipFuncAttributeMaxDynamicSharedMemorySize,
-                                    (int)lds));
-    attr_set = true;
-  }
+  AXN_HIP_TRY(hipFuncSetAttribute((const void*)kern,
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
   const long long nwg = (long long)g.tiles_m * g.tiles_n;
   if (nwg > 0x7fffffffLL) {
     set_error("gemm: too many output tiles (%lld)", nwg);
@@ -332,18 +642,35 @@ int launch_cfg(const GemmArgs& in, hipStream_t stream) {
   return AXN_OK;
 }
 
-// Tile selection.  Large aligned problems take 256 x 256 tiles on 8 waves;
-// problems that would leave most of the 256 CUs idle at that size, and ragged
-// ones, take 128 x 128 tiles with bounds checks.
+template <bool AK, bool BKM, int EPI, bool OUT_F32>
+int launch_pingpong(const GemmArgs& in, hipStream_t stream) {
+  GemmArgs g = in;
+  g.tiles_m = g.M / 256;
+  g.tiles_n = g.N / 256;
+  constexpr size_t lds = 4 * 2 * 256 * 32 * 2;  // ring of 4 stages, 128 KiB
+  auto kern = gemm_bf16_pingpong_kernel<AK, BKM, EPI, OUT_F32>;
+  AXN_HIP_TRY(hipFuncSetAttribute((const void*)kern,
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+  hipLaunchKernelGGL(kern, dim3((unsigned)(g.tiles_m * g.tiles_n)), dim3(512), lds, stream, g);
+  AXN_HIP_TRY(hipGetLastError());
+  return AXN_OK;
+}
+
+// Kernel selection.  Large problems made of whole 256 x 256 tiles take the
+// ping-pong kernel; problems that would leave most of the 256 CUs idle at that
+// tile size, and ragged ones, take 128 x 128 tiles on the register-staged kernel.
 template <bool AK, bool BKM, int EPI, bool OUT_F32>
 int launch_shape(const GemmArgs& g, hipStream_t stream) {
-  const bool aligned256 = (g.M % 256 == 0) && (g.N % 256 == 0) && (g.Kc % BK == 0);
+  const bool whole256 = (g.M % 256 == 0) && (g.N % 256 == 0) && (g.Kc % BK == 0);
   const long long tiles256 = (long long)((g.M + 255) / 256) * ((g.N + 255) / 256);
-  if (aligned256 && tiles256 >= 192)
+#ifndef AXN_NO_PINGPONG
+  if (whole256 && tiles256 >= 192) return launch_pingpong<AK, BKM, EPI, OUT_F32>(g, stream);
+#else
+  if (whole256 && tiles256 >= 192)
     return launch_cfg<256, 256, 2, 4, AK, BKM, EPI, OUT_F32, false>(g, stream);
-  const bool aligned128 = (g.M % 128 == 0) && (g.N % 128 == 0) && (g.Kc % BK == 0);
-  if (aligned128)
-    return launch_cfg<128, 128, 2, 2, AK, BKM, EPI, OUT_F32, false>(g, stream);
+#endif
+  const bool whole128 = (g.M % 128 == 0) && (g.N % 128 == 0) && (g.Kc % BK == 0);
+  if (whole128) return launch_cfg<128, 128, 2, 2, AK, BKM, EPI, OUT_F32, false>(g, stream);
   return launch_cfg<128, 128, 2, 2, AK, BKM, EPI, OUT_F32, true>(g, stream);
 }
 

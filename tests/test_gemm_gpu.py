@@ -182,6 +182,56 @@ def test_fp32_gemms_match_oracle(M, N, K):
     assert rel(dw.cpu().numpy(), 2 * bw["dw"].reshape(N, K)) < F32_TOL
 
 
+# ---- the 256 x 256 ping-pong kernel: few and many k-stages, all layouts/epilogues --------
+@pytest.mark.parametrize("K", [64, 128, 192, 256, 448])
+def test_pingpong_kernel_short_contractions(K):
+    """Shapes of >= 192 whole 256 x 256 tiles take the ping-pong kernel; its LDS
+    ring holds 4 stages of 32, so K = 64 .. 192 exercise the start-up and
+    drain paths (fewer stages than the ring) and 448 the steady state."""
+    from axonn_amd import ops
+
+    M, N = 4096, 3072
+    g = torch.Generator(device="cuda").manual_seed(K)
+    X = torch.randn(M, K, generator=g, device="cuda").bfloat16()
+    W = (torch.randn(N, K, generator=g, device="cuda") * 0.05).bfloat16()
+    b = torch.randn(N, generator=g, device="cuda")
+    y, z = ops.gemm_fwd(X, W, bias=b, activation="gelu", save_z=True)
+    zr = X.float() @ W.float().t() + b           # fp32 reference of the same op
+    assert rel(np64(z), np64(zr)) < BF16_TOL
+    assert rel(np64(y), np64(torch.nn.functional.gelu(zr))) < BF16_TOL
+    rows = torch.arange(0, M, 97, device="cuda")
+    yo, zo = ol.linear_forward(np64(X[rows]), np64(W).reshape(-1), (N, K), bias=np64(b),
+                               activation="gelu")
+    assert rel(np64(y[rows]), yo) < BF16_TOL and rel(np64(z[rows]), zo) < BF16_TOL
+
+
+@pytest.mark.parametrize("Kc", [64, 192, 320])
+def test_pingpong_kernel_backward_layouts(Kc):
+    """dgrad (B operand contraction-strided) and wgrad (both operands
+    contraction-strided, bf16 and fp32 accumulate) on the ping-pong kernel."""
+    from axonn_amd import ops
+
+    g = torch.Generator(device="cuda").manual_seed(Kc + 1)
+    # dgrad: dX[M, K] = dY[M, N] W[N, K], contraction N = Kc, output 4096 x 3072
+    dY = torch.randn(4096, Kc, generator=g, device="cuda").bfloat16()
+    W = torch.randn(Kc, 3072, generator=g, device="cuda").bfloat16()
+    dx = ops.gemm_dgrad(dY, W)
+    assert rel(np64(dx), np64(dY.float() @ W.float())) < BF16_TOL
+    # wgrad: dW[N, K] = dY[M, N]^T X[M, K], contraction M = Kc, output 3072 x 4096
+    dY2 = torch.randn(Kc, 3072, generator=g, device="cuda").bfloat16()
+    X2 = torch.randn(Kc, 4096, generator=g, device="cuda").bfloat16()
+    ref = dY2.float().t() @ X2.float()
+    dw = ops.gemm_wgrad(dY2, X2)
+    dw32 = ops.gemm_wgrad(dY2, X2, out_dtype=torch.float32)
+    assert rel(np64(dw), np64(ref)) < BF16_TOL
+    assert rel(np64(dw32), np64(ref)) < F32_TOL
+    ops.gemm_wgrad(dY2, X2, out=dw32, accumulate=True)
+    assert rel(np64(dw32), 2 * np64(ref)) < F32_TOL
+    rows = torch.arange(0, 3072, 61, device="cuda")
+    dwo = np64(dY2[:, rows]).T @ np64(X2)
+    assert rel(np64(dw32[rows]), 2 * dwo) < F32_TOL
+
+
 # ---- full benchmark shapes: size-independent properties + sampled oracle ------
 FULL = {
     "qkv": (4096, 6144, 4096), "o": (4096, 4096, 4096), "gate_up": (4096, 14336, 4096),
