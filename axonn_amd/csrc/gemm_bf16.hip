@@ -301,33 +301,35 @@ struct PingPongOperand {
   static constexpr int DMA_N = BYTES / 1024 / 8; // 2 copies per wave
   static constexpr int NADDR = KMAJOR ? 2 : FR;  // address registers for the reads
 
-  // Source pointer of this lane for copy 0 of the tile at contraction offset 0,
-  // and the uniform element stride from copy i to copy i + 1.  Lane l of copy i
+  // Copies are buffer loads to LDS: descriptor and tile offset in SGPRs, one
+  // constant 32-bit byte offset per lane in a VGPR, no address arithmetic per
+  // copy, and accesses past the operand return zeros instead of faulting.
+  // This is the lane's byte offset for copy 0 of the tile at contraction offset
+  // 0, and the uniform byte stride from copy i to copy i + 1.  Lane l of copy i
   // lands at tile + (8 i + wave) * 1024 + 16 l, so the LDS swizzle is applied here.
-  __device__ __forceinline__ static const uint16_t* dma_base(const uint16_t* base, int64_t ld,
-                                                             int row0, int wave, int lane,
-                                                             int64_t& istride) {
+  __device__ __forceinline__ static uint32_t dma_offset(int64_t ld, int row0, int wave,
+                                                        int lane, uint32_t& istride) {
     if (KMAJOR) {
       const int row = wave * 16 + (lane >> 2);        // + 128 i
       const int c = (lane & 3) ^ ((row >> 2) & 3);    // 128 i does not change the swizzle
-      istride = 128 * ld;
-      return base + (int64_t)(row0 + row) * ld + c * 8;
+      istride = (uint32_t)(128 * ld * 2);
+      return (uint32_t)(((int64_t)(row0 + row) * ld + c * 8) * 2);
     } else {
       const int k = wave * 2 + (lane >> 5);           // + 16 i
       const int p16 = lane & 31;
       const int c64 = (p16 >> 2) ^ (k & 3);           // 16 i does not change k & 3
-      istride = 16 * ld;
-      return base + (int64_t)k * ld + row0 + (c64 * 4 + (p16 & 3)) * 8;
+      istride = (uint32_t)(16 * ld * 2);
+      return (uint32_t)(((int64_t)k * ld + row0 + (c64 * 4 + (p16 & 3)) * 8) * 2);
     }
   }
 
   template <int I>
-  __device__ __forceinline__ static void dma_one(const uint16_t* p, int64_t istride,
+  __device__ __forceinline__ static void dma_one(__amdgpu_buffer_rsrc_t rsrc, uint32_t voff,
+                                                 uint32_t tile_ofs, uint32_t istride,
                                                  char* lds_tile, int wave) {
     static_assert(I >= 0 && I < DMA_N, "copy index");
-    __builtin_amdgcn_global_load_lds(
-        (const __attribute__((address_space(1))) void*)(p + I * istride),
-        LDS_PTR(void, lds_tile + (8 * I + wave) * 1024), 16, 0, 0);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, LDS_PTR(void, lds_tile + (8 * I + wave) * 1024),
+                                             16, (int)voff, (int)(tile_ofs + I * istride), 0, 0);
   }
 
   // Per-lane LDS addresses (relative to the tile) the fragment reads start from.
@@ -407,11 +409,20 @@ __global__ void __launch_bounds__(512) gemm_bf16_pingpong_kernel(const GemmArgs 
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
   const int KT = g.Kc / PK;
-  int64_t a_is, b_is;
-  const uint16_t* pa = OA::dma_base(g.A, g.lda, m0, wave, lane, a_is);
-  const uint16_t* pb = OB::dma_base(g.B, g.ldb, n0, wave, lane, b_is);
-  const int64_t a_step = A_KMAJOR ? (int64_t)PK : (int64_t)PK * g.lda;
-  const int64_t b_step = B_KMAJOR ? (int64_t)PK : (int64_t)PK * g.ldb;
+  // Operands as raw buffers (byte-addressed, range checked); the host side
+  // guarantees that each operand spans less than 2 GiB.
+  const uint32_t a_bytes = (uint32_t)((int64_t)(A_KMAJOR ? g.M : g.Kc) * g.lda * 2);
+  const uint32_t b_bytes = (uint32_t)((int64_t)(B_KMAJOR ? g.N : g.Kc) * g.ldb * 2);
+  const __amdgpu_buffer_rsrc_t ra_rsrc =
+      __builtin_amdgcn_make_buffer_rsrc((void*)g.A, 0, (int)a_bytes, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rb_rsrc =
+      __builtin_amdgcn_make_buffer_rsrc((void*)g.B, 0, (int)b_bytes, 0x00020000);
+  uint32_t a_is, b_is;
+  const uint32_t va = OA::dma_offset(g.lda, m0, wave, lane, a_is);
+  const uint32_t vb = OB::dma_offset(g.ldb, n0, wave, lane, b_is);
+  const uint32_t a_step = (uint32_t)((A_KMAJOR ? (int64_t)PK : (int64_t)PK * g.lda) * 2);
+  const uint32_t b_step = (uint32_t)((B_KMAJOR ? (int64_t)PK : (int64_t)PK * g.ldb) * 2);
+  uint32_t ka = 0, kb = 0;  // byte offset of the next tile to copy
 
   const uint32_t lds0 = (uint32_t)(uintptr_t)LDS_PTR(char, lds);
   uint32_t ra0[OA::NADDR], rb0[OB::NADDR];
@@ -422,18 +433,18 @@ __global__ void __launch_bounds__(512) gemm_bf16_pingpong_kernel(const GemmArgs 
 #pragma unroll
   for (int i = 0; i < OB::NADDR; ++i) rb0[i] += lds0 + OA::BYTES;
 
-  // Tiles 0, 1, 2 up front; pa/pb then point at tile 3.
+  // Tiles 0, 1, 2 up front; ka/kb then point at tile 3.
 #pragma unroll
   for (int t = 0; t < NSTAGE - 1; ++t) {
     if (t < KT) {
       char* st = lds + t * STAGE;
-      OA::template dma_one<0>(pa, a_is, st, wave);
-      OA::template dma_one<1>(pa, a_is, st, wave);
-      OB::template dma_one<0>(pb, b_is, st + OA::BYTES, wave);
-      OB::template dma_one<1>(pb, b_is, st + OA::BYTES, wave);
+      OA::template dma_one<0>(ra_rsrc, va, ka, a_is, st, wave);
+      OA::template dma_one<1>(ra_rsrc, va, ka, a_is, st, wave);
+      OB::template dma_one<0>(rb_rsrc, vb, kb, b_is, st + OA::BYTES, wave);
+      OB::template dma_one<1>(rb_rsrc, vb, kb, b_is, st + OA::BYTES, wave);
     }
-    pa += a_step;
-    pb += b_step;
+    ka += a_step;
+    kb += b_step;
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __builtin_amdgcn_s_barrier();
@@ -493,22 +504,22 @@ __global__ void __launch_bounds__(512) gemm_bf16_pingpong_kernel(const GemmArgs 
                                                               acc[i][j], 0, 0, 0);
     };
     mfma4(0, 0);
-    if (COPY) OA::template dma_one<0>(pa, a_is, dst, wave);
+    if (COPY) OA::template dma_one<0>(ra_rsrc, va, ka, a_is, dst, wave);
     __builtin_amdgcn_sched_barrier(0);
     mfma4(0, 2);
-    if (COPY) OB::template dma_one<0>(pb, b_is, dst + OA::BYTES, wave);
+    if (COPY) OB::template dma_one<0>(rb_rsrc, vb, kb, b_is, dst + OA::BYTES, wave);
     __builtin_amdgcn_sched_barrier(0);
     mfma4(1, 0);
-    if (COPY) OA::template dma_one<1>(pa, a_is, dst, wave);
+    if (COPY) OA::template dma_one<1>(ra_rsrc, va, ka, a_is, dst, wave);
     __builtin_amdgcn_sched_barrier(0);
     mfma4(1, 2);
-    if (COPY) OB::template dma_one<1>(pb, b_is, dst + OA::BYTES, wave);
+    if (COPY) OB::template dma_one<1>(rb_rsrc, vb, kb, b_is, dst + OA::BYTES, wave);
     __builtin_amdgcn_s_setprio(0);
     __builtin_amdgcn_sched_barrier(0);
 #ifndef AXN_EXP_SAMETILE
     if (COPY) {
-      pa += a_step;
-      pb += b_step;
+      ka += a_step;
+      kb += b_step;
     }
 #endif
     AXN_LOOP_BARRIER();
@@ -664,7 +675,12 @@ int launch_shape(const GemmArgs& g, hipStream_t stream) {
   const bool whole256 = (g.M % 256 == 0) && (g.N % 256 == 0) && (g.Kc % BK == 0);
   const long long tiles256 = (long long)((g.M + 255) / 256) * ((g.N + 255) / 256);
 #ifndef AXN_NO_PINGPONG
-  if (whole256 && tiles256 >= 192) return launch_pingpong<AK, BKM, EPI, OUT_F32>(g, stream);
+  // The ping-pong kernel addresses its operands with 32-bit byte offsets.
+  const int64_t a_span = (int64_t)(AK ? g.M : g.Kc) * g.lda * 2;
+  const int64_t b_span = (int64_t)(BKM ? g.N : g.Kc) * g.ldb * 2;
+  const bool small_spans = a_span < (1LL << 31) && b_span < (1LL << 31);
+  if (whole256 && tiles256 >= 192 && small_spans)
+    return launch_pingpong<AK, BKM, EPI, OUT_F32>(g, stream);
 #else
   if (whole256 && tiles256 >= 192)
     return launch_cfg<256, 256, 2, 4, AK, BKM, EPI, OUT_F32, false>(g, stream);
