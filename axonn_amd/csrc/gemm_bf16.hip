@@ -451,11 +451,6 @@ __global__ void __launch_bounds__(512) gemm_bf16_pingpong_kernel(const GemmArgs 
   // Group 1 runs one cluster behind group 0 from here on.
   if (group == 1) __builtin_amdgcn_s_barrier();
 
-#ifdef AXN_EXP_NOBARRIER
-#define AXN_LOOP_BARRIER()
-#else
-#define AXN_LOOP_BARRIER() __builtin_amdgcn_s_barrier()
-#endif
   bf16x8 fa[KK][FM], fb[KK][FN];
   // One wave iteration.  COPY: this wave's four copies of tile kt + 3 are issued
   // between the MFMAs (steady state); otherwise the ring is draining.
@@ -473,15 +468,8 @@ __global__ void __launch_bounds__(512) gemm_bf16_pingpong_kernel(const GemmArgs 
     for (int i = 0; i < OA::NADDR; ++i) ra[i] = ra0[i] + cur;
 #pragma unroll
     for (int i = 0; i < OB::NADDR; ++i) rb[i] = rb0[i] + cur;
-#ifdef AXN_EXP_NOREAD
-    if (kt == 0) {
-      OA::read_all(fa, ra);
-      OB::read_all(fb, rb);
-    }
-#else
     OA::read_all(fa, ra);
     OB::read_all(fb, rb);
-#endif
     // All 12 fragments flow through the wait, so no MFMA can move above it.
     asm volatile("s_waitcnt lgkmcnt(0)"
                  : "+v"(fa[0][0]), "+v"(fa[0][1]), "+v"(fa[0][2]), "+v"(fa[0][3]),
@@ -490,11 +478,10 @@ __global__ void __launch_bounds__(512) gemm_bf16_pingpong_kernel(const GemmArgs 
     if (COPY) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
     else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __builtin_amdgcn_sched_barrier(0);
-    AXN_LOOP_BARRIER();
+    __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_sched_barrier(0);
     // ---- compute cluster -----------------------------------------------------
     char* dst = lds + (uint32_t)((kt + NSTAGE - 1) & (NSTAGE - 1)) * STAGE;
-    __builtin_amdgcn_s_setprio(1);
     auto mfma4 = [&](int kk, int i0) {  // 4 MFMAs: rows i0, i0 + 1 x both column fragments
 #pragma unroll
       for (int i = i0; i < i0 + 2; ++i)
@@ -514,22 +501,15 @@ __global__ void __launch_bounds__(512) gemm_bf16_pingpong_kernel(const GemmArgs 
     __builtin_amdgcn_sched_barrier(0);
     mfma4(1, 2);
     if (COPY) OB::template dma_one<1>(rb_rsrc, vb, kb, b_is, dst + OA::BYTES, wave);
-    __builtin_amdgcn_s_setprio(0);
     __builtin_amdgcn_sched_barrier(0);
-#ifndef AXN_EXP_SAMETILE
     if (COPY) {
       ka += a_step;
       kb += b_step;
     }
-#endif
-    AXN_LOOP_BARRIER();
+    __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_sched_barrier(0);
   };
-#ifdef AXN_EXP_NODMA
-  const int steady = 0;
-#else
   const int steady = KT - (NSTAGE - 1) > 0 ? KT - (NSTAGE - 1) : 0;
-#endif
   for (int kt = 0; kt < steady; ++kt) iteration(kt, std::true_type{});
   for (int kt = steady; kt < KT; ++kt) iteration(kt, std::false_type{});
   if (group == 0) __builtin_amdgcn_s_barrier();  // group 1 is one barrier ahead in count
@@ -674,17 +654,12 @@ template <bool AK, bool BKM, int EPI, bool OUT_F32>
 int launch_shape(const GemmArgs& g, hipStream_t stream) {
   const bool whole256 = (g.M % 256 == 0) && (g.N % 256 == 0) && (g.Kc % BK == 0);
   const long long tiles256 = (long long)((g.M + 255) / 256) * ((g.N + 255) / 256);
-#ifndef AXN_NO_PINGPONG
   // The ping-pong kernel addresses its operands with 32-bit byte offsets.
   const int64_t a_span = (int64_t)(AK ? g.M : g.Kc) * g.lda * 2;
   const int64_t b_span = (int64_t)(BKM ? g.N : g.Kc) * g.ldb * 2;
   const bool small_spans = a_span < (1LL << 31) && b_span < (1LL << 31);
   if (whole256 && tiles256 >= 192 && small_spans)
     return launch_pingpong<AK, BKM, EPI, OUT_F32>(g, stream);
-#else
-  if (whole256 && tiles256 >= 192)
-    return launch_cfg<256, 256, 2, 4, AK, BKM, EPI, OUT_F32, false>(g, stream);
-#endif
   const bool whole128 = (g.M % 128 == 0) && (g.N % 128 == 0) && (g.Kc % BK == 0);
   if (whole128) return launch_cfg<128, 128, 2, 2, AK, BKM, EPI, OUT_F32, false>(g, stream);
   return launch_cfg<128, 128, 2, 2, AK, BKM, EPI, OUT_F32, true>(g, stream);

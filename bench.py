@@ -35,6 +35,14 @@ if ROOT not in sys.path:
 PEAK_BF16_TFLOPS = 2516.6   # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 
+# HBM bytes per launch (read + written), averaged over the launches of each kernel in
+# this workload, from `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE` runs of this
+# file, scaled by what the same counters read for the 1 GiB copy below
+# (profiles/gemm_pingpong_adam_llama_set_pmc.txt has the runs and the arithmetic).  The
+# counters sit between L2 and the fabric, so hits in the memory-side cache are included.
+TRAFFIC_BYTES_PER_LAUNCH = {"fwd": 634530629, "dgrad": 587315840, "wgrad": 687972470}
+ADAM_TRAFFIC_BYTES_PER_STEP = 39818604266   # scan + update, 1.3e9 elements
+
 LLAMA_SET = [  # (name, M, N, K), gate and up are two layers of one shape
     ("qkv", 4096, 6144, 4096),
     ("o", 4096, 4096, 4096),
@@ -109,6 +117,14 @@ def main():
     layers = [Layer(n, M, N, K, i, torch) for i, (n, M, N, K) in enumerate(LLAMA_SET)]
     total_flops = sum(L.flops for L in layers)
 
+    # One plain copy of known size (1 GiB read + 1 GiB written), outside every timed
+    # region: the yardstick that scales the FETCH_SIZE / WRITE_SIZE counters of a
+    # profiler run of this same command.
+    cal = torch.empty(1 << 28, dtype=torch.float32, device="cuda").normal_()
+    cal_dst = torch.empty_like(cal)
+    cal_dst.copy_(cal)
+    del cal, cal_dst
+
     def ev():
         return torch.cuda.Event(enable_timing=True)
 
@@ -148,16 +164,17 @@ def main():
             "tflops": tot_fl / (tot_ms * 1e-3) / 1e12, "total_ms": tot_ms,
         }
     dom = max(kinds, key=lambda k: kinds[k]["total_ms"])
-    kernel_names = {"fwd": "gemm_bf16_kernel<A K-major, B K-major> (Y = X W^T)",
-                    "dgrad": "gemm_bf16_kernel<A K-major, B MN-major> (dX = dY W)",
-                    "wgrad": "gemm_bf16_kernel<A MN-major, B MN-major> (dW = dY^T X)"}
+    # template arguments: <A contraction-contiguous, B contraction-contiguous, epilogue, fp32 out>
+    kernel_names = {"fwd": "gemm_bf16_pingpong_kernel<true, true, 0, false> (Y = X W^T)",
+                    "dgrad": "gemm_bf16_pingpong_kernel<true, false, 0, false> (dX = dY W)",
+                    "wgrad": "gemm_bf16_pingpong_kernel<false, false, 0, false> (dW = dY^T X)"}
     roofline = {
         "bound": "mfma", "kernel": kernel_names[dom],
         "achieved": round(kinds[dom]["tflops"], 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
         "frac": round(kinds[dom]["tflops"] / PEAK_BF16_TFLOPS, 4),
         "avg_launch_us": round(kinds[dom]["avg_us"], 1),
         "flops_per_launch": kinds[dom]["tflops"] * 1e12 * kinds[dom]["avg_us"] * 1e-6,
-        "traffic": None,
+        "traffic": TRAFFIC_BYTES_PER_LAUNCH.get(dom),
         "per_kernel": {k: {"avg_us": round(v["avg_us"], 1), "tflops": round(v["tflops"], 1),
                            "frac": round(v["tflops"] / PEAK_BF16_TFLOPS, 4)}
                        for k, v in kinds.items()},
@@ -325,7 +342,7 @@ def bench_adam(args, torch, nv, lib, stream, time_loop):
         "roofline": {"bound": "hbm", "kernel": "mt_adam_kernel + mt_scan_kernel",
                      "achieved": round(30.0 * total / t_full / 1e9, 1), "peak": PEAK_HBM_GBS,
                      "unit": "GB/s", "frac": round(30.0 * total / t_full / 1e9 / PEAK_HBM_GBS, 4),
-                     "traffic": None},
+                     "traffic": ADAM_TRAFFIC_BYTES_PER_STEP if total == 1300000000 else None},
         "scan_ms": round(t_scan * 1e3, 4), "scan_gbs": round(2.0 * total / t_scan / 1e9, 1),
         "update_ms": round(t_upd * 1e3, 4), "update_gbs": round(28.0 * total / t_upd / 1e9, 1),
         "found_inf": found,
@@ -344,12 +361,20 @@ def cpu_baseline(torch):
     from oracle import torch_cpu as ot
 
     cores = torch.get_num_threads()
-    sample = [(4096, 4096, 4096), (4096, 6144, 4096)]
+    sample = [(M, N, K) for _, M, N, K in LLAMA_SET]
+    # time_linear_set returns seconds and flops PER PASS over the set (after one
+    # warm-up pass per layer).  A first single pass sizes the sample: about 10 s of
+    # timed CPU work, so that with the warm-ups the leg stays under 30 s.
     secs, flops = ot.time_linear_set(sample, reps=1)
+    reps = 1
+    more = min(int(10.0 / max(secs, 1e-3)), 8)
+    if more >= 2:
+        secs, flops = ot.time_linear_set(sample, reps=more)
+        reps = more
     return {"value": round(flops / secs / 1e12, 4), "unit": "TFLOP/s", "cores": cores,
             "kind": "port",
-            "sample": "fp32 torch-CPU fwd+bwd of the o (4096x4096x4096) and qkv (4096x6144x4096) "
-                      "layers, 1 warm-up + 1 timed pass each (%.1f s)" % secs}
+            "sample": "fp32 torch-CPU fwd+bwd of all 5 layers of the step, %d timed passes "
+                      "(%.1f s of CPU work)" % (reps, secs * reps)}
 
 
 def cpu_adam_baseline(torch):
