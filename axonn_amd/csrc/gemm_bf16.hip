@@ -182,6 +182,54 @@ struct OperandTile {
   }
 };
 
+// Epilogue of 8 consecutive columns of one output row, held in fp32: bias,
+// exact GELU with optional save of the pre-activation, accumulation into the
+// existing output (beta), conversion and one 16- or 32-byte store.
+template <int EPI, bool OUT_F32>
+__device__ __forceinline__ void store_row8(float (&v)[8], const GemmArgs& g, int row, int col) {
+  const int64_t o = (int64_t)row * g.ldc + col;
+  if (EPI == AXN_EPI_BIAS || EPI == AXN_EPI_BIAS_GELU) {
+    const f32x4 b0 = *(const f32x4*)(g.bias + col);
+    const f32x4 b1 = *(const f32x4*)(g.bias + col + 4);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      v[e] += b0[e];
+      v[4 + e] += b1[e];
+    }
+  }
+  if (EPI == AXN_EPI_BIAS_GELU || EPI == AXN_EPI_GELU) {
+    if (g.Z != nullptr) {
+      bf16x8 z;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) z[e] = (__bf16)v[e];
+      *(bf16x8*)(g.Z + o) = z;
+    }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] = gelu_exact(v[e]);
+  }
+  if (OUT_F32) {
+    float* C = (float*)g.C + o;
+    f32x4 o0 = {v[0], v[1], v[2], v[3]}, o1 = {v[4], v[5], v[6], v[7]};
+    if (g.beta) {
+      o0 += *(const f32x4*)C;
+      o1 += *(const f32x4*)(C + 4);
+    }
+    *(f32x4*)C = o0;
+    *(f32x4*)(C + 4) = o1;
+  } else {
+    uint16_t* C = (uint16_t*)g.C + o;
+    if (g.beta) {
+      const bf16x8 old = *(const bf16x8*)C;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v[e] += (float)old[e];
+    }
+    bf16x8 y;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) y[e] = (__bf16)v[e];
+    *(bf16x8*)C = y;
+  }
+}
+
 // Writes a wave's accumulators to C with the fused epilogue.  With the operands
 // swapped, lane l register r of acc[i][j] is the output element
 //   row = l % 32,  col = 8 * (r / 4) + 4 * (l / 32) + r % 4
@@ -223,47 +271,7 @@ __device__ __forceinline__ void store_tile(const f32x16 (&acc)[FM][FN], const Ge
         const int row = row0 + i * 32 + r;
         const int col = col0 + jp * EPC + c;
         if (EDGE && (row >= g.M || col >= g.N)) continue;
-        const int64_t o = (int64_t)row * g.ldc + col;
-        if (EPI == AXN_EPI_BIAS || EPI == AXN_EPI_BIAS_GELU) {
-          const f32x4 b0 = *(const f32x4*)(g.bias + col);
-          const f32x4 b1 = *(const f32x4*)(g.bias + col + 4);
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            v[e] += b0[e];
-            v[4 + e] += b1[e];
-          }
-        }
-        if (EPI == AXN_EPI_BIAS_GELU || EPI == AXN_EPI_GELU) {
-          if (g.Z != nullptr) {
-            bf16x8 z;
-#pragma unroll
-            for (int e = 0; e < 8; ++e) z[e] = (__bf16)v[e];
-            *(bf16x8*)(g.Z + o) = z;
-          }
-#pragma unroll
-          for (int e = 0; e < 8; ++e) v[e] = gelu_exact(v[e]);
-        }
-        if (OUT_F32) {
-          float* C = (float*)g.C + o;
-          f32x4 o0 = {v[0], v[1], v[2], v[3]}, o1 = {v[4], v[5], v[6], v[7]};
-          if (g.beta) {
-            o0 += *(const f32x4*)C;
-            o1 += *(const f32x4*)(C + 4);
-          }
-          *(f32x4*)C = o0;
-          *(f32x4*)(C + 4) = o1;
-        } else {
-          uint16_t* C = (uint16_t*)g.C + o;
-          if (g.beta) {
-            const bf16x8 old = *(const bf16x8*)C;
-#pragma unroll
-            for (int e = 0; e < 8; ++e) v[e] += (float)old[e];
-          }
-          bf16x8 y;
-#pragma unroll
-          for (int e = 0; e < 8; ++e) y[e] = (__bf16)v[e];
-          *(bf16x8*)C = y;
-        }
+        store_row8<EPI, OUT_F32>(v, g, row, col);
       }
     }
   }
@@ -293,12 +301,12 @@ __device__ __forceinline__ s16x4 lds_read_tr16_b64(uint32_t addr) {
 //                              chunk c ^ ((r >> 2) & 3)
 //   MN-major tile [32][256]  : 512-byte rows, 64-byte chunk c of contraction row
 //                              k lives at chunk c ^ (k & 3)
-template <bool KMAJOR, int FR /* fragments per wave */>
+template <bool KMAJOR, int FR /* fragments per wave */, int NW = 8 /* waves that copy */>
 struct PingPongOperand {
   static constexpr int ROWS = 256;
-  static constexpr int PK = 32;                  // contraction depth of a stage
-  static constexpr int BYTES = ROWS * PK * 2;    // 16 KiB
-  static constexpr int DMA_N = BYTES / 1024 / 8; // 2 copies per wave
+  static constexpr int PK = 32;                   // contraction depth of a stage
+  static constexpr int BYTES = ROWS * PK * 2;     // 16 KiB
+  static constexpr int DMA_N = BYTES / 1024 / NW; // copies per wave: 2 (8 waves) or 4 (4 waves)
   static constexpr int NADDR = KMAJOR ? 2 : FR;  // address registers for the reads
 
   // Copies are buffer loads to LDS: descriptor and tile offset in SGPRs, one
@@ -306,19 +314,19 @@ struct PingPongOperand {
   // copy, and accesses past the operand return zeros instead of faulting.
   // This is the lane's byte offset for copy 0 of the tile at contraction offset
   // 0, and the uniform byte stride from copy i to copy i + 1.  Lane l of copy i
-  // lands at tile + (8 i + wave) * 1024 + 16 l, so the LDS swizzle is applied here.
+  // lands at tile + (NW i + wave) * 1024 + 16 l, so the LDS swizzle is applied here.
   __device__ __forceinline__ static uint32_t dma_offset(int64_t ld, int row0, int wave,
                                                         int lane, uint32_t& istride) {
     if (KMAJOR) {
-      const int row = wave * 16 + (lane >> 2);        // + 128 i
-      const int c = (lane & 3) ^ ((row >> 2) & 3);    // 128 i does not change the swizzle
-      istride = (uint32_t)(128 * ld * 2);
+      const int row = wave * 16 + (lane >> 2);        // + 16 NW i
+      const int c = (lane & 3) ^ ((row >> 2) & 3);    // 16 NW i does not change the swizzle
+      istride = (uint32_t)(16 * NW * ld * 2);
       return (uint32_t)(((int64_t)(row0 + row) * ld + c * 8) * 2);
     } else {
-      const int k = wave * 2 + (lane >> 5);           // + 16 i
+      const int k = wave * 2 + (lane >> 5);           // + 2 NW i
       const int p16 = lane & 31;
-      const int c64 = (p16 >> 2) ^ (k & 3);           // 16 i does not change k & 3
-      istride = (uint32_t)(16 * ld * 2);
+      const int c64 = (p16 >> 2) ^ (k & 3);           // 2 NW i (8 or 16) does not change k & 3
+      istride = (uint32_t)(2 * NW * ld * 2);
       return (uint32_t)(((int64_t)k * ld + row0 + (c64 * 4 + (p16 & 3)) * 8) * 2);
     }
   }
@@ -328,7 +336,7 @@ struct PingPongOperand {
                                                  uint32_t tile_ofs, uint32_t istride,
                                                  char* lds_tile, int wave) {
     static_assert(I >= 0 && I < DMA_N, "copy index");
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, LDS_PTR(void, lds_tile + (8 * I + wave) * 1024),
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, LDS_PTR(void, lds_tile + (NW * I + wave) * 1024),
                                              16, (int)voff, (int)(tile_ofs + I * istride), 0, 0);
   }
 
@@ -349,6 +357,36 @@ struct PingPongOperand {
         a[i] = (uint32_t)(k * (ROWS * 2) + ((((colbyte >> 6) ^ kq) << 6) | (colbyte & 63)));
       }
     }
+  }
+
+  // LDS read instructions behind one half (16 contraction elements) of a stage.
+  static constexpr int HALF_READS = KMAJOR ? FR : 2 * FR;
+
+  // Fragment I of contraction half KKH of a stage.
+  template <int KKH, int I>
+  __device__ __forceinline__ static void read_frag(bf16x8& f, const uint32_t (&a)[NADDR]) {
+    if constexpr (KMAJOR) {
+      f = lds_read_b128<I * 32 * 64>(a[KKH]);
+    } else {
+      const s16x4 lo = lds_read_tr16_b64<KKH * 16 * ROWS * 2>(a[I]);
+      const s16x4 hi = lds_read_tr16_b64<(KKH * 16 + 4) * ROWS * 2>(a[I]);
+      f = __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+    }
+  }
+
+  // The fragments of contraction half KKH of a stage: f[i], 16 x 32 each.
+  template <int KKH>
+  __device__ __forceinline__ static void read_half(bf16x8 (&f)[FR], const uint32_t (&a)[NADDR]) {
+    static_for<FR>([&](auto i_) {
+      constexpr int i = decltype(i_)::value;
+      if constexpr (KMAJOR) {
+        f[i] = lds_read_b128<i * 32 * 64>(a[KKH]);
+      } else {
+        const s16x4 lo = lds_read_tr16_b64<KKH * 16 * ROWS * 2>(a[i]);
+        const s16x4 hi = lds_read_tr16_b64<(KKH * 16 + 4) * ROWS * 2>(a[i]);
+        f[i] = __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+      }
+    });
   }
 
   // All fragments of one stage: f[kk][i], 16 contraction elements x 32 rows each.
@@ -520,6 +558,265 @@ __global__ void __launch_bounds__(512) gemm_bf16_pingpong_kernel(const GemmArgs 
 }
 
 // ---------------------------------------------------------------------------
+// One-wave-per-SIMD kernel: 64-deep operand tiles, v_mfma_f32_16x16x32_bf16.
+// ---------------------------------------------------------------------------
+// Measured on MI355X, which runs these kernels power-limited: at equal FLOPs the
+// 16x16x32 MFMA sustains about 10 % more clock than 32x32x16 (half the
+// accumulator traffic per FLOP), and LDS fragment reads cost clock rather than
+// issue slots.
+//
+// One operand tile: 256 rows x 64 deep (32 KiB), contraction-contiguous in
+// memory, copied by 4 waves (8 copies each) and read as 16-row x 32-deep MFMA
+// fragments (lane l: row l % 16, contraction elements 8 (l / 16) .. + 8).
+// Tile layout [256][64]: 128-byte rows = whole cache lines of the operand;
+// 16-byte chunk c of row r lives at chunk c ^ ((r >> 1) & 7), which spreads the
+// 16 lanes of a fragment quarter over all 64 banks.
+struct DeepOperand {
+  static constexpr int ROWS = 256;
+  static constexpr int PK = 64;
+  static constexpr int BYTES = ROWS * PK * 2;  // 32 KiB
+  static constexpr int NW = 4;
+  static constexpr int DMA_N = BYTES / 1024 / NW;  // 8 copies per wave
+  static constexpr int NADDR = 2;
+
+  // Byte offset of this lane's 16 bytes for copy 0 of the tile at contraction
+  // offset 0, and the uniform stride from copy i to i + 1.  Lane l of copy i
+  // lands at tile + (4 i + wave) * 1024 + 16 l; the swizzle is applied here.
+  __device__ __forceinline__ static uint32_t dma_offset(int64_t ld, int row0, int wave,
+                                                        int lane, uint32_t& istride) {
+    const int row = wave * 8 + (lane >> 3);          // + 32 i
+    const int c = (lane & 7) ^ ((row >> 1) & 7);     // 32 i does not change the swizzle
+    istride = (uint32_t)(32 * ld * 2);
+    return (uint32_t)(((int64_t)(row0 + row) * ld + c * 8) * 2);
+  }
+
+  template <int I>
+  __device__ __forceinline__ static void dma_one(__amdgpu_buffer_rsrc_t rsrc, uint32_t voff,
+                                                 uint32_t tile_ofs, uint32_t istride,
+                                                 char* lds_tile, int wave) {
+    static_assert(I >= 0 && I < DMA_N, "copy index");
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, LDS_PTR(void, lds_tile + (NW * I + wave) * 1024),
+                                             16, (int)voff, (int)(tile_ofs + I * istride), 0, 0);
+  }
+
+  // Per-lane LDS byte offsets (relative to the tile) the fragment reads start
+  // from: a[s] for the 32-deep step s; fragment i adds 16 rows = 2048 bytes (the
+  // swizzle repeats every 16 rows).
+  __device__ __forceinline__ static void read_bases(uint32_t (&a)[NADDR], int wrow0, int lane) {
+    const int r = wrow0 + (lane & 15);
+    const int swz = (r >> 1) & 7;
+#pragma unroll
+    for (int st = 0; st < 2; ++st)
+      a[st] = (uint32_t)(r * 128 + (((st * 4 + (lane >> 4)) ^ swz) << 4));
+  }
+
+  // Fragment I (rows 16 I ..) of the 32-deep step ST of the tile.
+  template <int ST, int I>
+  __device__ __forceinline__ static void read_frag(bf16x8& f, const uint32_t (&a)[NADDR]) {
+    f = lds_read_b128<I * 16 * 128>(a[ST]);
+  }
+};
+
+// Waits for every outstanding LDS read; the fragments flow through the
+// statement, so no MFMA on them can move above the wait.
+__device__ __forceinline__ void wait_all_fragments(bf16x8 (&fa)[8], bf16x8 (&fb)[8]) {
+  asm volatile("s_waitcnt lgkmcnt(0)"
+               : "+v"(fa[0]), "+v"(fa[1]), "+v"(fa[2]), "+v"(fa[3]), "+v"(fa[4]), "+v"(fa[5]),
+                 "+v"(fa[6]), "+v"(fa[7]), "+v"(fb[0]), "+v"(fb[1]), "+v"(fb[2]), "+v"(fb[3]),
+                 "+v"(fb[4]), "+v"(fb[5]), "+v"(fb[6]), "+v"(fb[7]));
+}
+
+// Accumulators of the 16 x 16 blocks of a wave's 128 x 128 tile to C.  With the
+// operands swapped, lane l register r of acc[i][j] is the output element
+//   row = 16 i + l % 16,  col = 16 j + 4 (l / 16) + r.
+// 32 rows x 64 columns at a time go through the wave's LDS buffer, after which
+// every lane owns 8 consecutive columns of one row.
+template <int EPI, bool OUT_F32>
+__device__ __forceinline__ void store_tile16(const f32x4 (&acc)[8][8], const GemmArgs& g, char* lds,
+                                             int wave, int lane, int row0, int col0) {
+  float* E = (float*)lds + wave * (32 * EPI_LD);
+#pragma unroll
+  for (int ip = 0; ip < 4; ++ip) {
+#pragma unroll
+    for (int jp = 0; jp < 2; ++jp) {
+#pragma unroll
+      for (int ii = 0; ii < 2; ++ii)
+#pragma unroll
+        for (int jj = 0; jj < 4; ++jj)
+          *(f32x4*)&E[(ii * 16 + (lane & 15)) * EPI_LD + jj * 16 + 4 * (lane >> 4)] =
+              acc[ip * 2 + ii][jp * 4 + jj];
+#pragma unroll
+      for (int it = 0; it < 4; ++it) {
+        const int r = it * 8 + (lane >> 3);
+        const int c = (lane & 7) * 8;
+        const f32x4 v0 = *(const f32x4*)&E[r * EPI_LD + c];
+        const f32x4 v1 = *(const f32x4*)&E[r * EPI_LD + c + 4];
+        float v[8] = {v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
+        store_row8<EPI, OUT_F32>(v, g, row0 + ip * 32 + r, col0 + jp * 64 + c);
+      }
+    }
+  }
+}
+
+// 4 waves, one per SIMD, each owning 128 x 128 of the 256 x 256 tile: 8 x 8
+// blocks of 16 x 16, 256 accumulator registers, 64 MFMAs per 32-deep step.  A
+// wave pipelines against itself: while the MFMAs of one step run on one register
+// set (8 + 8 fragments), the fragments of the next step are read into the other,
+// one fragment between two MFMAs.
+//
+// LDS holds a ring of 5 operand tiles (160 KiB); the tiles A0 B0 A1 B1 A2 ... of
+// the contraction stages take the slots 0 1 2 3 4 0 1 ...  Stage p (64 deep):
+//   step 0 : MFMAs | reads of (p, 1) | this wave's 8 copies of A(p+2)
+//   step 1 : wait for own copies of A(p+1), B(p+1); barrier;
+//            MFMAs | reads of (p+1, 0) | this wave's 8 copies of B(p+2)
+// At the barrier every wave holds the last fragments of stage p in registers, so
+// both of its slots are free: B(p+2) takes A(p)'s, A(p+3) (next step 0) B(p)'s.
+// A tile has at least two steps (128 MFMAs per wave) to land.
+template <int EPI, bool OUT_F32>
+__global__ void __launch_bounds__(256) gemm_bf16_solo_kernel(const GemmArgs g) {
+  constexpr int BM = 256, BN = 256, WTM = 128, WTN = 128, FR = 8;
+  constexpr int PK = 64, NSLOT = 5;
+  constexpr bool A_KMAJOR = true, B_KMAJOR = true;  // both operands contraction-contiguous
+  using OA = DeepOperand;
+  using OB = DeepOperand;
+  constexpr uint32_t SLOT = OA::BYTES;  // 32 KiB
+  static_assert(OA::DMA_N == 8 && OB::DMA_N == 8 && OA::BYTES == OB::BYTES, "copy schedule below");
+
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave >> 1, wn = wave & 1;
+
+  int tm, tn;
+  tile_of_workgroup(blockIdx.x, g.tiles_m, g.tiles_n, tm, tn);
+  const int m0 = tm * BM, n0 = tn * BN;
+
+  f32x4 acc[FR][FR];
+#pragma unroll
+  for (int i = 0; i < FR; ++i)
+#pragma unroll
+    for (int j = 0; j < FR; ++j) acc[i][j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+
+  const int KP = g.Kc / PK;  // stages
+  const uint32_t a_bytes = (uint32_t)((int64_t)(A_KMAJOR ? g.M : g.Kc) * g.lda * 2);
+  const uint32_t b_bytes = (uint32_t)((int64_t)(B_KMAJOR ? g.N : g.Kc) * g.ldb * 2);
+  const __amdgpu_buffer_rsrc_t ra_rsrc =
+      __builtin_amdgcn_make_buffer_rsrc((void*)g.A, 0, (int)a_bytes, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rb_rsrc =
+      __builtin_amdgcn_make_buffer_rsrc((void*)g.B, 0, (int)b_bytes, 0x00020000);
+  uint32_t a_is, b_is;
+  const uint32_t va = OA::dma_offset(g.lda, m0, wave, lane, a_is);
+  const uint32_t vb = OB::dma_offset(g.ldb, n0, wave, lane, b_is);
+  const uint32_t a_step = (uint32_t)((A_KMAJOR ? (int64_t)PK : (int64_t)PK * g.lda) * 2);
+  const uint32_t b_step = (uint32_t)((B_KMAJOR ? (int64_t)PK : (int64_t)PK * g.ldb) * 2);
+  uint32_t ka = 0, kb = 0;  // byte offsets of the next A / B tile to copy
+  uint32_t wslot = 0;       // ring slot (byte offset) the next copied tile takes
+
+  const uint32_t lds0 = (uint32_t)(uintptr_t)LDS_PTR(char, lds);
+  uint32_t ra0[OA::NADDR], rb0[OB::NADDR];
+  OA::read_bases(ra0, wm * WTM, lane);
+  OB::read_bases(rb0, wn * WTN, lane);
+#pragma unroll
+  for (int i = 0; i < OA::NADDR; ++i) ra0[i] += lds0;
+#pragma unroll
+  for (int i = 0; i < OB::NADDR; ++i) rb0[i] += lds0;
+
+  auto next_slot = [&](uint32_t s_) { return s_ + SLOT == NSLOT * SLOT ? 0u : s_ + SLOT; };
+  auto copy_a = [&](auto c_) {
+    OA::template dma_one<decltype(c_)::value>(ra_rsrc, va, ka, a_is, lds + wslot, wave);
+  };
+  auto copy_b = [&](auto c_) {
+    OB::template dma_one<decltype(c_)::value>(rb_rsrc, vb, kb, b_is, lds + wslot, wave);
+  };
+  auto a_done = [&]() { ka += a_step; wslot = next_slot(wslot); };
+  auto b_done = [&]() { kb += b_step; wslot = next_slot(wslot); };
+
+  // A0 B0 (A1 B1) up front.
+  static_for<8>(copy_a); a_done();
+  static_for<8>(copy_b); b_done();
+  if (KP > 1) {
+    static_for<8>(copy_a); a_done();
+    static_for<8>(copy_b); b_done();
+    asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+  } else {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  }
+  __builtin_amdgcn_s_barrier();
+
+  bf16x8 fa0[FR], fb0[FR], fa1[FR], fb1[FR];  // register sets of steps 0 / 1
+  // fragment f of 16 (A 0-7, B 0-7) of step ST of the stage whose tiles sit at
+  // sa / sb, into register set ST
+  auto read = [&](auto st_, auto f_, uint32_t sa, uint32_t sb) {
+    constexpr int ST = decltype(st_)::value, f = decltype(f_)::value;
+    bf16x8(&fa)[FR] = ST ? fa1 : fa0;
+    bf16x8(&fb)[FR] = ST ? fb1 : fb0;
+    if constexpr (f < FR) {
+      uint32_t ra[OA::NADDR];
+#pragma unroll
+      for (int i = 0; i < OA::NADDR; ++i) ra[i] = ra0[i] + sa;
+      OA::template read_frag<ST, f>(fa[f], ra);
+    } else {
+      uint32_t rb[OB::NADDR];
+#pragma unroll
+      for (int i = 0; i < OB::NADDR; ++i) rb[i] = rb0[i] + sb;
+      OB::template read_frag<ST, f - FR>(fb[f - FR], rb);
+    }
+  };
+  uint32_t sa = 0, sb = SLOT;  // slots of the current stage's tiles
+  static_for<16>([&](auto f_) { read(std::integral_constant<int, 0>{}, f_, sa, sb); });
+
+  // HAS2: stage p + 2 exists (its tiles are copied during this stage);
+  // LAST: no stage follows.
+  auto stage = [&](auto has2_, auto last_) {
+    constexpr bool HAS2 = decltype(has2_)::value;
+    constexpr bool LAST = decltype(last_)::value;
+    const uint32_t na = next_slot(sb), nb = next_slot(na);  // slots of stage p + 1
+    static_for<2>([&](auto st_) {
+      constexpr int ST = decltype(st_)::value;
+      bf16x8(&fa)[FR] = ST ? fa1 : fa0;
+      bf16x8(&fb)[FR] = ST ? fb1 : fb0;
+      wait_all_fragments(fa, fb);  // every read of this set was issued during the previous step
+      if constexpr (ST == 1 && !LAST) {
+        if (HAS2) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");  // A(p+2) may be in flight
+        else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      static_for<64>([&](auto m_) {
+        constexpr int m = decltype(m_)::value;
+        constexpr int i = m / FR, j = m % FR;
+        acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fb[j], fa[i], acc[i][j], 0, 0, 0);
+        if constexpr (m < 32 && m % 2 == 0) {
+          if constexpr (ST == 0) read(std::integral_constant<int, 1>{},
+                                      std::integral_constant<int, m / 2>{}, sa, sb);
+          else if constexpr (!LAST) read(std::integral_constant<int, 0>{},
+                                         std::integral_constant<int, m / 2>{}, na, nb);
+        } else if constexpr (HAS2 && m >= 32 && m % 4 == 1) {
+          if constexpr (ST == 0) copy_a(std::integral_constant<int, (m - 32) / 4>{});
+          else copy_b(std::integral_constant<int, (m - 32) / 4>{});
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      });
+      if constexpr (HAS2 && ST == 0) a_done();
+      if constexpr (HAS2 && ST == 1) b_done();
+    });
+    sa = na;
+    sb = nb;
+  };
+  using T = std::true_type;
+  using F = std::false_type;
+  for (int p = 0; p < KP - 2; ++p) stage(T{}, F{});
+  if (KP > 1) stage(F{}, F{});
+  stage(F{}, T{});
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+
+  store_tile16<EPI, OUT_F32>(acc, g, lds, wave, lane, m0 + wm * WTM, n0 + wn * WTN);
+}
+
+// ---------------------------------------------------------------------------
 // Register-staged kernel.
 // ---------------------------------------------------------------------------
 template <int BM, int BN, int WAVES_M, int WAVES_N, bool A_KMAJOR, bool B_KMAJOR,
@@ -647,9 +944,25 @@ int launch_pingpong(const GemmArgs& in, hipStream_t stream) {
   return AXN_OK;
 }
 
+template <int EPI, bool OUT_F32>
+int launch_solo(const GemmArgs& in, hipStream_t stream) {
+  GemmArgs g = in;
+  g.tiles_m = g.M / 256;
+  g.tiles_n = g.N / 256;
+  constexpr size_t lds = 5 * 256 * 64 * 2;  // ring of 5 operand tiles, 160 KiB: all of a CU's LDS
+  auto kern = gemm_bf16_solo_kernel<EPI, OUT_F32>;
+  AXN_HIP_TRY(hipFuncSetAttribute((const void*)kern,
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+  hipLaunchKernelGGL(kern, dim3((unsigned)(g.tiles_m * g.tiles_n)), dim3(256), lds, stream, g);
+  AXN_HIP_TRY(hipGetLastError());
+  return AXN_OK;
+}
+
 // Kernel selection.  Large problems made of whole 256 x 256 tiles take the
-// ping-pong kernel; problems that would leave most of the 256 CUs idle at that
-// tile size, and ragged ones, take 128 x 128 tiles on the register-staged kernel.
+// one-wave-per-SIMD kernel when both operands are contraction-contiguous (the
+// forward GEMM) and the ping-pong kernel otherwise; problems that would leave
+// most of the 256 CUs idle at that tile size, and ragged ones, take 128 x 128
+// tiles on the register-staged kernel.
 template <bool AK, bool BKM, int EPI, bool OUT_F32>
 int launch_shape(const GemmArgs& g, hipStream_t stream) {
   const bool whole256 = (g.M % 256 == 0) && (g.N % 256 == 0) && (g.Kc % BK == 0);
@@ -658,8 +971,10 @@ int launch_shape(const GemmArgs& g, hipStream_t stream) {
   const int64_t a_span = (int64_t)(AK ? g.M : g.Kc) * g.lda * 2;
   const int64_t b_span = (int64_t)(BKM ? g.N : g.Kc) * g.ldb * 2;
   const bool small_spans = a_span < (1LL << 31) && b_span < (1LL << 31);
-  if (whole256 && tiles256 >= 192 && small_spans)
-    return launch_pingpong<AK, BKM, EPI, OUT_F32>(g, stream);
+  if (whole256 && tiles256 >= 192 && small_spans) {
+    if constexpr (AK && BKM) return launch_solo<EPI, OUT_F32>(g, stream);
+    else return launch_pingpong<AK, BKM, EPI, OUT_F32>(g, stream);
+  }
   const bool whole128 = (g.M % 128 == 0) && (g.N % 128 == 0) && (g.Kc % BK == 0);
   if (whole128) return launch_cfg<128, 128, 2, 2, AK, BKM, EPI, OUT_F32, false>(g, stream);
   return launch_cfg<128, 128, 2, 2, AK, BKM, EPI, OUT_F32, true>(g, stream);
