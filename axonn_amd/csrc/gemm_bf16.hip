@@ -277,6 +277,39 @@ __device__ __forceinline__ void store_tile(const f32x16 (&acc)[FM][FN], const Ge
   }
 }
 
+// Same for accumulators of v_mfma_f32_16x16x32_bf16: FM x FN blocks of 16 x 16.
+// With the operands swapped, lane l register r of acc[i][j] is the output element
+//   row = 16 i + l % 16,  col = 16 j + 4 (l / 16) + r.
+// 32 rows x 64 columns at a time go through the wave's LDS buffer, after which
+// every lane owns 8 consecutive columns of one row.
+template <int FM, int FN, int EPI, bool OUT_F32>
+__device__ __forceinline__ void store_tile16(const f32x4 (&acc)[FM][FN], const GemmArgs& g,
+                                             char* lds, int wave, int lane, int row0, int col0) {
+  static_assert(FM % 2 == 0 && FN % 4 == 0, "staged in blocks of 32 x 64");
+  float* E = (float*)lds + wave * (32 * EPI_LD);
+#pragma unroll
+  for (int ip = 0; ip < FM / 2; ++ip) {
+#pragma unroll
+    for (int jp = 0; jp < FN / 4; ++jp) {
+#pragma unroll
+      for (int ii = 0; ii < 2; ++ii)
+#pragma unroll
+        for (int jj = 0; jj < 4; ++jj)
+          *(f32x4*)&E[(ii * 16 + (lane & 15)) * EPI_LD + jj * 16 + 4 * (lane >> 4)] =
+              acc[ip * 2 + ii][jp * 4 + jj];
+#pragma unroll
+      for (int it = 0; it < 4; ++it) {
+        const int r = it * 8 + (lane >> 3);
+        const int c = (lane & 7) * 8;
+        const f32x4 v0 = *(const f32x4*)&E[r * EPI_LD + c];
+        const f32x4 v1 = *(const f32x4*)&E[r * EPI_LD + c + 4];
+        float v[8] = {v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
+        store_row8<EPI, OUT_F32>(v, g, row0 + ip * 32 + r, col0 + jp * 64 + c);
+      }
+    }
+  }
+}
+
 // ---------------------------------------------------------------------------
 // Ping-pong kernel.
 // ---------------------------------------------------------------------------
@@ -294,39 +327,42 @@ __device__ __forceinline__ s16x4 lds_read_tr16_b64(uint32_t addr) {
 }
 
 // One operand of the ping-pong kernel: a 256-row x 32-deep tile (16 KiB), copied
-// by all 8 waves (2 copies each) and read as 32-row MFMA fragments.  The reads
-// are inline assembly: the compiler neither waits for them nor orders them
-// behind outstanding copies.
+// by all 8 waves (2 copies each) and read as 16-row x 32-deep MFMA fragments
+// (v_mfma_f32_16x16x32_bf16: lane l holds row l % 16, contraction elements
+// 8 (l / 16) .. + 8).  The reads are inline assembly: the compiler neither waits
+// for them nor orders them behind outstanding copies.
 //   K-major  tile [256][32]  : 64-byte rows, 16-byte chunk c of row r lives at
 //                              chunk c ^ ((r >> 2) & 3)
 //   MN-major tile [32][256]  : 512-byte rows, 64-byte chunk c of contraction row
-//                              k lives at chunk c ^ (k & 3)
-template <bool KMAJOR, int FR /* fragments per wave */, int NW = 8 /* waves that copy */>
+//                              k lives at chunk c ^ (k & 3); read with the
+//                              transposing ds_read_b64_tr_b16, two per fragment
+template <bool KMAJOR, int FR /* 16-row fragments per wave */>
 struct PingPongOperand {
   static constexpr int ROWS = 256;
   static constexpr int PK = 32;                   // contraction depth of a stage
   static constexpr int BYTES = ROWS * PK * 2;     // 16 KiB
-  static constexpr int DMA_N = BYTES / 1024 / NW; // copies per wave: 2 (8 waves) or 4 (4 waves)
-  static constexpr int NADDR = KMAJOR ? 2 : FR;  // address registers for the reads
+  static constexpr int NW = 8;                    // waves that copy
+  static constexpr int DMA_N = BYTES / 1024 / NW; // 2 copies per wave
+  static constexpr int NADDR = KMAJOR ? 1 : FR / 2;  // address registers for the reads
 
   // Copies are buffer loads to LDS: descriptor and tile offset in SGPRs, one
   // constant 32-bit byte offset per lane in a VGPR, no address arithmetic per
   // copy, and accesses past the operand return zeros instead of faulting.
   // This is the lane's byte offset for copy 0 of the tile at contraction offset
   // 0, and the uniform byte stride from copy i to copy i + 1.  Lane l of copy i
-  // lands at tile + (NW i + wave) * 1024 + 16 l, so the LDS swizzle is applied here.
+  // lands at tile + (8 i + wave) * 1024 + 16 l, so the LDS swizzle is applied here.
   __device__ __forceinline__ static uint32_t dma_offset(int64_t ld, int row0, int wave,
                                                         int lane, uint32_t& istride) {
     if (KMAJOR) {
-      const int row = wave * 16 + (lane >> 2);        // + 16 NW i
-      const int c = (lane & 3) ^ ((row >> 2) & 3);    // 16 NW i does not change the swizzle
-      istride = (uint32_t)(16 * NW * ld * 2);
+      const int row = wave * 16 + (lane >> 2);        // + 128 i
+      const int c = (lane & 3) ^ ((row >> 2) & 3);    // 128 i does not change the swizzle
+      istride = (uint32_t)(128 * ld * 2);
       return (uint32_t)(((int64_t)(row0 + row) * ld + c * 8) * 2);
     } else {
-      const int k = wave * 2 + (lane >> 5);           // + 2 NW i
+      const int k = wave * 2 + (lane >> 5);           // + 16 i
       const int p16 = lane & 31;
-      const int c64 = (p16 >> 2) ^ (k & 3);           // 2 NW i (8 or 16) does not change k & 3
-      istride = (uint32_t)(2 * NW * ld * 2);
+      const int c64 = (p16 >> 2) ^ (k & 3);           // 16 i does not change k & 3
+      istride = (uint32_t)(16 * ld * 2);
       return (uint32_t)(((int64_t)k * ld + row0 + (c64 * 4 + (p16 & 3)) * 8) * 2);
     }
   }
@@ -341,69 +377,38 @@ struct PingPongOperand {
   }
 
   // Per-lane LDS addresses (relative to the tile) the fragment reads start from.
+  //   K-major : one address; fragment i adds 16 rows = 1024 bytes (the swizzle
+  //             repeats every 16 rows).
+  //   MN-major: a[i >> 1] for fragment i, (i & 1) adds 32 bytes.  The 16 lanes of
+  //             a block address contraction rows 8 (l / 16) + (l & 15) / 4 and 4
+  //             columns each; the transposing read hands lane i of the block
+  //             column i of rows 8 (l / 16) + 0..3 (second read: rows + 4..7).
   __device__ __forceinline__ static void read_bases(uint32_t (&a)[NADDR], int wrow0, int lane) {
     if (KMAJOR) {
-      const int r = wrow0 + (lane & 31);
-      const int swz = ((lane & 31) >> 2) & 3;
-#pragma unroll
-      for (int kk = 0; kk < 2; ++kk)
-        a[kk] = (uint32_t)(r * 64 + (((kk * 2 + (lane >> 5)) ^ swz) << 4));
+      const int r = wrow0 + (lane & 15);
+      a[0] = (uint32_t)(r * 64 + (((lane >> 4) ^ ((r >> 2) & 3)) << 4));
     } else {
       const int kq = (lane & 15) >> 2;
-      const int k = 8 * (lane >> 5) + kq;
+      const int k = 8 * (lane >> 4) + kq;
 #pragma unroll
-      for (int i = 0; i < FR; ++i) {
-        const int colbyte = (wrow0 + i * 32 + 16 * ((lane >> 4) & 1) + 4 * (lane & 3)) * 2;
-        a[i] = (uint32_t)(k * (ROWS * 2) + ((((colbyte >> 6) ^ kq) << 6) | (colbyte & 63)));
+      for (int h = 0; h < NADDR; ++h) {
+        const int colbyte = (wrow0 + h * 32 + 4 * (lane & 3)) * 2;
+        a[h] = (uint32_t)(k * (ROWS * 2) + ((((colbyte >> 6) ^ kq) << 6) | (colbyte & 63)));
       }
     }
   }
 
-  // LDS read instructions behind one half (16 contraction elements) of a stage.
-  static constexpr int HALF_READS = KMAJOR ? FR : 2 * FR;
-
-  // Fragment I of contraction half KKH of a stage.
-  template <int KKH, int I>
-  __device__ __forceinline__ static void read_frag(bf16x8& f, const uint32_t (&a)[NADDR]) {
-    if constexpr (KMAJOR) {
-      f = lds_read_b128<I * 32 * 64>(a[KKH]);
-    } else {
-      const s16x4 lo = lds_read_tr16_b64<KKH * 16 * ROWS * 2>(a[I]);
-      const s16x4 hi = lds_read_tr16_b64<(KKH * 16 + 4) * ROWS * 2>(a[I]);
-      f = __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
-    }
-  }
-
-  // The fragments of contraction half KKH of a stage: f[i], 16 x 32 each.
-  template <int KKH>
-  __device__ __forceinline__ static void read_half(bf16x8 (&f)[FR], const uint32_t (&a)[NADDR]) {
+  // All fragments of one stage: f[i] = rows 16 i .. + 16, 32 contraction elements.
+  __device__ __forceinline__ static void read_all(bf16x8 (&f)[FR], const uint32_t (&a)[NADDR]) {
     static_for<FR>([&](auto i_) {
       constexpr int i = decltype(i_)::value;
       if constexpr (KMAJOR) {
-        f[i] = lds_read_b128<i * 32 * 64>(a[KKH]);
+        f[i] = lds_read_b128<i * 16 * 64>(a[0]);
       } else {
-        const s16x4 lo = lds_read_tr16_b64<KKH * 16 * ROWS * 2>(a[i]);
-        const s16x4 hi = lds_read_tr16_b64<(KKH * 16 + 4) * ROWS * 2>(a[i]);
+        const s16x4 lo = lds_read_tr16_b64<(i & 1) * 32>(a[i >> 1]);
+        const s16x4 hi = lds_read_tr16_b64<4 * ROWS * 2 + (i & 1) * 32>(a[i >> 1]);
         f[i] = __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
       }
-    });
-  }
-
-  // All fragments of one stage: f[kk][i], 16 contraction elements x 32 rows each.
-  __device__ __forceinline__ static void read_all(bf16x8 (&f)[2][FR], const uint32_t (&a)[NADDR]) {
-    static_for<2>([&](auto kk_) {
-      constexpr int kk = decltype(kk_)::value;
-      static_for<FR>([&](auto i_) {
-        constexpr int i = decltype(i_)::value;
-        if constexpr (KMAJOR) {
-          f[kk][i] = lds_read_b128<i * 32 * 64>(a[kk]);
-        } else {
-          const s16x4 lo = lds_read_tr16_b64<kk * 16 * ROWS * 2>(a[i]);
-          const s16x4 hi = lds_read_tr16_b64<(kk * 16 + 4) * ROWS * 2>(a[i]);
-          f[kk][i] = __builtin_bit_cast(
-              bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
-        }
-      });
     });
   }
 };
@@ -411,7 +416,9 @@ struct PingPongOperand {
 // Schedule of the ping-pong kernel.  Stages of 256 x 256 x 32 (32 KiB) form a
 // ring of 4 in LDS.  Wave iteration i handles stage-tile i:
 //   memory cluster  : read the 12 fragments of tile i into registers, wait
-//   compute cluster : 16 MFMAs; between them this wave's 4 copies of tile i + 3
+//   compute cluster : 32 MFMAs (16x16x32: at equal FLOPs this part, which runs
+//                     power-limited, sustains about 10 % more clock with them than
+//                     with 32x32x16); between them this wave's 4 copies of tile i + 3
 // Group 0 (waves 0-3) runs its memory cluster in global cluster 2i and its
 // compute cluster in 2i + 1; group 1 (waves 4-7) one cluster later.  Tile i + 3
 // goes to the stage of tile i - 1, whose last reader (group 1, cluster 2i - 1)
@@ -419,7 +426,7 @@ struct PingPongOperand {
 // cluster 2i + 6, so every copy has at least three clusters to land.
 template <bool A_KMAJOR, bool B_KMAJOR, int EPI, bool OUT_F32>
 __global__ void __launch_bounds__(512) gemm_bf16_pingpong_kernel(const GemmArgs g) {
-  constexpr int BM = 256, BN = 256, WTM = 128, WTN = 64, FM = 4, FN = 2, KK = 2;
+  constexpr int BM = 256, BN = 256, WTM = 128, WTN = 64, FM = 8, FN = 4;  // 16 x 16 blocks
   constexpr int PK = 32, NSTAGE = 4;
   using OA = PingPongOperand<A_KMAJOR, FM>;
   using OB = PingPongOperand<B_KMAJOR, FN>;
@@ -438,13 +445,11 @@ __global__ void __launch_bounds__(512) gemm_bf16_pingpong_kernel(const GemmArgs 
   tile_of_workgroup(blockIdx.x, g.tiles_m, g.tiles_n, tm, tn);
   const int m0 = tm * BM, n0 = tn * BN;
 
-  f32x16 acc[FM][FN];
+  f32x4 acc[FM][FN];
 #pragma unroll
   for (int i = 0; i < FM; ++i)
 #pragma unroll
-    for (int j = 0; j < FN; ++j)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+    for (int j = 0; j < FN; ++j) acc[i][j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
 
   const int KT = g.Kc / PK;
   // Operands as raw buffers (byte-addressed, range checked); the host side
@@ -489,7 +494,7 @@ __global__ void __launch_bounds__(512) gemm_bf16_pingpong_kernel(const GemmArgs 
   // Group 1 runs one cluster behind group 0 from here on.
   if (group == 1) __builtin_amdgcn_s_barrier();
 
-  bf16x8 fa[KK][FM], fb[KK][FN];
+  bf16x8 fa[FM], fb[FN];
   // One wave iteration.  COPY: this wave's four copies of tile kt + 3 are issued
   // between the MFMAs (steady state); otherwise the ring is draining.
   // Copy completion: a wave's copies complete in order.  At the end of its memory
@@ -510,9 +515,8 @@ __global__ void __launch_bounds__(512) gemm_bf16_pingpong_kernel(const GemmArgs 
     OB::read_all(fb, rb);
     // All 12 fragments flow through the wait, so no MFMA can move above it.
     asm volatile("s_waitcnt lgkmcnt(0)"
-                 : "+v"(fa[0][0]), "+v"(fa[0][1]), "+v"(fa[0][2]), "+v"(fa[0][3]),
-                   "+v"(fa[1][0]), "+v"(fa[1][1]), "+v"(fa[1][2]), "+v"(fa[1][3]),
-                   "+v"(fb[0][0]), "+v"(fb[0][1]), "+v"(fb[1][0]), "+v"(fb[1][1]));
+                 : "+v"(fa[0]), "+v"(fa[1]), "+v"(fa[2]), "+v"(fa[3]), "+v"(fa[4]), "+v"(fa[5]),
+                   "+v"(fa[6]), "+v"(fa[7]), "+v"(fb[0]), "+v"(fb[1]), "+v"(fb[2]), "+v"(fb[3]));
     if (COPY) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
     else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __builtin_amdgcn_sched_barrier(0);
@@ -520,24 +524,23 @@ __global__ void __launch_bounds__(512) gemm_bf16_pingpong_kernel(const GemmArgs 
     __builtin_amdgcn_sched_barrier(0);
     // ---- compute cluster -----------------------------------------------------
     char* dst = lds + (uint32_t)((kt + NSTAGE - 1) & (NSTAGE - 1)) * STAGE;
-    auto mfma4 = [&](int kk, int i0) {  // 4 MFMAs: rows i0, i0 + 1 x both column fragments
+    auto mfma8 = [&](int i0) {  // 8 MFMAs: block rows i0, i0 + 1 x the 4 block columns
 #pragma unroll
       for (int i = i0; i < i0 + 2; ++i)
 #pragma unroll
         for (int j = 0; j < FN; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[kk][j], fa[kk][i],
-                                                              acc[i][j], 0, 0, 0);
+          acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fb[j], fa[i], acc[i][j], 0, 0, 0);
     };
-    mfma4(0, 0);
+    mfma8(0);
     if (COPY) OA::template dma_one<0>(ra_rsrc, va, ka, a_is, dst, wave);
     __builtin_amdgcn_sched_barrier(0);
-    mfma4(0, 2);
+    mfma8(2);
     if (COPY) OB::template dma_one<0>(rb_rsrc, vb, kb, b_is, dst + OA::BYTES, wave);
     __builtin_amdgcn_sched_barrier(0);
-    mfma4(1, 0);
+    mfma8(4);
     if (COPY) OA::template dma_one<1>(ra_rsrc, va, ka, a_is, dst, wave);
     __builtin_amdgcn_sched_barrier(0);
-    mfma4(1, 2);
+    mfma8(6);
     if (COPY) OB::template dma_one<1>(rb_rsrc, vb, kb, b_is, dst + OA::BYTES, wave);
     __builtin_amdgcn_sched_barrier(0);
     if (COPY) {
@@ -554,7 +557,7 @@ __global__ void __launch_bounds__(512) gemm_bf16_pingpong_kernel(const GemmArgs 
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
 
-  store_tile<FM, FN, EPI, OUT_F32, false>(acc, g, lds, wave, lane, m0 + wm * WTM, n0 + wn * WTN);
+  store_tile16<FM, FN, EPI, OUT_F32>(acc, g, lds, wave, lane, m0 + wm * WTM, n0 + wn * WTN);
 }
 
 // ---------------------------------------------------------------------------
@@ -624,38 +627,6 @@ __device__ __forceinline__ void wait_all_fragments(bf16x8 (&fa)[8], bf16x8 (&fb)
                : "+v"(fa[0]), "+v"(fa[1]), "+v"(fa[2]), "+v"(fa[3]), "+v"(fa[4]), "+v"(fa[5]),
                  "+v"(fa[6]), "+v"(fa[7]), "+v"(fb[0]), "+v"(fb[1]), "+v"(fb[2]), "+v"(fb[3]),
                  "+v"(fb[4]), "+v"(fb[5]), "+v"(fb[6]), "+v"(fb[7]));
-}
-
-// Accumulators of the 16 x 16 blocks of a wave's 128 x 128 tile to C.  With the
-// operands swapped, lane l register r of acc[i][j] is the output element
-//   row = 16 i + l % 16,  col = 16 j + 4 (l / 16) + r.
-// 32 rows x 64 columns at a time go through the wave's LDS buffer, after which
-// every lane owns 8 consecutive columns of one row.
-template <int EPI, bool OUT_F32>
-__device__ __forceinline__ void store_tile16(const f32x4 (&acc)[8][8], const GemmArgs& g, char* lds,
-                                             int wave, int lane, int row0, int col0) {
-  float* E = (float*)lds + wave * (32 * EPI_LD);
-#pragma unroll
-  for (int ip = 0; ip < 4; ++ip) {
-#pragma unroll
-    for (int jp = 0; jp < 2; ++jp) {
-#pragma unroll
-      for (int ii = 0; ii < 2; ++ii)
-#pragma unroll
-        for (int jj = 0; jj < 4; ++jj)
-          *(f32x4*)&E[(ii * 16 + (lane & 15)) * EPI_LD + jj * 16 + 4 * (lane >> 4)] =
-              acc[ip * 2 + ii][jp * 4 + jj];
-#pragma unroll
-      for (int it = 0; it < 4; ++it) {
-        const int r = it * 8 + (lane >> 3);
-        const int c = (lane & 7) * 8;
-        const f32x4 v0 = *(const f32x4*)&E[r * EPI_LD + c];
-        const f32x4 v1 = *(const f32x4*)&E[r * EPI_LD + c + 4];
-        float v[8] = {v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
-        store_row8<EPI, OUT_F32>(v, g, row0 + ip * 32 + r, col0 + jp * 64 + c);
-      }
-    }
-  }
 }
 
 // 4 waves, one per SIMD, each owning 128 x 128 of the 256 x 256 tile: 8 x 8
@@ -813,7 +784,7 @@ __global__ void __launch_bounds__(256) gemm_bf16_solo_kernel(const GemmArgs g) {
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
 
-  store_tile16<EPI, OUT_F32>(acc, g, lds, wave, lane, m0 + wm * WTM, n0 + wn * WTN);
+  store_tile16<FR, FR, EPI, OUT_F32>(acc, g, lds, wave, lane, m0 + wm * WTM, n0 + wn * WTN);
 }
 
 // ---------------------------------------------------------------------------
