@@ -18,6 +18,41 @@ int hip_fail(hipError_t e, const char* what);
     if (e__ != hipSuccess) return ::axn::hip_fail(e__, #expr); \
   } while (0)
 
+// ---- exact-erf GELU -----------------------------------------------------------
+// gelu(x) = x * Phi(x), Phi(x) = (1 + erf(x / sqrt 2)) / 2, the definition behind
+// torch.nn.GELU() (approximate='none').  The library erff costs about 100 VALU
+// operations per element with both of its branches taken in a wave, which made
+// the fused epilogue as expensive as the GEMM's main loop.  Here
+//   erfc(z) = t (a1 + t (a2 + t (a3 + t (a4 + t a5)))) exp(-z^2),  t = 1 / (1 + p z),
+// Abramowitz & Stegun 7.1.26, |error| <= 1.5e-7 absolute for z >= 0; the negative
+// side uses Phi(-x) = 1 - Phi(x) without cancellation.  The same exponential
+// serves the density in the derivative.
+struct GeluTerms {
+  float cdf;   // Phi(x)
+  float expo;  // exp(-x^2 / 2)
+};
+__device__ __forceinline__ GeluTerms gelu_terms(float x) {
+  const float z = fabsf(x) * 0.70710678118654752440f;
+  const float t = __builtin_amdgcn_rcpf(fmaf(0.3275911f, z, 1.0f));
+  float p = 1.061405429f;
+  p = fmaf(p, t, -1.453152027f);
+  p = fmaf(p, t, 1.421413741f);
+  p = fmaf(p, t, -0.284496736f);
+  p = fmaf(p, t, 0.254829592f);
+  const float e = __expf(-z * z);
+  const float q = 0.5f * p * t * e;  // Phi(-|x|)
+  GeluTerms r;
+  r.cdf = x < 0.0f ? q : 1.0f - q;
+  r.expo = e;
+  return r;
+}
+__device__ __forceinline__ float gelu_exact(float x) { return x * gelu_terms(x).cdf; }
+// d/dx gelu(x) = Phi(x) + x phi(x), phi the standard normal density.
+__device__ __forceinline__ float dgelu_exact(float x) {
+  const GeluTerms g = gelu_terms(x);
+  return fmaf(x * 0.39894228040143267794f, g.expo, g.cdf);
+}
+
 // ---- bf16 GEMM ------------------------------------------------------------
 // C[M x N] (+)= A * B over a contraction of length Kc, bf16 operands, fp32
 // accumulate.  Each operand is either "K-major" (stored [rows][Kc], the

@@ -19,12 +19,6 @@ constexpr int EW_TY = 4;           // row phases per workgroup
 constexpr int EW_COLS = EW_TX * 8; // 512 columns per workgroup
 constexpr int EW_BAND = 128;       // rows per workgroup
 
-__device__ __forceinline__ float dgelu_exact(float z) {
-  const float cdf = 0.5f * (1.0f + erff(z * 0.70710678118654752440f));
-  const float pdf = 0.39894228040143267794f * __expf(-0.5f * z * z);
-  return cdf + z * pdf;
-}
-
 // 8 consecutive columns as floats, for bf16 (16 bytes) and fp32 (32 bytes) rows.
 __device__ __forceinline__ void load8(const uint16_t* p, float (&x)[8]) {
   const bf16x8 v = *(const bf16x8*)p;
@@ -93,14 +87,26 @@ __global__ void __launch_bounds__(EW_TX* EW_TY)
   }
 }
 
+// Column sums over the band partials in a fixed order: 64 columns per workgroup,
+// the bands split in 4 consecutive quarters summed by 4 threads each in band
+// order, the quarters then combined as (q0 + q1) + (q2 + q3).
 __global__ void __launch_bounds__(256)
     dbias_reduce_kernel(const float* partial, float* dbias, int64_t bands,
                         int64_t N, int beta) {
-  const int64_t c = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (c >= N) return;
+  __shared__ float red[4][64];
+  const int tx = threadIdx.x & 63, q = threadIdx.x >> 6;
+  const int64_t c = (int64_t)blockIdx.x * 64 + tx;
+  const int64_t per = (bands + 3) / 4;
+  const int64_t b0 = q * per, b1 = (b0 + per < bands) ? b0 + per : bands;
   float s = 0.f;
-  for (int64_t b = 0; b < bands; ++b) s += partial[b * N + c];
-  dbias[c] = beta ? dbias[c] + s : s;
+  if (c < N)
+    for (int64_t b = b0; b < b1; ++b) s += partial[b * N + c];
+  red[q][tx] = s;
+  __syncthreads();
+  if (q == 0 && c < N) {
+    const float t = (red[0][tx] + red[1][tx]) + (red[2][tx] + red[3][tx]);
+    dbias[c] = beta ? dbias[c] + t : t;
+  }
 }
 
 }  // namespace
@@ -148,7 +154,7 @@ int launch_dgelu_dbias(const void* dY, const void* Z, void* dZ, int dtype,
   }
   AXN_HIP_TRY(hipGetLastError());
   if (dbias != nullptr) {
-    hipLaunchKernelGGL(dbias_reduce_kernel, dim3((unsigned)((N + 255) / 256)),
+    hipLaunchKernelGGL(dbias_reduce_kernel, dim3((unsigned)((N + 63) / 64)),
                        dim3(256), 0, stream, partial, dbias, bands, N, beta);
     AXN_HIP_TRY(hipGetLastError());
   }

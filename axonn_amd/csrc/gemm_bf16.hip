@@ -71,10 +71,6 @@ __device__ __forceinline__ void static_for(F&& f) {
   static_for_impl(std::make_integer_sequence<int, N>{}, f);
 }
 
-__device__ __forceinline__ float gelu_exact(float z) {
-  return 0.5f * z * (1.0f + erff(z * 0.70710678118654752440f));
-}
-
 // Workgroup id -> output tile, XCD aware.  Consecutive workgroup ids go to
 // different XCDs, so ids are first regrouped per XCD into contiguous ranges and
 // then walked in bands of GROUP_M tile rows.
@@ -427,7 +423,7 @@ struct PingPongOperand {
 template <bool A_KMAJOR, bool B_KMAJOR, int EPI, bool OUT_F32>
 __global__ void __launch_bounds__(512) gemm_bf16_pingpong_kernel(const GemmArgs g) {
   constexpr int BM = 256, BN = 256, WTM = 128, WTN = 64, FM = 8, FN = 4;  // 16 x 16 blocks
-  constexpr int PK = 32, NSTAGE = 4;
+  constexpr int PK = 32, NSTAGE = 4;  // a ring of 5 (160 KiB) measured no better, wgrad 5 % worse
   using OA = PingPongOperand<A_KMAJOR, FM>;
   using OB = PingPongOperand<B_KMAJOR, FN>;
   constexpr int STAGE = OA::BYTES + OB::BYTES;  // 32 KiB

@@ -12,7 +12,8 @@ namespace {
 constexpr int FT = 64;   // output tile edge
 constexpr int FK = 16;   // contraction steps per stage
 
-__device__ __forceinline__ float gelu_exact(float z) {
+// Full-precision layers keep the library erff.
+__device__ __forceinline__ float gelu_erff(float z) {
   return 0.5f * z * (1.0f + erff(z * 0.70710678118654752440f));
 }
 
@@ -78,7 +79,7 @@ __global__ void __launch_bounds__(256)
       if (EPI == AXN_EPI_BIAS || EPI == AXN_EPI_BIAS_GELU) v += bias[col];
       if (EPI == AXN_EPI_BIAS_GELU || EPI == AXN_EPI_GELU) {
         if (Z != nullptr) Z[o] = v;
-        v = gelu_exact(v);
+        v = gelu_erff(v);
       }
       if (beta) v += C[o];
       C[o] = v;
