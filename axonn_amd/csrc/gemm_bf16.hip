@@ -3,43 +3,33 @@
 //   forward  Y  = X  W^T   (axonn/intra_layer/fully_connected.py:118)
 //   dgrad    dX = dY W     (fully_connected.py:140)
 //   wgrad    dW = dY^T X   (fully_connected.py:147-151)
-// templated over the operand storage orders.
+// templated over the operand storage orders: an operand is "K-major" when the
+// contraction index is contiguous in memory ([rows][Kc]) and "MN-major" when it
+// is strided ([Kc][rows]).  No transposed copy of an operand is ever made.
 //
 // Common to both kernels in this file
-//   * v_mfma_f32_32x32x16_bf16, fp32 accumulate in registers.
-//   * A workgroup owns a BM x BN output tile and walks the contraction in
-//     steps of 64 through double-buffered LDS tiles.
-//   * LDS layouts are chosen per storage order so that fragment reads are free
-//     of bank conflicts on the 64-bank LDS:
-//       K-major  tile [rows][64]   : 16-byte chunk c of row r lives at chunk
-//                                    c ^ ((r >> 1) & 7); read with ds_read_b128.
-//       MN-major tile [64][rows]   : 64-byte chunk c of contraction row k lives
-//                                    at chunk c ^ (k & 3); read with the
-//                                    transposing ds_read_b64_tr_b16, which hands
-//                                    every lane 4 consecutive contraction
-//                                    elements of one output row/column.
+//   * fp32 accumulation in registers; a workgroup owns a BM x BN output tile and
+//     walks the contraction through LDS tiles.
+//   * LDS layouts per storage order such that fragment reads are free of bank
+//     conflicts on the 64-bank LDS; MN-major tiles are read with the transposing
+//     ds_read_b64_tr_b16.
 //   * The MFMA is issued with the operands swapped (D^T = B^T A^T) so a lane
-//     ends up with 4 consecutive output columns per register quad; the
-//     epilogue transposes through LDS once more so every lane writes 16
-//     contiguous bytes and a row segment of 128 bytes is written by 8 lanes.
+//     ends up with 4 consecutive output columns; the epilogue transposes
+//     through LDS once more so every lane writes 16 contiguous bytes and a row
+//     segment of 128 bytes is written by 8 lanes.
 //   * Workgroup ids are remapped so that each of the 8 XCDs (private L2 each)
 //     works on a compact block of neighbouring tiles.
 //
-// gemm_bf16_pingpong_kernel (whole 256 x 256 tiles, contraction % 64 == 0)
-//   8 waves, two per SIMD.  Operand tiles go global -> LDS directly
-//   (global_load_lds, 16 bytes per lane, no registers, no ds_write) into a ring
-//   of four 32-deep stages.  Every wave alternates between a memory cluster
-//   (the 12 fragment reads of one stage into registers) and a compute cluster
-//   (16 MFMAs on registers, with the wave's 4 copies of a stage three ahead
-//   issued between them).  The two waves of a SIMD run one cluster apart, so
-//   the matrix pipe always has a wave whose operands are already in registers
-//   while the other one waits on LDS, and the copies of all 8 waves trickle out
-//   evenly instead of in bursts that block instruction issue.
+// gemm_bf16_solo_kernel (whole 256 x 256 tiles, contraction % 64 == 0, at least
+// 192 tiles): 4 waves, one per SIMD, 128 x 128 per wave on v_mfma_f32_16x16x32_bf16;
+// operand tiles go global -> LDS directly (buffer loads to LDS, 16 bytes per
+// lane, no registers) into a ring of five 64-deep tiles; each wave pipelines its
+// LDS fragment reads and its share of the copies between its own MFMAs.
 //
-// gemm_bf16_kernel (any shape with N % 8 == 0 and K % 8 == 0)
-//   Operand tiles are staged global -> VGPR -> LDS with bounds checks, one
-//   barrier per step; used for ragged shapes and for problems too small to fill
-//   the chip with 256 x 256 tiles.
+// gemm_bf16_kernel (any shape with N % 8 == 0 and K % 8 == 0): 128 x 128 tiles,
+// v_mfma_f32_32x32x16_bf16, operand tiles staged global -> VGPR -> LDS with
+// bounds checks, one barrier per step; used for ragged shapes and for problems
+// too small to fill the chip with 256 x 256 tiles.
 #include <utility>
 
 #include "axn_internal.h"
@@ -307,7 +297,8 @@ __device__ __forceinline__ void store_tile16(const f32x4 (&acc)[FM][FN], const G
 }
 
 // ---------------------------------------------------------------------------
-// Ping-pong kernel.
+// LDS fragment reads as inline assembly: the compiler neither waits for them nor
+// orders them behind outstanding copies; the kernels place the waits themselves.
 // ---------------------------------------------------------------------------
 template <int IMM>
 __device__ __forceinline__ bf16x8 lds_read_b128(uint32_t addr) {
@@ -322,43 +313,50 @@ __device__ __forceinline__ s16x4 lds_read_tr16_b64(uint32_t addr) {
   return v;
 }
 
-// One operand of the ping-pong kernel: a 256-row x 32-deep tile (16 KiB), copied
-// by all 8 waves (2 copies each) and read as 16-row x 32-deep MFMA fragments
-// (v_mfma_f32_16x16x32_bf16: lane l holds row l % 16, contraction elements
-// 8 (l / 16) .. + 8).  The reads are inline assembly: the compiler neither waits
-// for them nor orders them behind outstanding copies.
-//   K-major  tile [256][32]  : 64-byte rows, 16-byte chunk c of row r lives at
-//                              chunk c ^ ((r >> 2) & 3)
-//   MN-major tile [32][256]  : 512-byte rows, 64-byte chunk c of contraction row
-//                              k lives at chunk c ^ (k & 3); read with the
-//                              transposing ds_read_b64_tr_b16, two per fragment
-template <bool KMAJOR, int FR /* 16-row fragments per wave */>
-struct PingPongOperand {
+// ---------------------------------------------------------------------------
+// One-wave-per-SIMD kernel: 64-deep operand tiles, v_mfma_f32_16x16x32_bf16.
+// ---------------------------------------------------------------------------
+// Measured on MI355X, which runs these kernels power-limited: at equal FLOPs the
+// 16x16x32 MFMA sustains about 10 % more clock than 32x32x16 (half the
+// accumulator traffic per FLOP), and LDS fragment reads cost clock rather than
+// issue slots.
+//
+// One operand tile: 256 rows x 64 deep (32 KiB), copied by 4 waves (8 copies
+// each) and read as 16-row x 32-deep MFMA fragments (lane l: row l % 16,
+// contraction elements 8 (l / 16) .. + 8).
+//   K-major  tile [256][64] : 128-byte rows = whole cache lines of the operand;
+//                             16-byte chunk c of row r lives at chunk c ^ ((r >> 1) & 7),
+//                             which spreads the 16 lanes of a fragment quarter over
+//                             all 64 banks
+//   MN-major tile [64][256] : 512-byte rows; 64-byte chunk c of contraction row k
+//                             lives at chunk c ^ (k & 3); read with the transposing
+//                             ds_read_b64_tr_b16 (two per fragment)
+template <bool KMAJOR>
+struct DeepOperand {
   static constexpr int ROWS = 256;
-  static constexpr int PK = 32;                   // contraction depth of a stage
-  static constexpr int BYTES = ROWS * PK * 2;     // 16 KiB
-  static constexpr int NW = 8;                    // waves that copy
-  static constexpr int DMA_N = BYTES / 1024 / NW; // 2 copies per wave
-  static constexpr int NADDR = KMAJOR ? 1 : FR / 2;  // address registers for the reads
+  static constexpr int PK = 64;
+  static constexpr int BYTES = ROWS * PK * 2;  // 32 KiB
+  static constexpr int NW = 4;
+  static constexpr int DMA_N = BYTES / 1024 / NW;  // 8 copies per wave
+  static constexpr int FR = 8;                     // 16-row fragments of a wave's 128 rows
+  static constexpr int NADDR = KMAJOR ? 2 : 4;
+  static constexpr int READS_PER_FRAG = KMAJOR ? 1 : 2;
 
-  // Copies are buffer loads to LDS: descriptor and tile offset in SGPRs, one
-  // constant 32-bit byte offset per lane in a VGPR, no address arithmetic per
-  // copy, and accesses past the operand return zeros instead of faulting.
-  // This is the lane's byte offset for copy 0 of the tile at contraction offset
-  // 0, and the uniform byte stride from copy i to copy i + 1.  Lane l of copy i
-  // lands at tile + (8 i + wave) * 1024 + 16 l, so the LDS swizzle is applied here.
+  // Byte offset of this lane's 16 bytes for copy 0 of the tile at contraction
+  // offset 0, and the uniform stride from copy i to i + 1.  Lane l of copy i
+  // lands at tile + (4 i + wave) * 1024 + 16 l; the swizzle is applied here.
   __device__ __forceinline__ static uint32_t dma_offset(int64_t ld, int row0, int wave,
                                                         int lane, uint32_t& istride) {
     if (KMAJOR) {
-      const int row = wave * 16 + (lane >> 2);        // + 128 i
-      const int c = (lane & 3) ^ ((row >> 2) & 3);    // 128 i does not change the swizzle
-      istride = (uint32_t)(128 * ld * 2);
+      const int row = wave * 8 + (lane >> 3);          // + 32 i
+      const int c = (lane & 7) ^ ((row >> 1) & 7);     // 32 i does not change the swizzle
+      istride = (uint32_t)(32 * ld * 2);
       return (uint32_t)(((int64_t)(row0 + row) * ld + c * 8) * 2);
     } else {
-      const int k = wave * 2 + (lane >> 5);           // + 16 i
+      const int k = wave * 2 + (lane >> 5);            // + 8 i
       const int p16 = lane & 31;
-      const int c64 = (p16 >> 2) ^ (k & 3);           // 16 i does not change k & 3
-      istride = (uint32_t)(16 * ld * 2);
+      const int c64 = (p16 >> 2) ^ (k & 3);            // 8 i does not change k & 3
+      istride = (uint32_t)(8 * ld * 2);
       return (uint32_t)(((int64_t)k * ld + row0 + (c64 * 4 + (p16 & 3)) * 8) * 2);
     }
   }
@@ -372,247 +370,41 @@ struct PingPongOperand {
                                              16, (int)voff, (int)(tile_ofs + I * istride), 0, 0);
   }
 
-  // Per-lane LDS addresses (relative to the tile) the fragment reads start from.
-  //   K-major : one address; fragment i adds 16 rows = 1024 bytes (the swizzle
-  //             repeats every 16 rows).
-  //   MN-major: a[i >> 1] for fragment i, (i & 1) adds 32 bytes.  The 16 lanes of
-  //             a block address contraction rows 8 (l / 16) + (l & 15) / 4 and 4
-  //             columns each; the transposing read hands lane i of the block
-  //             column i of rows 8 (l / 16) + 0..3 (second read: rows + 4..7).
+  // Per-lane LDS byte offsets (relative to the tile) the fragment reads start from.
+  //   K-major : a[s] for the 32-deep step s; fragment i adds 16 rows = 2048 bytes
+  //             (the swizzle repeats every 16 rows)
+  //   MN-major: a[i >> 1] for fragment i, (i & 1) adds 32 bytes, step s adds 32 rows.
+  //             The 16 lanes of a block address contraction rows 8 (l / 16) + (l & 15) / 4
+  //             and 4 columns each; the transposing read hands lane i of the block
+  //             column i of rows 8 (l / 16) + 0..3 (second read: + 4..7).
   __device__ __forceinline__ static void read_bases(uint32_t (&a)[NADDR], int wrow0, int lane) {
     if (KMAJOR) {
       const int r = wrow0 + (lane & 15);
-      a[0] = (uint32_t)(r * 64 + (((lane >> 4) ^ ((r >> 2) & 3)) << 4));
+      const int swz = (r >> 1) & 7;
+#pragma unroll
+      for (int st = 0; st < 2; ++st)
+        a[st] = (uint32_t)(r * 128 + (((st * 4 + (lane >> 4)) ^ swz) << 4));
     } else {
       const int kq = (lane & 15) >> 2;
       const int k = 8 * (lane >> 4) + kq;
 #pragma unroll
-      for (int h = 0; h < NADDR; ++h) {
+      for (int h = 0; h < 4; ++h) {
         const int colbyte = (wrow0 + h * 32 + 4 * (lane & 3)) * 2;
         a[h] = (uint32_t)(k * (ROWS * 2) + ((((colbyte >> 6) ^ kq) << 6) | (colbyte & 63)));
       }
     }
   }
 
-  // All fragments of one stage: f[i] = rows 16 i .. + 16, 32 contraction elements.
-  __device__ __forceinline__ static void read_all(bf16x8 (&f)[FR], const uint32_t (&a)[NADDR]) {
-    static_for<FR>([&](auto i_) {
-      constexpr int i = decltype(i_)::value;
-      if constexpr (KMAJOR) {
-        f[i] = lds_read_b128<i * 16 * 64>(a[0]);
-      } else {
-        const s16x4 lo = lds_read_tr16_b64<(i & 1) * 32>(a[i >> 1]);
-        const s16x4 hi = lds_read_tr16_b64<4 * ROWS * 2 + (i & 1) * 32>(a[i >> 1]);
-        f[i] = __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
-      }
-    });
-  }
-};
-
-// Schedule of the ping-pong kernel.  Stages of 256 x 256 x 32 (32 KiB) form a
-// ring of 4 in LDS.  Wave iteration i handles stage-tile i:
-//   memory cluster  : read the 12 fragments of tile i into registers, wait
-//   compute cluster : 32 MFMAs (16x16x32: at equal FLOPs this part, which runs
-//                     power-limited, sustains about 10 % more clock with them than
-//                     with 32x32x16); between them this wave's 4 copies of tile i + 3
-// Group 0 (waves 0-3) runs its memory cluster in global cluster 2i and its
-// compute cluster in 2i + 1; group 1 (waves 4-7) one cluster later.  Tile i + 3
-// goes to the stage of tile i - 1, whose last reader (group 1, cluster 2i - 1)
-// finished before either group's compute cluster i starts; it is first read in
-// cluster 2i + 6, so every copy has at least three clusters to land.
-template <bool A_KMAJOR, bool B_KMAJOR, int EPI, bool OUT_F32>
-__global__ void __launch_bounds__(512) gemm_bf16_pingpong_kernel(const GemmArgs g) {
-  constexpr int BM = 256, BN = 256, WTM = 128, WTN = 64, FM = 8, FN = 4;  // 16 x 16 blocks
-  constexpr int PK = 32, NSTAGE = 4;  // a ring of 5 (160 KiB) measured no better, wgrad 5 % worse
-  using OA = PingPongOperand<A_KMAJOR, FM>;
-  using OB = PingPongOperand<B_KMAJOR, FN>;
-  constexpr int STAGE = OA::BYTES + OB::BYTES;  // 32 KiB
-  static_assert(OA::DMA_N == 2 && OB::DMA_N == 2, "copy interleave below");
-
-  extern __shared__ __attribute__((aligned(16))) char lds[];
-
-  const int tid = threadIdx.x;
-  const int lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: scalar branches
-  const int group = wave >> 2;  // 0: waves 0-3, 1: waves 4-7; one of each per SIMD
-  const int wm = group, wn = wave & 3;
-
-  int tm, tn;
-  tile_of_workgroup(blockIdx.x, g.tiles_m, g.tiles_n, tm, tn);
-  const int m0 = tm * BM, n0 = tn * BN;
-
-  f32x4 acc[FM][FN];
-#pragma unroll
-  for (int i = 0; i < FM; ++i)
-#pragma unroll
-    for (int j = 0; j < FN; ++j) acc[i][j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-
-  const int KT = g.Kc / PK;
-  // Operands as raw buffers (byte-addressed, range checked); the host side
-  // guarantees that each operand spans less than 2 GiB.
-  const uint32_t a_bytes = (uint32_t)((int64_t)(A_KMAJOR ? g.M : g.Kc) * g.lda * 2);
-  const uint32_t b_bytes = (uint32_t)((int64_t)(B_KMAJOR ? g.N : g.Kc) * g.ldb * 2);
-  const __amdgpu_buffer_rsrc_t ra_rsrc =
-      __builtin_amdgcn_make_buffer_rsrc((void*)g.A, 0, (int)a_bytes, 0x00020000);
-  const __amdgpu_buffer_rsrc_t rb_rsrc =
-      __builtin_amdgcn_make_buffer_rsrc((void*)g.B, 0, (int)b_bytes, 0x00020000);
-  uint32_t a_is, b_is;
-  const uint32_t va = OA::dma_offset(g.lda, m0, wave, lane, a_is);
-  const uint32_t vb = OB::dma_offset(g.ldb, n0, wave, lane, b_is);
-  const uint32_t a_step = (uint32_t)((A_KMAJOR ? (int64_t)PK : (int64_t)PK * g.lda) * 2);
-  const uint32_t b_step = (uint32_t)((B_KMAJOR ? (int64_t)PK : (int64_t)PK * g.ldb) * 2);
-  uint32_t ka = 0, kb = 0;  // byte offset of the next tile to copy
-
-  const uint32_t lds0 = (uint32_t)(uintptr_t)LDS_PTR(char, lds);
-  uint32_t ra0[OA::NADDR], rb0[OB::NADDR];
-  OA::read_bases(ra0, wm * WTM, lane);
-  OB::read_bases(rb0, wn * WTN, lane);
-#pragma unroll
-  for (int i = 0; i < OA::NADDR; ++i) ra0[i] += lds0;
-#pragma unroll
-  for (int i = 0; i < OB::NADDR; ++i) rb0[i] += lds0 + OA::BYTES;
-
-  // Tiles 0, 1, 2 up front; ka/kb then point at tile 3.
-#pragma unroll
-  for (int t = 0; t < NSTAGE - 1; ++t) {
-    if (t < KT) {
-      char* st = lds + t * STAGE;
-      OA::template dma_one<0>(ra_rsrc, va, ka, a_is, st, wave);
-      OA::template dma_one<1>(ra_rsrc, va, ka, a_is, st, wave);
-      OB::template dma_one<0>(rb_rsrc, vb, kb, b_is, st + OA::BYTES, wave);
-      OB::template dma_one<1>(rb_rsrc, vb, kb, b_is, st + OA::BYTES, wave);
-    }
-    ka += a_step;
-    kb += b_step;
-  }
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  __builtin_amdgcn_s_barrier();
-  // Group 1 runs one cluster behind group 0 from here on.
-  if (group == 1) __builtin_amdgcn_s_barrier();
-
-  bf16x8 fa[FM], fb[FN];
-  // One wave iteration.  COPY: this wave's four copies of tile kt + 3 are issued
-  // between the MFMAs (steady state); otherwise the ring is draining.
-  // Copy completion: a wave's copies complete in order.  At the end of its memory
-  // cluster kt a wave has at most the copies of tiles kt + 1 (issued in compute
-  // cluster kt - 2) and kt + 2 (compute cluster kt - 1) in flight; tile kt + 1 is
-  // first read (by group 0) in the cluster after group 1's memory cluster kt, so
-  // both groups wait there until only the 4 copies of tile kt + 2 are left.
-  auto iteration = [&](int kt, auto copy_) {
-    constexpr bool COPY = decltype(copy_)::value;
-    const uint32_t cur = (uint32_t)(kt & (NSTAGE - 1)) * STAGE;
-    // ---- memory cluster ------------------------------------------------------
-    uint32_t ra[OA::NADDR], rb[OB::NADDR];
-#pragma unroll
-    for (int i = 0; i < OA::NADDR; ++i) ra[i] = ra0[i] + cur;
-#pragma unroll
-    for (int i = 0; i < OB::NADDR; ++i) rb[i] = rb0[i] + cur;
-    OA::read_all(fa, ra);
-    OB::read_all(fb, rb);
-    // All 12 fragments flow through the wait, so no MFMA can move above it.
-    asm volatile("s_waitcnt lgkmcnt(0)"
-                 : "+v"(fa[0]), "+v"(fa[1]), "+v"(fa[2]), "+v"(fa[3]), "+v"(fa[4]), "+v"(fa[5]),
-                   "+v"(fa[6]), "+v"(fa[7]), "+v"(fb[0]), "+v"(fb[1]), "+v"(fb[2]), "+v"(fb[3]));
-    if (COPY) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
-    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __builtin_amdgcn_sched_barrier(0);
-    __builtin_amdgcn_s_barrier();
-    __builtin_amdgcn_sched_barrier(0);
-    // ---- compute cluster -----------------------------------------------------
-    char* dst = lds + (uint32_t)((kt + NSTAGE - 1) & (NSTAGE - 1)) * STAGE;
-    auto mfma8 = [&](int i0) {  // 8 MFMAs: block rows i0, i0 + 1 x the 4 block columns
-#pragma unroll
-      for (int i = i0; i < i0 + 2; ++i)
-#pragma unroll
-        for (int j = 0; j < FN; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fb[j], fa[i], acc[i][j], 0, 0, 0);
-    };
-    mfma8(0);
-    if (COPY) OA::template dma_one<0>(ra_rsrc, va, ka, a_is, dst, wave);
-    __builtin_amdgcn_sched_barrier(0);
-    mfma8(2);
-    if (COPY) OB::template dma_one<0>(rb_rsrc, vb, kb, b_is, dst + OA::BYTES, wave);
-    __builtin_amdgcn_sched_barrier(0);
-    mfma8(4);
-    if (COPY) OA::template dma_one<1>(ra_rsrc, va, ka, a_is, dst, wave);
-    __builtin_amdgcn_sched_barrier(0);
-    mfma8(6);
-    if (COPY) OB::template dma_one<1>(rb_rsrc, vb, kb, b_is, dst + OA::BYTES, wave);
-    __builtin_amdgcn_sched_barrier(0);
-    if (COPY) {
-      ka += a_step;
-      kb += b_step;
-    }
-    __builtin_amdgcn_s_barrier();
-    __builtin_amdgcn_sched_barrier(0);
-  };
-  const int steady = KT - (NSTAGE - 1) > 0 ? KT - (NSTAGE - 1) : 0;
-  for (int kt = 0; kt < steady; ++kt) iteration(kt, std::true_type{});
-  for (int kt = steady; kt < KT; ++kt) iteration(kt, std::false_type{});
-  if (group == 0) __builtin_amdgcn_s_barrier();  // group 1 is one barrier ahead in count
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  __syncthreads();
-
-  store_tile16<FM, FN, EPI, OUT_F32>(acc, g, lds, wave, lane, m0 + wm * WTM, n0 + wn * WTN);
-}
-
-// ---------------------------------------------------------------------------
-// One-wave-per-SIMD kernel: 64-deep operand tiles, v_mfma_f32_16x16x32_bf16.
-// ---------------------------------------------------------------------------
-// Measured on MI355X, which runs these kernels power-limited: at equal FLOPs the
-// 16x16x32 MFMA sustains about 10 % more clock than 32x32x16 (half the
-// accumulator traffic per FLOP), and LDS fragment reads cost clock rather than
-// issue slots.
-//
-// One operand tile: 256 rows x 64 deep (32 KiB), contraction-contiguous in
-// memory, copied by 4 waves (8 copies each) and read as 16-row x 32-deep MFMA
-// fragments (lane l: row l % 16, contraction elements 8 (l / 16) .. + 8).
-// Tile layout [256][64]: 128-byte rows = whole cache lines of the operand;
-// 16-byte chunk c of row r lives at chunk c ^ ((r >> 1) & 7), which spreads the
-// 16 lanes of a fragment quarter over all 64 banks.
-struct DeepOperand {
-  static constexpr int ROWS = 256;
-  static constexpr int PK = 64;
-  static constexpr int BYTES = ROWS * PK * 2;  // 32 KiB
-  static constexpr int NW = 4;
-  static constexpr int DMA_N = BYTES / 1024 / NW;  // 8 copies per wave
-  static constexpr int NADDR = 2;
-
-  // Byte offset of this lane's 16 bytes for copy 0 of the tile at contraction
-  // offset 0, and the uniform stride from copy i to i + 1.  Lane l of copy i
-  // lands at tile + (4 i + wave) * 1024 + 16 l; the swizzle is applied here.
-  __device__ __forceinline__ static uint32_t dma_offset(int64_t ld, int row0, int wave,
-                                                        int lane, uint32_t& istride) {
-    const int row = wave * 8 + (lane >> 3);          // + 32 i
-    const int c = (lane & 7) ^ ((row >> 1) & 7);     // 32 i does not change the swizzle
-    istride = (uint32_t)(32 * ld * 2);
-    return (uint32_t)(((int64_t)(row0 + row) * ld + c * 8) * 2);
-  }
-
-  template <int I>
-  __device__ __forceinline__ static void dma_one(__amdgpu_buffer_rsrc_t rsrc, uint32_t voff,
-                                                 uint32_t tile_ofs, uint32_t istride,
-                                                 char* lds_tile, int wave) {
-    static_assert(I >= 0 && I < DMA_N, "copy index");
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, LDS_PTR(void, lds_tile + (NW * I + wave) * 1024),
-                                             16, (int)voff, (int)(tile_ofs + I * istride), 0, 0);
-  }
-
-  // Per-lane LDS byte offsets (relative to the tile) the fragment reads start
-  // from: a[s] for the 32-deep step s; fragment i adds 16 rows = 2048 bytes (the
-  // swizzle repeats every 16 rows).
-  __device__ __forceinline__ static void read_bases(uint32_t (&a)[NADDR], int wrow0, int lane) {
-    const int r = wrow0 + (lane & 15);
-    const int swz = (r >> 1) & 7;
-#pragma unroll
-    for (int st = 0; st < 2; ++st)
-      a[st] = (uint32_t)(r * 128 + (((st * 4 + (lane >> 4)) ^ swz) << 4));
-  }
-
   // Fragment I (rows 16 I ..) of the 32-deep step ST of the tile.
   template <int ST, int I>
   __device__ __forceinline__ static void read_frag(bf16x8& f, const uint32_t (&a)[NADDR]) {
-    f = lds_read_b128<I * 16 * 128>(a[ST]);
+    if constexpr (KMAJOR) {
+      f = lds_read_b128<I * 16 * 128>(a[ST]);
+    } else {
+      const s16x4 lo = lds_read_tr16_b64<ST * 32 * ROWS * 2 + (I & 1) * 32>(a[I >> 1]);
+      const s16x4 hi = lds_read_tr16_b64<(ST * 32 + 4) * ROWS * 2 + (I & 1) * 32>(a[I >> 1]);
+      f = __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+    }
   }
 };
 
@@ -639,13 +431,12 @@ __device__ __forceinline__ void wait_all_fragments(bf16x8 (&fa)[8], bf16x8 (&fb)
 // At the barrier every wave holds the last fragments of stage p in registers, so
 // both of its slots are free: B(p+2) takes A(p)'s, A(p+3) (next step 0) B(p)'s.
 // A tile has at least two steps (128 MFMAs per wave) to land.
-template <int EPI, bool OUT_F32>
+template <bool A_KMAJOR, bool B_KMAJOR, int EPI, bool OUT_F32>
 __global__ void __launch_bounds__(256) gemm_bf16_solo_kernel(const GemmArgs g) {
   constexpr int BM = 256, BN = 256, WTM = 128, WTN = 128, FR = 8;
   constexpr int PK = 64, NSLOT = 5;
-  constexpr bool A_KMAJOR = true, B_KMAJOR = true;  // both operands contraction-contiguous
-  using OA = DeepOperand;
-  using OB = DeepOperand;
+  using OA = DeepOperand<A_KMAJOR>;
+  using OB = DeepOperand<B_KMAJOR>;
   constexpr uint32_t SLOT = OA::BYTES;  // 32 KiB
   static_assert(OA::DMA_N == 8 && OB::DMA_N == 8 && OA::BYTES == OB::BYTES, "copy schedule below");
 
@@ -754,7 +545,14 @@ __global__ void __launch_bounds__(256) gemm_bf16_solo_kernel(const GemmArgs g) {
       static_for<64>([&](auto m_) {
         constexpr int m = decltype(m_)::value;
         constexpr int i = m / FR, j = m % FR;
-        acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fb[j], fa[i], acc[i][j], 0, 0, 0);
+        // Inline assembly pins the register classes (accumulators in AGPRs, fragments
+        // in VGPRs): with the builtin the allocator moves two-instruction
+        // (transposed) fragments through AGPRs and spills.  No MFMA hazard can arise:
+        // fragments come from LDS behind s_waitcnt, and an accumulator is touched
+        // again only 63 MFMAs later.
+        asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0"
+                     : "+a"(acc[i][j])
+                     : "v"(fb[j]), "v"(fa[i]));
         if constexpr (m < 32 && m % 2 == 0) {
           if constexpr (ST == 0) read(std::integral_constant<int, 1>{},
                                       std::integral_constant<int, m / 2>{}, sa, sb);
@@ -777,6 +575,8 @@ __global__ void __launch_bounds__(256) gemm_bf16_solo_kernel(const GemmArgs g) {
   for (int p = 0; p < KP - 2; ++p) stage(T{}, F{});
   if (KP > 1) stage(F{}, F{});
   stage(F{}, T{});
+  // the last MFMAs have left the pipeline before the accumulators are read
+  asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
 
@@ -898,26 +698,12 @@ int launch_cfg(const GemmArgs& in, hipStream_t stream) {
 }
 
 template <bool AK, bool BKM, int EPI, bool OUT_F32>
-int launch_pingpong(const GemmArgs& in, hipStream_t stream) {
-  GemmArgs g = in;
-  g.tiles_m = g.M / 256;
-  g.tiles_n = g.N / 256;
-  constexpr size_t lds = 4 * 2 * 256 * 32 * 2;  // ring of 4 stages, 128 KiB
-  auto kern = gemm_bf16_pingpong_kernel<AK, BKM, EPI, OUT_F32>;
-  AXN_HIP_TRY(hipFuncSetAttribute((const void*)kern,
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-  hipLaunchKernelGGL(kern, dim3((unsigned)(g.tiles_m * g.tiles_n)), dim3(512), lds, stream, g);
-  AXN_HIP_TRY(hipGetLastError());
-  return AXN_OK;
-}
-
-template <int EPI, bool OUT_F32>
 int launch_solo(const GemmArgs& in, hipStream_t stream) {
   GemmArgs g = in;
   g.tiles_m = g.M / 256;
   g.tiles_n = g.N / 256;
   constexpr size_t lds = 5 * 256 * 64 * 2;  // ring of 5 operand tiles, 160 KiB: all of a CU's LDS
-  auto kern = gemm_bf16_solo_kernel<EPI, OUT_F32>;
+  auto kern = gemm_bf16_solo_kernel<AK, BKM, EPI, OUT_F32>;
   AXN_HIP_TRY(hipFuncSetAttribute((const void*)kern,
                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
   hipLaunchKernelGGL(kern, dim3((unsigned)(g.tiles_m * g.tiles_n)), dim3(256), lds, stream, g);
@@ -926,21 +712,19 @@ int launch_solo(const GemmArgs& in, hipStream_t stream) {
 }
 
 // Kernel selection.  Large problems made of whole 256 x 256 tiles take the
-// one-wave-per-SIMD kernel when both operands are contraction-contiguous (the
-// forward GEMM) and the ping-pong kernel otherwise; problems that would leave
-// most of the 256 CUs idle at that tile size, and ragged ones, take 128 x 128
-// tiles on the register-staged kernel.
+// one-wave-per-SIMD kernel; problems that would leave most of the 256 CUs idle
+// at that tile size, and ragged ones, take 128 x 128 tiles on the
+// register-staged kernel.
 template <bool AK, bool BKM, int EPI, bool OUT_F32>
 int launch_shape(const GemmArgs& g, hipStream_t stream) {
   const bool whole256 = (g.M % 256 == 0) && (g.N % 256 == 0) && (g.Kc % BK == 0);
   const long long tiles256 = (long long)((g.M + 255) / 256) * ((g.N + 255) / 256);
-  // The ping-pong kernel addresses its operands with 32-bit byte offsets.
+  // The one-wave-per-SIMD kernel addresses its operands with 32-bit byte offsets.
   const int64_t a_span = (int64_t)(AK ? g.M : g.Kc) * g.lda * 2;
   const int64_t b_span = (int64_t)(BKM ? g.N : g.Kc) * g.ldb * 2;
   const bool small_spans = a_span < (1LL << 31) && b_span < (1LL << 31);
   if (whole256 && tiles256 >= 192 && small_spans) {
-    if constexpr (AK && BKM) return launch_solo<EPI, OUT_F32>(g, stream);
-    else return launch_pingpong<AK, BKM, EPI, OUT_F32>(g, stream);
+    return launch_solo<AK, BKM, EPI, OUT_F32>(g, stream);
   }
   const bool whole128 = (g.M % 128 == 0) && (g.N % 128 == 0) && (g.Kc % BK == 0);
   if (whole128) return launch_cfg<128, 128, 2, 2, AK, BKM, EPI, OUT_F32, false>(g, stream);

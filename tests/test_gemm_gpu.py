@@ -182,12 +182,13 @@ def test_fp32_gemms_match_oracle(M, N, K):
     assert rel(dw.cpu().numpy(), 2 * bw["dw"].reshape(N, K)) < F32_TOL
 
 
-# ---- the 256 x 256 ping-pong kernel: few and many k-stages, all layouts/epilogues --------
+# ---- the 256 x 256-tile kernel: few and many contraction stages, all layouts/epilogues ----
 @pytest.mark.parametrize("K", [64, 128, 192, 256, 448])
-def test_pingpong_kernel_short_contractions(K):
-    """Shapes of >= 192 whole 256 x 256 tiles take the ping-pong kernel; its LDS
-    ring holds 4 stages of 32, so K = 64 .. 192 exercise the start-up and
-    drain paths (fewer stages than the ring) and 448 the steady state."""
+def test_tile256_kernel_short_contractions(K):
+    """Shapes of >= 192 whole 256 x 256 tiles take the one-wave-per-SIMD kernel; it
+    walks the contraction in stages of 64 and copies two stages ahead, so K = 64 and
+    128 exercise the start-up and drain paths alone (1 and 2 stages), 192 and 256 a
+    single or two steady-state stages, and 448 the steady state proper."""
     from axonn_amd import ops
 
     M, N = 4096, 3072
@@ -206,9 +207,9 @@ def test_pingpong_kernel_short_contractions(K):
 
 
 @pytest.mark.parametrize("Kc", [64, 192, 320])
-def test_pingpong_kernel_backward_layouts(Kc):
+def test_tile256_kernel_backward_layouts(Kc):
     """dgrad (B operand contraction-strided) and wgrad (both operands
-    contraction-strided, bf16 and fp32 accumulate) on the ping-pong kernel."""
+    contraction-strided, bf16 and fp32 accumulate) on the 256 x 256-tile kernel."""
     from axonn_amd import ops
 
     g = torch.Generator(device="cuda").manual_seed(Kc + 1)
