@@ -351,6 +351,20 @@ def bench_adam(args, torch, nv, lib, stream, time_loop):
     }
     del P, G, M, V, PL, ws
     torch.cuda.empty_cache()
+    # What plain streams reach on this box, for scale: the runtime's device-to-device
+    # copy and a torch elementwise kernel (both 1 read : 1 write, like the update) and a
+    # fill (writes only), 4 GiB each.
+    a = torch.empty(1 << 30, dtype=torch.float32, device="cuda").normal_()
+    b = torch.empty_like(a)
+    nb = a.numel() * 4.0
+    out["hbm_reference_streams"] = {
+        "copy_gbs": round(2 * nb / time_loop(lambda: b.copy_(a), 5, 2) / 1e9, 1),
+        "elementwise_1r1w_gbs": round(2 * nb / time_loop(lambda: torch.mul(a, 2.0, out=b), 5, 2) / 1e9, 1),
+        "fill_gbs": round(nb / time_loop(lambda: b.fill_(1.0), 5, 2) / 1e9, 1),
+        "unit": "GB/s",
+    }
+    del a, b
+    torch.cuda.empty_cache()
     return out
 
 

@@ -102,6 +102,43 @@ def test_dgelu_dbias_matches_oracle():
     assert rel(dz32.cpu().numpy(), want) < 1e-6 and rel(db32.cpu().numpy(), want.sum(0)) < 1e-5
 
 
+def test_gelu_and_its_derivative_elementwise_over_the_tails():
+    """The kernels evaluate erf by a 5-term rational formula (|error| <= 1.5e-7);
+    checked element by element from -12 to 12, not just in norm: the derivative in
+    fp32 against the oracle's math.erf, the fused forward epilogue (identity weight,
+    so Z = X exactly) to one bf16 rounding of the oracle's value."""
+    from axonn_amd import ops
+
+    n = 256 * 256
+    z32 = torch.linspace(-12.0, 12.0, n).reshape(256, 256)
+    dz, _ = ops.dgelu_dbias(torch.ones_like(z32).cuda(), z32.cuda(), want_dbias=False)
+    want = ol.dgelu(z32.double().numpy())
+    assert np.max(np.abs(dz.cpu().numpy().astype(np.float64) - want)) < 1e-6
+    x = z32.bfloat16()
+    eye = torch.eye(256).bfloat16()
+    y, z = ops.gemm_fwd(x.cuda(), eye.cuda(), activation="gelu", save_z=True)
+    assert torch.equal(z.cpu(), x)
+    exact = ol.gelu(np64(x))
+    got = np64(y)
+    ulp = np.maximum(np.abs(exact), 2.0 ** -126) * 2.0 ** -8   # half a bf16 ulp is 2^-9 relative
+    assert np.all(np.abs(got - exact) <= ulp + 5e-7)
+
+
+def test_dbias_reduction_with_few_bands_and_ragged_columns():
+    """Column sums over 1, 3 and 9 row bands of 128 (the reduction splits the
+    bands over 4 threads) and a column count that is not a multiple of 64."""
+    from axonn_amd import ops
+
+    g = torch.Generator().manual_seed(11)
+    for M in (5, 300, 1100):
+        dY = torch.randn(M, 72, generator=g).bfloat16()
+        _, db = ops.dgelu_dbias(dY.cuda(), None, want_dbias=True)
+        assert rel(db.cpu().numpy(), np64(dY).sum(0)) < 1e-6
+        acc = torch.ones(72, device="cuda")
+        ops.dgelu_dbias(dY.cuda(), None, want_dbias=True, dbias_out=acc, accumulate=True)
+        assert rel(acc.cpu().numpy(), 1.0 + np64(dY).sum(0)) < 1e-6
+
+
 def test_wgrad_accumulates_over_micro_batches():
     """dW += dY^T X over 4 micro-batches equals the weight gradient of the
     concatenated batch (overlap_communication.py:38-47 semantics, in fp32 and in
