@@ -263,39 +263,6 @@ __device__ __forceinline__ void store_tile(const f32x16 (&acc)[FM][FN], const Ge
   }
 }
 
-// Same for accumulators of v_mfma_f32_16x16x32_bf16: FM x FN blocks of 16 x 16.
-// With the operands swapped, lane l register r of acc[i][j] is the output element
-//   row = 16 i + l % 16,  col = 16 j + 4 (l / 16) + r.
-// 32 rows x 64 columns at a time go through the wave's LDS buffer, after which
-// every lane owns 8 consecutive columns of one row.
-template <int FM, int FN, int EPI, bool OUT_F32>
-__device__ __forceinline__ void store_tile16(const f32x4 (&acc)[FM][FN], const GemmArgs& g,
-                                             char* lds, int wave, int lane, int row0, int col0) {
-  static_assert(FM % 2 == 0 && FN % 4 == 0, "staged in blocks of 32 x 64");
-  float* E = (float*)lds + wave * (32 * EPI_LD);
-#pragma unroll
-  for (int ip = 0; ip < FM / 2; ++ip) {
-#pragma unroll
-    for (int jp = 0; jp < FN / 4; ++jp) {
-#pragma unroll
-      for (int ii = 0; ii < 2; ++ii)
-#pragma unroll
-        for (int jj = 0; jj < 4; ++jj)
-          *(f32x4*)&E[(ii * 16 + (lane & 15)) * EPI_LD + jj * 16 + 4 * (lane >> 4)] =
-              acc[ip * 2 + ii][jp * 4 + jj];
-#pragma unroll
-      for (int it = 0; it < 4; ++it) {
-        const int r = it * 8 + (lane >> 3);
-        const int c = (lane & 7) * 8;
-        const f32x4 v0 = *(const f32x4*)&E[r * EPI_LD + c];
-        const f32x4 v1 = *(const f32x4*)&E[r * EPI_LD + c + 4];
-        float v[8] = {v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
-        store_row8<EPI, OUT_F32>(v, g, row0 + ip * 32 + r, col0 + jp * 64 + c);
-      }
-    }
-  }
-}
-
 // ---------------------------------------------------------------------------
 // LDS fragment reads as inline assembly: the compiler neither waits for them nor
 // orders them behind outstanding copies; the kernels place the waits themselves.
@@ -331,16 +298,27 @@ __device__ __forceinline__ s16x4 lds_read_tr16_b64(uint32_t addr) {
 //   MN-major tile [64][256] : 512-byte rows; 64-byte chunk c of contraction row k
 //                             lives at chunk c ^ (k & 3); read with the transposing
 //                             ds_read_b64_tr_b16 (two per fragment)
-template <bool KMAJOR>
+//
+// PERMUTED (the operand that supplies the output columns): fragment j holds the
+// tile rows 32 (j / 2) + 8 (q / 4) + 4 (j % 2) + q % 4 in its lane-rows
+// q = 0..15 instead of 16 j + q.  The MFMA result then leaves lane l with
+// columns 8 (l / 16) .. + 3 of a 32-column group in block 2t and .. + 4 .. + 7
+// in block 2t + 1: eight consecutive output columns per lane, stored from
+// registers without a transpose through LDS.  Its K-major swizzle is
+// chunk ^ (((r >> 1) & 1) | ((r >> 3) & 3) << 1), which again gives the 16 rows
+// of a fragment quarter 16 distinct (row parity, chunk) pairs.
+template <bool KMAJOR, bool PERMUTED>
 struct DeepOperand {
   static constexpr int ROWS = 256;
   static constexpr int PK = 64;
   static constexpr int BYTES = ROWS * PK * 2;  // 32 KiB
   static constexpr int NW = 4;
   static constexpr int DMA_N = BYTES / 1024 / NW;  // 8 copies per wave
-  static constexpr int FR = 8;                     // 16-row fragments of a wave's 128 rows
   static constexpr int NADDR = KMAJOR ? 2 : 4;
-  static constexpr int READS_PER_FRAG = KMAJOR ? 1 : 2;
+
+  __device__ __forceinline__ static int kmajor_swizzle(int row) {
+    return PERMUTED ? (((row >> 1) & 1) | (((row >> 3) & 3) << 1)) : ((row >> 1) & 7);
+  }
 
   // Byte offset of this lane's 16 bytes for copy 0 of the tile at contraction
   // offset 0, and the uniform stride from copy i to i + 1.  Lane l of copy i
@@ -348,8 +326,8 @@ struct DeepOperand {
   __device__ __forceinline__ static uint32_t dma_offset(int64_t ld, int row0, int wave,
                                                         int lane, uint32_t& istride) {
     if (KMAJOR) {
-      const int row = wave * 8 + (lane >> 3);          // + 32 i
-      const int c = (lane & 7) ^ ((row >> 1) & 7);     // 32 i does not change the swizzle
+      const int row = wave * 8 + (lane >> 3);              // + 32 i
+      const int c = (lane & 7) ^ kmajor_swizzle(row);      // 32 i does not change the swizzle
       istride = (uint32_t)(32 * ld * 2);
       return (uint32_t)(((int64_t)(row0 + row) * ld + c * 8) * 2);
     } else {
@@ -371,38 +349,42 @@ struct DeepOperand {
   }
 
   // Per-lane LDS byte offsets (relative to the tile) the fragment reads start from.
-  //   K-major : a[s] for the 32-deep step s; fragment i adds 16 rows = 2048 bytes
-  //             (the swizzle repeats every 16 rows)
-  //   MN-major: a[i >> 1] for fragment i, (i & 1) adds 32 bytes, step s adds 32 rows.
-  //             The 16 lanes of a block address contraction rows 8 (l / 16) + (l & 15) / 4
-  //             and 4 columns each; the transposing read hands lane i of the block
-  //             column i of rows 8 (l / 16) + 0..3 (second read: + 4..7).
+  //   K-major : a[s] for the 32-deep step s; fragments add whole rows (frag_offset),
+  //             which leave the swizzle unchanged.
+  //   MN-major: a[i >> 1] for fragment i, step s adds 32 rows.  The 16 lanes of a
+  //             block address contraction rows 8 (l / 16) + (l & 15) / 4 and 4
+  //             columns each; the transposing read hands lane i of the block the
+  //             column that lane 4 (i / 4) .. addressed, rows 8 (l / 16) + 0..3
+  //             (second read: + 4..7).
   __device__ __forceinline__ static void read_bases(uint32_t (&a)[NADDR], int wrow0, int lane) {
+    const int q = lane & 15;
     if (KMAJOR) {
-      const int r = wrow0 + (lane & 15);
-      const int swz = (r >> 1) & 7;
+      const int r = wrow0 + (PERMUTED ? 8 * (q >> 2) + (q & 3) : q);
+      const int swz = kmajor_swizzle(r);
 #pragma unroll
       for (int st = 0; st < 2; ++st)
         a[st] = (uint32_t)(r * 128 + (((st * 4 + (lane >> 4)) ^ swz) << 4));
     } else {
-      const int kq = (lane & 15) >> 2;
+      const int kq = q >> 2;
       const int k = 8 * (lane >> 4) + kq;
 #pragma unroll
       for (int h = 0; h < 4; ++h) {
-        const int colbyte = (wrow0 + h * 32 + 4 * (lane & 3)) * 2;
+        const int colbyte = (wrow0 + h * 32 + (PERMUTED ? 8 : 4) * (lane & 3)) * 2;
         a[h] = (uint32_t)(k * (ROWS * 2) + ((((colbyte >> 6) ^ kq) << 6) | (colbyte & 63)));
       }
     }
   }
 
-  // Fragment I (rows 16 I ..) of the 32-deep step ST of the tile.
+  // Fragment I of the 32-deep step ST of the tile.
   template <int ST, int I>
   __device__ __forceinline__ static void read_frag(bf16x8& f, const uint32_t (&a)[NADDR]) {
     if constexpr (KMAJOR) {
-      f = lds_read_b128<I * 16 * 128>(a[ST]);
+      constexpr int row_ofs = PERMUTED ? 32 * (I >> 1) + 4 * (I & 1) : 16 * I;
+      f = lds_read_b128<row_ofs * 128>(a[ST]);
     } else {
-      const s16x4 lo = lds_read_tr16_b64<ST * 32 * ROWS * 2 + (I & 1) * 32>(a[I >> 1]);
-      const s16x4 hi = lds_read_tr16_b64<(ST * 32 + 4) * ROWS * 2 + (I & 1) * 32>(a[I >> 1]);
+      constexpr int col_ofs = PERMUTED ? 4 * (I & 1) : 16 * (I & 1);  // elements
+      const s16x4 lo = lds_read_tr16_b64<ST * 32 * ROWS * 2 + col_ofs * 2>(a[I >> 1]);
+      const s16x4 hi = lds_read_tr16_b64<(ST * 32 + 4) * ROWS * 2 + col_ofs * 2>(a[I >> 1]);
       f = __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
     }
   }
@@ -435,8 +417,8 @@ template <bool A_KMAJOR, bool B_KMAJOR, int EPI, bool OUT_F32>
 __global__ void __launch_bounds__(256) gemm_bf16_solo_kernel(const GemmArgs g) {
   constexpr int BM = 256, BN = 256, WTM = 128, WTN = 128, FR = 8;
   constexpr int PK = 64, NSLOT = 5;
-  using OA = DeepOperand<A_KMAJOR>;
-  using OB = DeepOperand<B_KMAJOR>;
+  using OA = DeepOperand<A_KMAJOR, false>;
+  using OB = DeepOperand<B_KMAJOR, true>;
   constexpr uint32_t SLOT = OA::BYTES;  // 32 KiB
   static_assert(OA::DMA_N == 8 && OB::DMA_N == 8 && OA::BYTES == OB::BYTES, "copy schedule below");
 
@@ -577,10 +559,20 @@ __global__ void __launch_bounds__(256) gemm_bf16_solo_kernel(const GemmArgs g) {
   stage(F{}, T{});
   // the last MFMAs have left the pipeline before the accumulators are read
   asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  __syncthreads();
-
-  store_tile16<FR, FR, EPI, OUT_F32>(acc, g, lds, wave, lane, m0 + wm * WTM, n0 + wn * WTN);
+  // With the permuted column fragments a lane owns, per block row i and block
+  // pair t, the 8 consecutive columns 32 t + 8 (l / 16) .. + 7 of row 16 i + l % 16:
+  // they go out straight from the registers, 64 contiguous bytes per row and
+  // instruction.
+  const int orow = m0 + wm * WTM + (lane & 15);
+  const int ocol = n0 + wn * WTN + 8 * (lane >> 4);
+#pragma unroll
+  for (int i = 0; i < FR; ++i)
+#pragma unroll
+    for (int t = 0; t < FR / 2; ++t) {
+      const f32x4 lo = acc[i][2 * t], hi = acc[i][2 * t + 1];
+      float v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+      store_row8<EPI, OUT_F32>(v, g, orow + 16 * i, ocol + 32 * t);
+    }
 }
 
 // ---------------------------------------------------------------------------
