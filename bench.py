@@ -61,6 +61,8 @@ def parse():
     ap.add_argument("--no-adam", action="store_true")
     ap.add_argument("--no-extra-shapes", action="store_true")
     ap.add_argument("--adam-elements", type=float, default=1.3e9)
+    ap.add_argument("--no-launch-events", action="store_true",
+                    help="do not bracket every launch with events (no per-kernel figures)")
     return ap.parse_args()
 
 
@@ -129,15 +131,24 @@ def main():
         return torch.cuda.Event(enable_timing=True)
 
     spans = {"fwd": [], "dgrad": [], "wgrad": []}  # (start, end, flops) per launch
+    # One event between consecutive launches: launch j of a step runs between events j
+    # and j + 1, so a span is the kernel plus the gap to the next launch (3-5 us).  Half
+    # the event traffic of a start/stop pair per launch, which cost 2.5 % of the step.
+    chain = {"last": None}
 
     def timed(kind, fn, L):
-        s, e = ev(), ev()
-        s.record()
+        if chain["last"] is None:
+            chain["last"] = ev()
+            chain["last"].record()
         fn(L)
+        e = ev()
         e.record()
-        spans[kind].append((s, e, L.flops / 3.0))
+        spans[kind].append((chain["last"], e, L.flops / 3.0))
+        chain["last"] = e
 
     def step(record):
+        record = record and not args.no_launch_events
+        chain["last"] = None
         for L in layers:
             timed("fwd", fwd, L) if record else fwd(L)
         for L in reversed(layers):
@@ -155,30 +166,32 @@ def main():
     ms_per_step = elapsed / args.steps * 1e3
     value = total_flops / (elapsed / args.steps) / 1e12
 
-    kinds = {}
-    for kind, lst in spans.items():
-        tot_ms = sum(s.elapsed_time(e) for s, e, _ in lst)
-        tot_fl = sum(f for _, _, f in lst)
-        kinds[kind] = {
-            "launches": len(lst), "avg_us": tot_ms / len(lst) * 1e3,
-            "tflops": tot_fl / (tot_ms * 1e-3) / 1e12, "total_ms": tot_ms,
+    roofline = None
+    if not args.no_launch_events:
+        kinds = {}
+        for kind, lst in spans.items():
+            tot_ms = sum(s.elapsed_time(e) for s, e, _ in lst)
+            tot_fl = sum(f for _, _, f in lst)
+            kinds[kind] = {
+                "launches": len(lst), "avg_us": tot_ms / len(lst) * 1e3,
+                "tflops": tot_fl / (tot_ms * 1e-3) / 1e12, "total_ms": tot_ms,
+            }
+        dom = max(kinds, key=lambda k: kinds[k]["total_ms"])
+        # template arguments: <A contraction-contiguous, B contraction-contiguous, epilogue, fp32 out>
+        kernel_names = {"fwd": "gemm_bf16_solo_kernel<true, true, 0, false> (Y = X W^T)",
+                        "dgrad": "gemm_bf16_solo_kernel<true, false, 0, false> (dX = dY W)",
+                        "wgrad": "gemm_bf16_solo_kernel<false, false, 0, false> (dW = dY^T X)"}
+        roofline = {
+            "bound": "mfma", "kernel": kernel_names[dom],
+            "achieved": round(kinds[dom]["tflops"], 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+            "frac": round(kinds[dom]["tflops"] / PEAK_BF16_TFLOPS, 4),
+            "avg_launch_us": round(kinds[dom]["avg_us"], 1),
+            "flops_per_launch": kinds[dom]["tflops"] * 1e12 * kinds[dom]["avg_us"] * 1e-6,
+            "traffic": TRAFFIC_BYTES_PER_LAUNCH.get(dom),
+            "per_kernel": {k: {"avg_us": round(v["avg_us"], 1), "tflops": round(v["tflops"], 1),
+                               "frac": round(v["tflops"] / PEAK_BF16_TFLOPS, 4)}
+                           for k, v in kinds.items()},
         }
-    dom = max(kinds, key=lambda k: kinds[k]["total_ms"])
-    # template arguments: <A contraction-contiguous, B contraction-contiguous, epilogue, fp32 out>
-    kernel_names = {"fwd": "gemm_bf16_solo_kernel<true, true, 0, false> (Y = X W^T)",
-                    "dgrad": "gemm_bf16_solo_kernel<true, false, 0, false> (dX = dY W)",
-                    "wgrad": "gemm_bf16_solo_kernel<false, false, 0, false> (dW = dY^T X)"}
-    roofline = {
-        "bound": "mfma", "kernel": kernel_names[dom],
-        "achieved": round(kinds[dom]["tflops"], 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-        "frac": round(kinds[dom]["tflops"] / PEAK_BF16_TFLOPS, 4),
-        "avg_launch_us": round(kinds[dom]["avg_us"], 1),
-        "flops_per_launch": kinds[dom]["tflops"] * 1e12 * kinds[dom]["avg_us"] * 1e-6,
-        "traffic": TRAFFIC_BYTES_PER_LAUNCH.get(dom),
-        "per_kernel": {k: {"avg_us": round(v["avg_us"], 1), "tflops": round(v["tflops"], 1),
-                           "frac": round(v["tflops"] / PEAK_BF16_TFLOPS, 4)}
-                       for k, v in kinds.items()},
-    }
     del layers
     torch.cuda.empty_cache()
 
