@@ -307,14 +307,16 @@ __device__ __forceinline__ s16x4 lds_read_tr16_b64(uint32_t addr) {
 // registers without a transpose through LDS.  Its K-major swizzle is
 // chunk ^ (((r >> 1) & 1) | ((r >> 3) & 3) << 1), which again gives the 16 rows
 // of a fragment quarter 16 distinct (row parity, chunk) pairs.
-template <bool KMAJOR, bool PERMUTED>
+template <bool KMAJOR, bool PERMUTED, int ROWS_ /* 256 or 128 */>
 struct DeepOperand {
-  static constexpr int ROWS = 256;
+  static constexpr int ROWS = ROWS_;
   static constexpr int PK = 64;
-  static constexpr int BYTES = ROWS * PK * 2;  // 32 KiB
+  static constexpr int BYTES = ROWS * PK * 2;      // 32 or 16 KiB
   static constexpr int NW = 4;
-  static constexpr int DMA_N = BYTES / 1024 / NW;  // 8 copies per wave
-  static constexpr int NADDR = KMAJOR ? 2 : 4;
+  static constexpr int DMA_N = BYTES / 1024 / NW;  // 8 or 4 copies per wave
+  static constexpr int FR = ROWS / 32;             // 16-row fragments of a wave's half of the rows
+  static constexpr int NADDR = KMAJOR ? 2 : FR / 2;
+  static constexpr int LPR = ROWS / 8;             // MN-major: lanes per contraction row of a copy
 
   __device__ __forceinline__ static int kmajor_swizzle(int row) {
     return PERMUTED ? (((row >> 1) & 1) | (((row >> 3) & 3) << 1)) : ((row >> 1) & 7);
@@ -331,10 +333,11 @@ struct DeepOperand {
       istride = (uint32_t)(32 * ld * 2);
       return (uint32_t)(((int64_t)(row0 + row) * ld + c * 8) * 2);
     } else {
-      const int k = wave * 2 + (lane >> 5);            // + 8 i
-      const int p16 = lane & 31;
-      const int c64 = (p16 >> 2) ^ (k & 3);            // 8 i does not change k & 3
-      istride = (uint32_t)(8 * ld * 2);
+      constexpr int KPI = 64 / LPR;                    // contraction rows per copy: 2 or 4
+      const int k = wave * KPI + lane / LPR;           // + 4 KPI i
+      const int p16 = lane % LPR;
+      const int c64 = (p16 >> 2) ^ (k & 3);            // 4 KPI i does not change k & 3
+      istride = (uint32_t)(4 * KPI * ld * 2);
       return (uint32_t)(((int64_t)k * ld + row0 + (c64 * 4 + (p16 & 3)) * 8) * 2);
     }
   }
@@ -368,7 +371,7 @@ struct DeepOperand {
       const int kq = q >> 2;
       const int k = 8 * (lane >> 4) + kq;
 #pragma unroll
-      for (int h = 0; h < 4; ++h) {
+      for (int h = 0; h < NADDR; ++h) {
         const int colbyte = (wrow0 + h * 32 + (PERMUTED ? 8 : 4) * (lane & 3)) * 2;
         a[h] = (uint32_t)(k * (ROWS * 2) + ((((colbyte >> 6) ^ kq) << 6) | (colbyte & 63)));
       }
@@ -398,12 +401,30 @@ __device__ __forceinline__ void wait_all_fragments(bf16x8 (&fa)[8], bf16x8 (&fb)
                  "+v"(fa[6]), "+v"(fa[7]), "+v"(fb[0]), "+v"(fb[1]), "+v"(fb[2]), "+v"(fb[3]),
                  "+v"(fb[4]), "+v"(fb[5]), "+v"(fb[6]), "+v"(fb[7]));
 }
+__device__ __forceinline__ void wait_all_fragments(bf16x8 (&fa)[4], bf16x8 (&fb)[4]) {
+  asm volatile("s_waitcnt lgkmcnt(0)"
+               : "+v"(fa[0]), "+v"(fa[1]), "+v"(fa[2]), "+v"(fa[3]), "+v"(fb[0]), "+v"(fb[1]),
+                 "+v"(fb[2]), "+v"(fb[3]));
+}
+// Passes a row of accumulators through a statement (see the end of the kernel).
+__device__ __forceinline__ void settle_accumulators(f32x4 (&a)[8]) {
+  asm volatile("s_nop 3"
+               : "+a"(a[0]), "+a"(a[1]), "+a"(a[2]), "+a"(a[3]), "+a"(a[4]), "+a"(a[5]),
+                 "+a"(a[6]), "+a"(a[7]));
+}
+__device__ __forceinline__ void settle_accumulators(f32x4 (&a)[4]) {
+  asm volatile("s_nop 3" : "+a"(a[0]), "+a"(a[1]), "+a"(a[2]), "+a"(a[3]));
+}
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
 
-// 4 waves, one per SIMD, each owning 128 x 128 of the 256 x 256 tile: 8 x 8
-// blocks of 16 x 16, 256 accumulator registers, 64 MFMAs per 32-deep step.  A
-// wave pipelines against itself: while the MFMAs of one step run on one register
-// set (8 + 8 fragments), the fragments of the next step are read into the other,
-// one fragment between two MFMAs.
+// TILE = 256: 4 waves, one per SIMD, each owning 128 x 128 of the 256 x 256 tile:
+// 8 x 8 blocks of 16 x 16, 256 accumulator registers, 64 MFMAs per 32-deep step.
+// A wave pipelines against itself: while the MFMAs of one step run on one
+// register set (8 + 8 fragments), the fragments of the next step are read into
+// the other, one fragment between two MFMAs.
 //
 // LDS holds a ring of 5 operand tiles (160 KiB); the tiles A0 B0 A1 B1 A2 ... of
 // the contraction stages take the slots 0 1 2 3 4 0 1 ...  Stage p (64 deep):
@@ -413,14 +434,22 @@ __device__ __forceinline__ void wait_all_fragments(bf16x8 (&fa)[8], bf16x8 (&fb)
 // At the barrier every wave holds the last fragments of stage p in registers, so
 // both of its slots are free: B(p+2) takes A(p)'s, A(p+3) (next step 0) B(p)'s.
 // A tile has at least two steps (128 MFMAs per wave) to land.
-template <bool A_KMAJOR, bool B_KMAJOR, int EPI, bool OUT_F32>
+//
+// TILE = 128 is the same schedule on a 128 x 128 tile for problems that do not
+// fill the chip with 256 x 256 tiles: 64 x 64 per wave (4 x 4 blocks, 16 MFMAs per
+// step, 4 copies per tile and wave), an 80 KiB ring, two workgroups per CU.
+template <int TILE, bool A_KMAJOR, bool B_KMAJOR, int EPI, bool OUT_F32>
 __global__ void __launch_bounds__(256) gemm_bf16_solo_kernel(const GemmArgs g) {
-  constexpr int BM = 256, BN = 256, WTM = 128, WTN = 128, FR = 8;
+  constexpr int BM = TILE, BN = TILE, WTM = TILE / 2, WTN = TILE / 2, FR = TILE / 32;
   constexpr int PK = 64, NSLOT = 5;
-  using OA = DeepOperand<A_KMAJOR, false>;
-  using OB = DeepOperand<B_KMAJOR, true>;
-  constexpr uint32_t SLOT = OA::BYTES;  // 32 KiB
-  static_assert(OA::DMA_N == 8 && OB::DMA_N == 8 && OA::BYTES == OB::BYTES, "copy schedule below");
+  constexpr int NM = FR * FR;           // MFMAs per step
+  using OA = DeepOperand<A_KMAJOR, false, TILE>;
+  using OB = DeepOperand<B_KMAJOR, true, TILE>;
+  constexpr uint32_t SLOT = OA::BYTES;  // 32 or 16 KiB
+  constexpr int NC = OA::DMA_N;         // copies per tile and wave
+  constexpr int READ_EVERY = NM / (4 * FR);  // a fragment read every .. MFMAs, first half of a step
+  constexpr int COPY_EVERY = NM / (2 * NC);  // a copy every .. MFMAs, second half
+  static_assert(TILE == 256 || TILE == 128, "tile sizes with a schedule below");
 
   extern __shared__ __attribute__((aligned(16))) char lds[];
 
@@ -474,20 +503,20 @@ __global__ void __launch_bounds__(256) gemm_bf16_solo_kernel(const GemmArgs g) {
   auto b_done = [&]() { kb += b_step; wslot = next_slot(wslot); };
 
   // A0 B0 (A1 B1) up front.
-  static_for<8>(copy_a); a_done();
-  static_for<8>(copy_b); b_done();
+  static_for<NC>(copy_a); a_done();
+  static_for<NC>(copy_b); b_done();
   if (KP > 1) {
-    static_for<8>(copy_a); a_done();
-    static_for<8>(copy_b); b_done();
-    asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+    static_for<NC>(copy_a); a_done();
+    static_for<NC>(copy_b); b_done();
+    wait_vmcnt<2 * NC>();
   } else {
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   }
   __builtin_amdgcn_s_barrier();
 
   bf16x8 fa0[FR], fb0[FR], fa1[FR], fb1[FR];  // register sets of steps 0 / 1
-  // fragment f of 16 (A 0-7, B 0-7) of step ST of the stage whose tiles sit at
-  // sa / sb, into register set ST
+  // fragment f of 2 FR (A fragments, then B fragments) of step ST of the stage
+  // whose tiles sit at sa / sb, into register set ST
   auto read = [&](auto st_, auto f_, uint32_t sa, uint32_t sb) {
     constexpr int ST = decltype(st_)::value, f = decltype(f_)::value;
     bf16x8(&fa)[FR] = ST ? fa1 : fa0;
@@ -505,7 +534,7 @@ __global__ void __launch_bounds__(256) gemm_bf16_solo_kernel(const GemmArgs g) {
     }
   };
   uint32_t sa = 0, sb = SLOT;  // slots of the current stage's tiles
-  static_for<16>([&](auto f_) { read(std::integral_constant<int, 0>{}, f_, sa, sb); });
+  static_for<2 * FR>([&](auto f_) { read(std::integral_constant<int, 0>{}, f_, sa, sb); });
 
   // HAS2: stage p + 2 exists (its tiles are copied during this stage);
   // LAST: no stage follows.
@@ -519,30 +548,30 @@ __global__ void __launch_bounds__(256) gemm_bf16_solo_kernel(const GemmArgs g) {
       bf16x8(&fb)[FR] = ST ? fb1 : fb0;
       wait_all_fragments(fa, fb);  // every read of this set was issued during the previous step
       if constexpr (ST == 1 && !LAST) {
-        if (HAS2) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");  // A(p+2) may be in flight
-        else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        if (HAS2) wait_vmcnt<NC>();  // A(p+2) may be in flight
+        else wait_vmcnt<0>();
         __builtin_amdgcn_s_barrier();
       }
       __builtin_amdgcn_sched_barrier(0);
-      static_for<64>([&](auto m_) {
+      static_for<NM>([&](auto m_) {
         constexpr int m = decltype(m_)::value;
         constexpr int i = m / FR, j = m % FR;
         // Inline assembly pins the register classes (accumulators in AGPRs, fragments
         // in VGPRs): with the builtin the allocator moves two-instruction
         // (transposed) fragments through AGPRs and spills.  No MFMA hazard can arise:
         // fragments come from LDS behind s_waitcnt, and an accumulator is touched
-        // again only 63 MFMAs later.
+        // again only NM - 1 (at least 15) independent MFMAs later.
         asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0"
                      : "+a"(acc[i][j])
                      : "v"(fb[j]), "v"(fa[i]));
-        if constexpr (m < 32 && m % 2 == 0) {
+        if constexpr (m < NM / 2 && m % READ_EVERY == 0) {
           if constexpr (ST == 0) read(std::integral_constant<int, 1>{},
-                                      std::integral_constant<int, m / 2>{}, sa, sb);
+                                      std::integral_constant<int, m / READ_EVERY>{}, sa, sb);
           else if constexpr (!LAST) read(std::integral_constant<int, 0>{},
-                                         std::integral_constant<int, m / 2>{}, na, nb);
-        } else if constexpr (HAS2 && m >= 32 && m % 4 == 1) {
-          if constexpr (ST == 0) copy_a(std::integral_constant<int, (m - 32) / 4>{});
-          else copy_b(std::integral_constant<int, (m - 32) / 4>{});
+                                         std::integral_constant<int, m / READ_EVERY>{}, na, nb);
+        } else if constexpr (HAS2 && m >= NM / 2 && (m - NM / 2) % COPY_EVERY == COPY_EVERY - 1) {
+          if constexpr (ST == 0) copy_a(std::integral_constant<int, (m - NM / 2) / COPY_EVERY>{});
+          else copy_b(std::integral_constant<int, (m - NM / 2) / COPY_EVERY>{});
         }
         __builtin_amdgcn_sched_barrier(0);
       });
@@ -557,8 +586,14 @@ __global__ void __launch_bounds__(256) gemm_bf16_solo_kernel(const GemmArgs g) {
   for (int p = 0; p < KP - 2; ++p) stage(T{}, F{});
   if (KP > 1) stage(F{}, F{});
   stage(F{}, T{});
-  // the last MFMAs have left the pipeline before the accumulators are read
+  // The compiler does not know that the statements above are MFMAs: left alone it
+  // copies an accumulator out of its AGPRs right behind the MFMA that writes it,
+  // before the result has left the pipeline.  Every accumulator is therefore
+  // passed through a statement that follows the last MFMA by more than its
+  // latency; the epilogue can only read the values these statements return.
   asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+#pragma unroll
+  for (int i = 0; i < FR; ++i) settle_accumulators(acc[i]);
   // With the permuted column fragments a lane owns, per block row i and block
   // pair t, the 8 consecutive columns 32 t + 8 (l / 16) .. + 7 of row 16 i + l % 16:
   // they go out straight from the registers, 64 contiguous bytes per row and
@@ -689,13 +724,14 @@ int launch_cfg(const GemmArgs& in, hipStream_t stream) {
   return AXN_OK;
 }
 
-template <bool AK, bool BKM, int EPI, bool OUT_F32>
+template <int TILE, bool AK, bool BKM, int EPI, bool OUT_F32>
 int launch_solo(const GemmArgs& in, hipStream_t stream) {
   GemmArgs g = in;
-  g.tiles_m = g.M / 256;
-  g.tiles_n = g.N / 256;
-  constexpr size_t lds = 5 * 256 * 64 * 2;  // ring of 5 operand tiles, 160 KiB: all of a CU's LDS
-  auto kern = gemm_bf16_solo_kernel<AK, BKM, EPI, OUT_F32>;
+  g.tiles_m = g.M / TILE;
+  g.tiles_n = g.N / TILE;
+  // ring of 5 operand tiles: 160 KiB (all of a CU's LDS) or 80 KiB (two workgroups per CU)
+  constexpr size_t lds = 5 * TILE * 64 * 2;
+  auto kern = gemm_bf16_solo_kernel<TILE, AK, BKM, EPI, OUT_F32>;
   AXN_HIP_TRY(hipFuncSetAttribute((const void*)kern,
                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
   hipLaunchKernelGGL(kern, dim3((unsigned)(g.tiles_m * g.tiles_n)), dim3(256), lds, stream, g);
@@ -703,22 +739,26 @@ int launch_solo(const GemmArgs& in, hipStream_t stream) {
   return AXN_OK;
 }
 
-// Kernel selection.  Large problems made of whole 256 x 256 tiles take the
-// one-wave-per-SIMD kernel; problems that would leave most of the 256 CUs idle
-// at that tile size, and ragged ones, take 128 x 128 tiles on the
+// Kernel selection.  Problems made of whole 256 x 256 tiles, at least 192 of
+// them (3/4 of the CUs), take the one-wave-per-SIMD kernel at that tile size;
+// other problems made of whole 128 x 128 tiles take it at 128 x 128; ragged
+// shapes, and operands too large for 32-bit byte offsets, take the
 // register-staged kernel.
 template <bool AK, bool BKM, int EPI, bool OUT_F32>
 int launch_shape(const GemmArgs& g, hipStream_t stream) {
-  const bool whole256 = (g.M % 256 == 0) && (g.N % 256 == 0) && (g.Kc % BK == 0);
+  const bool deep = g.Kc % 64 == 0;
+  const bool whole256 = (g.M % 256 == 0) && (g.N % 256 == 0) && deep;
+  const bool whole128 = (g.M % 128 == 0) && (g.N % 128 == 0) && deep;
   const long long tiles256 = (long long)((g.M + 255) / 256) * ((g.N + 255) / 256);
+  const long long tiles128 = (long long)((g.M + 127) / 128) * ((g.N + 127) / 128);
   // The one-wave-per-SIMD kernel addresses its operands with 32-bit byte offsets.
   const int64_t a_span = (int64_t)(AK ? g.M : g.Kc) * g.lda * 2;
   const int64_t b_span = (int64_t)(BKM ? g.N : g.Kc) * g.ldb * 2;
   const bool small_spans = a_span < (1LL << 31) && b_span < (1LL << 31);
-  if (whole256 && tiles256 >= 192 && small_spans) {
-    return launch_solo<AK, BKM, EPI, OUT_F32>(g, stream);
-  }
-  const bool whole128 = (g.M % 128 == 0) && (g.N % 128 == 0) && (g.Kc % BK == 0);
+  if (small_spans && whole256 && tiles256 >= 192)
+    return launch_solo<256, AK, BKM, EPI, OUT_F32>(g, stream);
+  if (small_spans && whole128 && tiles128 < (1LL << 31))
+    return launch_solo<128, AK, BKM, EPI, OUT_F32>(g, stream);
   if (whole128) return launch_cfg<128, 128, 2, 2, AK, BKM, EPI, OUT_F32, false>(g, stream);
   return launch_cfg<128, 128, 2, 2, AK, BKM, EPI, OUT_F32, true>(g, stream);
 }

@@ -219,6 +219,42 @@ def test_fp32_gemms_match_oracle(M, N, K):
     assert rel(dw.cpu().numpy(), 2 * bw["dw"].reshape(N, K)) < F32_TOL
 
 
+@pytest.mark.parametrize("M,N,K", [(128, 128, 64), (256, 384, 192), (512, 256, 320), (4096, 3072, 128),
+                                   (4096, 3072, 320)])
+def test_tile_kernels_every_output_block_with_epilogues(M, N, K):
+    """Whole-tile shapes on the one-wave-per-SIMD kernel (128 x 128 tiles below 192
+    tiles of 256 x 256, else 256 x 256), checked element by element so that a single
+    wrong 16 x 16 accumulator block shows (a block copied out of its registers before
+    its last MFMA had finished once passed the normwise checks of other shapes)."""
+    from axonn_amd import ops
+
+    g = torch.Generator(device="cuda").manual_seed(M + N + K)
+    X = torch.randn(M, K, generator=g, device="cuda").bfloat16()
+    W = (torch.randn(N, K, generator=g, device="cuda") * 0.2).bfloat16()
+    b = torch.randn(N, generator=g, device="cuda") * 0.5
+    dY = torch.randn(M, N, generator=g, device="cuda").bfloat16()
+    pre = X.float() @ W.float().t()
+    scale = pre.abs().max().item()
+
+    def close(got, want, ulps=1.0):
+        return bool(((got.float() - want).abs() <= ulps * 2.0 ** -8 * want.abs() + 1e-3 * scale).all())
+
+    for bias, act in ((None, None), (b, None), (b, "gelu"), (None, "gelu")):
+        y, z = ops.gemm_fwd(X, W, bias=bias, activation=act, save_z=act is not None)
+        zr = pre + (bias if bias is not None else 0)
+        assert close(y, torch.nn.functional.gelu(zr) if act else zr)
+        if act:
+            assert close(z, zr)
+    assert close(ops.gemm_dgrad(dY, W), dY.float() @ W.float())
+    dwr = dY.float().t() @ X.float()
+    dw = ops.gemm_wgrad(dY, X)
+    assert close(dw, dwr)
+    dw32 = ops.gemm_wgrad(dY, X, out_dtype=torch.float32)
+    assert bool(((dw32 - dwr).abs() <= 1e-4 * dwr.abs().max()).all())
+    ops.gemm_wgrad(dY, X, out=dw, accumulate=True)
+    assert close(dw, 2 * dwr, ulps=2.0)
+
+
 # ---- the 256 x 256-tile kernel: few and many contraction stages, all layouts/epilogues ----
 @pytest.mark.parametrize("K", [64, 128, 192, 256, 448])
 def test_tile256_kernel_short_contractions(K):
