@@ -207,6 +207,36 @@ int axn_dgelu_dbias(const void* dY, const void* Z, void* dZ, int dtype,
                             workspace_bytes, (hipStream_t)stream);
 }
 
+static int check_swiglu(const char* name, int dtype, int64_t M, int64_t N, int64_t ld) {
+  REQUIRE(dtype == AXN_BF16 || dtype == AXN_F32, AXN_EINVAL, "%s: dtype must be bf16 or fp32", name);
+  REQUIRE(M >= 1 && N >= 1, AXN_EINVAL, "%s: M and N must be >= 1", name);
+  REQUIRE(N % 8 == 0, AXN_ESHAPE, "%s: N must be a multiple of 8", name);
+  REQUIRE(ld >= N && ld % 8 == 0, AXN_EALIGN, "%s: ld must be >= N and a multiple of 8", name);
+  return AXN_OK;
+}
+
+int axn_swiglu_fwd(const void* gate, const void* up, void* out, int dtype, int64_t M,
+                   int64_t N, int64_t ld, void* stream) {
+  const char* name = "axn_swiglu_fwd";
+  REQUIRE(gate && up && out, AXN_EINVAL, "%s: null pointer", name);
+  int rc = check_swiglu(name, dtype, M, N, ld);
+  if (rc) return rc;
+  REQUIRE(aligned16(gate) && aligned16(up) && aligned16(out), AXN_EALIGN,
+          "%s: pointers must be 16-byte aligned", name);
+  return launch_swiglu_fwd(gate, up, out, dtype, M, N, ld, (hipStream_t)stream);
+}
+
+int axn_swiglu_bwd(const void* dout, const void* gate, const void* up, void* dgate,
+                   void* dup, int dtype, int64_t M, int64_t N, int64_t ld, void* stream) {
+  const char* name = "axn_swiglu_bwd";
+  REQUIRE(dout && gate && up && dgate && dup, AXN_EINVAL, "%s: null pointer", name);
+  int rc = check_swiglu(name, dtype, M, N, ld);
+  if (rc) return rc;
+  REQUIRE(aligned16(dout) && aligned16(gate) && aligned16(up) && aligned16(dgate) && aligned16(dup),
+          AXN_EALIGN, "%s: pointers must be 16-byte aligned", name);
+  return launch_swiglu_bwd(dout, gate, up, dgate, dup, dtype, M, N, ld, (hipStream_t)stream);
+}
+
 int axn_gemm_fwd_f32(const float* X, const float* W, const float* bias, float* Y,
                      float* Zsave, int64_t M, int64_t N, int64_t K, int epilogue,
                      void* stream) {

@@ -88,6 +88,12 @@ int launch_dgelu_dbias(const void* dY, const void* Z, void* dZ, int dtype,
                        float* dbias, int64_t M, int64_t N, int64_t ld, int beta,
                        void* ws, size_t ws_bytes, hipStream_t stream);
 
+// ---- SwiGLU activation of the Llama MLP and its backward -----------------------
+int launch_swiglu_fwd(const void* gate, const void* up, void* out, int dtype, int64_t M,
+                      int64_t N, int64_t ld, hipStream_t stream);
+int launch_swiglu_bwd(const void* dout, const void* gate, const void* up, void* dgate, void* dup,
+                      int dtype, int64_t M, int64_t N, int64_t ld, hipStream_t stream);
+
 // ---- multi-tensor optimizer ------------------------------------------------
 size_t mt_scan_workspace_bytes(int64_t n, int64_t total);
 int launch_mt_scan(const void* const* h_g, const int64_t* h_sizes, int64_t n,

@@ -6,6 +6,13 @@
 // registers over a band of rows, combined through LDS, written as one fp32
 // partial row per band and reduced over bands in a fixed order by a second
 // kernel, so the result does not depend on scheduling.
+//
+// Also here: the SwiGLU activation of the Llama MLP, h = silu(gate) * up, and its
+// backward, each one HBM pass.  The reference's Llama patch
+// (axonn/models/transformers/modify_llama.py:76-95) swaps the three projections
+// for its Linear and leaves `act_fn(gate_proj(x)) * up_proj(x)` to separate
+// elementwise kernels with a bf16 rounding in between; here the product is formed
+// in fp32 and rounded once.
 #include "axn_internal.h"
 
 namespace axn {
@@ -109,7 +116,97 @@ __global__ void __launch_bounds__(256)
   }
 }
 
+// sigmoid(x) = 1 / (1 + exp(-x)); exp overflows to +inf for x < -88 and the
+// reciprocal then gives the correct limit 0.
+__device__ __forceinline__ float sigmoid_f(float x) {
+  return __builtin_amdgcn_rcpf(1.0f + __expf(-x));
+}
+
+template <typename T>
+__global__ void __launch_bounds__(EW_TX* EW_TY)
+    swiglu_fwd_kernel(const T* gate, const T* up, T* out, int64_t M, int64_t N, int64_t ld) {
+  const int tx = threadIdx.x % EW_TX, ty = threadIdx.x / EW_TX;
+  const int64_t col = (int64_t)blockIdx.x * EW_COLS + tx * 8;
+  if (col >= N) return;
+  const int64_t r0 = (int64_t)blockIdx.y * EW_BAND;
+  const int64_t r1 = (r0 + EW_BAND < M) ? r0 + EW_BAND : M;
+  for (int64_t r = r0 + ty; r < r1; r += EW_TY) {
+    const int64_t o = r * ld + col;
+    float g[8], u[8];
+    load8(gate + o, g);
+    load8(up + o, u);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) g[e] = g[e] * sigmoid_f(g[e]) * u[e];
+    store8(out + o, g);
+  }
+}
+
+// dgate = dout * up * silu'(gate),  dup = dout * silu(gate),
+// silu'(x) = s (1 + x (1 - s)) with s = sigmoid(x).
+template <typename T>
+__global__ void __launch_bounds__(EW_TX* EW_TY)
+    swiglu_bwd_kernel(const T* dout, const T* gate, const T* up, T* dgate, T* dup, int64_t M,
+                      int64_t N, int64_t ld) {
+  const int tx = threadIdx.x % EW_TX, ty = threadIdx.x / EW_TX;
+  const int64_t col = (int64_t)blockIdx.x * EW_COLS + tx * 8;
+  if (col >= N) return;
+  const int64_t r0 = (int64_t)blockIdx.y * EW_BAND;
+  const int64_t r1 = (r0 + EW_BAND < M) ? r0 + EW_BAND : M;
+  for (int64_t r = r0 + ty; r < r1; r += EW_TY) {
+    const int64_t o = r * ld + col;
+    float d[8], g[8], u[8], dg[8], du[8];
+    load8(dout + o, d);
+    load8(gate + o, g);
+    load8(up + o, u);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float sg = sigmoid_f(g[e]);
+      du[e] = d[e] * g[e] * sg;
+      dg[e] = d[e] * u[e] * sg * (1.0f + g[e] * (1.0f - sg));
+    }
+    store8(dgate + o, dg);
+    store8(dup + o, du);
+  }
+}
+
 }  // namespace
+
+int launch_swiglu_fwd(const void* gate, const void* up, void* out, int dtype, int64_t M,
+                      int64_t N, int64_t ld, hipStream_t stream) {
+  const int64_t bands = (M + EW_BAND - 1) / EW_BAND;
+  if (bands > 65535) {
+    set_error("swiglu: too many rows (%lld)", (long long)M);
+    return AXN_ELIMIT;
+  }
+  const dim3 grid((unsigned)((N + EW_COLS - 1) / EW_COLS), (unsigned)bands), block(EW_TX * EW_TY);
+  if (dtype == AXN_F32)
+    hipLaunchKernelGGL(swiglu_fwd_kernel<float>, grid, block, 0, stream, (const float*)gate,
+                       (const float*)up, (float*)out, M, N, ld);
+  else
+    hipLaunchKernelGGL(swiglu_fwd_kernel<uint16_t>, grid, block, 0, stream, (const uint16_t*)gate,
+                       (const uint16_t*)up, (uint16_t*)out, M, N, ld);
+  AXN_HIP_TRY(hipGetLastError());
+  return AXN_OK;
+}
+
+int launch_swiglu_bwd(const void* dout, const void* gate, const void* up, void* dgate, void* dup,
+                      int dtype, int64_t M, int64_t N, int64_t ld, hipStream_t stream) {
+  const int64_t bands = (M + EW_BAND - 1) / EW_BAND;
+  if (bands > 65535) {
+    set_error("swiglu: too many rows (%lld)", (long long)M);
+    return AXN_ELIMIT;
+  }
+  const dim3 grid((unsigned)((N + EW_COLS - 1) / EW_COLS), (unsigned)bands), block(EW_TX * EW_TY);
+  if (dtype == AXN_F32)
+    hipLaunchKernelGGL(swiglu_bwd_kernel<float>, grid, block, 0, stream, (const float*)dout,
+                       (const float*)gate, (const float*)up, (float*)dgate, (float*)dup, M, N, ld);
+  else
+    hipLaunchKernelGGL(swiglu_bwd_kernel<uint16_t>, grid, block, 0, stream, (const uint16_t*)dout,
+                       (const uint16_t*)gate, (const uint16_t*)up, (uint16_t*)dgate,
+                       (uint16_t*)dup, M, N, ld);
+  AXN_HIP_TRY(hipGetLastError());
+  return AXN_OK;
+}
 
 size_t dgelu_dbias_workspace_bytes(int64_t M, int64_t N) {
   if (M <= 0 || N <= 0) return 0;

@@ -182,6 +182,50 @@ def dgelu_dbias(dy, z=None, want_dbias=True, dbias_out=None, accumulate=False):
     return (dz if dz is not None else dy), dbias
 
 
+def _same_2d(name, ref, *others):
+    for t in others:
+        if t.dtype != ref.dtype or t.shape != ref.shape:
+            raise ValueError("%s: operands must match in dtype and shape" % name)
+
+
+def _swiglu_operands(name, tensors):
+    ref = tensors[0]
+    if ref.dtype not in (torch.bfloat16, torch.float32):
+        raise TypeError("%s: bf16 or fp32 expected, got %s" % (name, ref.dtype))
+    if ref.dim() != 2 or ref.shape[1] % 8:
+        raise ValueError("%s: 2-D operands with a multiple of 8 columns expected, got %s"
+                         % (name, tuple(ref.shape)))
+    _same_2d(name, ref, *tensors[1:])
+    out = []
+    for t in tensors:
+        if not t.is_contiguous() or t.data_ptr() % 16:
+            t = t.contiguous().clone()
+        out.append(t)
+    return out
+
+
+def swiglu_fwd(gate, up):
+    """silu(gate) * up, the activation of the Llama MLP, in one pass."""
+    _require_gpu(gate, up)
+    gate, up = _swiglu_operands("swiglu_fwd", [gate, up])
+    M, N = gate.shape
+    out = torch.empty_like(gate)
+    nv.call("axn_swiglu_fwd", nv.ptr(gate), nv.ptr(up), nv.ptr(out), nv.dtype_code(gate.dtype),
+            M, N, N, nv.current_stream())
+    return out
+
+
+def swiglu_bwd(dout, gate, up):
+    """(dgate, dup) for out = silu(gate) * up."""
+    _require_gpu(dout, gate, up)
+    dout, gate, up = _swiglu_operands("swiglu_bwd", [dout, gate, up])
+    M, N = gate.shape
+    dgate, dup = torch.empty_like(gate), torch.empty_like(up)
+    nv.call("axn_swiglu_bwd", nv.ptr(dout), nv.ptr(gate), nv.ptr(up), nv.ptr(dgate), nv.ptr(dup),
+            nv.dtype_code(gate.dtype), M, N, N, nv.current_stream())
+    return dgate, dup
+
+
 # ---------------------------------------------------------- multi-tensor -----
 class ScanResult:
     """Device-resident axn_scan_result (32 bytes) with typed views."""

@@ -14,8 +14,8 @@ keys of the one JSON line:
   adam      the mixed-precision Adam step (scan + update) on 1.3e9 parameters in
             64 ragged tensors, GB/s at 30 algorithmic bytes per element, and the
             overflow (skip) variant
-  shapes    the 12B-style MLP shard with fused bias + GELU and the skinny
-            decode-like shard
+  shapes    the 12B-style MLP shard with fused bias + GELU, the skinny
+            decode-like shard, and the Llama MLP block with the one-pass SwiGLU
   cpu_baseline  the torch-CPU restatement of the same layer math on the host cores
 
 Every GEMM launch of the timed region is bracketed by HIP events on the launch
@@ -242,6 +242,50 @@ def main():
             "frac_mfma": round(L.flops / t / 1e12 / PEAK_BF16_TFLOPS, 4),
             "gbs": round(nbytes / t / 1e9, 1), "frac_hbm": round(nbytes / t / 1e9 / PEAK_HBM_GBS, 4)}
         del L
+        torch.cuda.empty_cache()
+
+        # Llama-3-8B MLP block, 4096 tokens: gate/up/down projections with the one-pass
+        # SwiGLU between them, forward + backward (9 GEMMs, 2 elementwise passes, and
+        # torch's add of the two input-gradient contributions).
+        Mt, H, I = 4096, 4096, 14336
+        g = torch.Generator(device="cuda").manual_seed(12)
+        x = torch.randn(Mt, H, generator=g, device="cuda").bfloat16()
+        wg, wu = ((torch.randn(I, H, generator=g, device="cuda") * 0.02).bfloat16() for _ in range(2))
+        wd = (torch.randn(H, I, generator=g, device="cuda") * 0.02).bfloat16()
+        dy = (torch.randn(Mt, H, generator=g, device="cuda") * 1e-3).bfloat16()
+        bf = dict(dtype=torch.bfloat16, device="cuda")
+        gt, up, act = (torch.empty(Mt, I, **bf) for _ in range(3))
+        dact, dgt, dup = (torch.empty(Mt, I, **bf) for _ in range(3))
+        y, dx1, dx2 = (torch.empty(Mt, H, **bf) for _ in range(3))
+        dwg, dwu, dwd = torch.empty(I, H, **bf), torch.empty(I, H, **bf), torch.empty(H, I, **bf)
+        P = lambda t: t.data_ptr()  # noqa: E731
+
+        def mlp_block_step():
+            chk = nv.check
+            chk(lib.axn_gemm_fwd(P(x), P(wg), None, P(gt), None, Mt, I, H, H, H, I, nv.EPI_NONE, stream))
+            chk(lib.axn_gemm_fwd(P(x), P(wu), None, P(up), None, Mt, I, H, H, H, I, nv.EPI_NONE, stream))
+            chk(lib.axn_swiglu_fwd(P(gt), P(up), P(act), nv.BF16, Mt, I, I, stream))
+            chk(lib.axn_gemm_fwd(P(act), P(wd), None, P(y), None, Mt, H, I, I, I, H, nv.EPI_NONE, stream))
+            chk(lib.axn_gemm_dgrad(P(dy), P(wd), P(dact), Mt, H, I, H, I, I, stream))
+            chk(lib.axn_gemm_wgrad(P(dy), P(act), P(dwd), Mt, H, I, H, I, I, 0, nv.BF16, stream))
+            chk(lib.axn_swiglu_bwd(P(dact), P(gt), P(up), P(dgt), P(dup), nv.BF16, Mt, I, I, stream))
+            chk(lib.axn_gemm_dgrad(P(dgt), P(wg), P(dx1), Mt, I, H, I, H, H, stream))
+            chk(lib.axn_gemm_dgrad(P(dup), P(wu), P(dx2), Mt, I, H, I, H, H, stream))
+            torch.add(dx1, dx2, out=dx1)
+            chk(lib.axn_gemm_wgrad(P(dgt), P(x), P(dwg), Mt, I, H, I, H, H, 0, nv.BF16, stream))
+            chk(lib.axn_gemm_wgrad(P(dup), P(x), P(dwu), Mt, I, H, I, H, H, 0, nv.BF16, stream))
+
+        t = time_loop(mlp_block_step, max(args.steps // 2, 3))
+        fl = 18.0 * Mt * H * I
+        t_sw = time_loop(lambda: nv.check(lib.axn_swiglu_fwd(P(gt), P(up), P(act), nv.BF16, Mt, I, I, stream)), 10)
+        t_swb = time_loop(lambda: nv.check(lib.axn_swiglu_bwd(P(dact), P(gt), P(up), P(dgt), P(dup), nv.BF16,
+                                                             Mt, I, I, stream)), 10)
+        shapes["llama_mlp_block_4096x4096x14336_swiglu"] = {
+            "us": round(t * 1e6, 1), "tflops": round(fl / t / 1e12, 1),
+            "frac_mfma": round(fl / t / 1e12 / PEAK_BF16_TFLOPS, 4),
+            "swiglu_fwd_gbs": round(6.0 * Mt * I / t_sw / 1e9, 1),
+            "swiglu_bwd_gbs": round(10.0 * Mt * I / t_swb / 1e9, 1)}
+        del x, wg, wu, wd, dy, gt, up, act, dact, dgt, dup, y, dx1, dx2, dwg, dwu, dwd
         torch.cuda.empty_cache()
 
     adam = None

@@ -30,7 +30,7 @@
 extern "C" {
 #endif
 
-#define AXN_ABI_VERSION 1
+#define AXN_ABI_VERSION 2
 
 #if defined(__GNUC__)
 #define AXN_API __attribute__((visibility("default")))
@@ -113,6 +113,27 @@ AXN_API int axn_dgelu_dbias(const void* dY, const void* Z, void* dZ, int dtype,
                     float* dbias, int64_t M, int64_t N, int64_t ld, int beta,
                     void* workspace, size_t workspace_bytes, void* stream);
 AXN_API size_t axn_dgelu_dbias_workspace_bytes(int64_t M, int64_t N);
+
+/* SwiGLU activation of the Llama MLP, one pass over [M,N]:
+ *   out = silu(gate) * up,  silu(x) = x / (1 + exp(-x)).
+ * The reference's Llama patch (axonn/models/transformers/modify_llama.py:76-95)
+ * replaces gate_proj / up_proj / down_proj by its Linear and leaves
+ * `act_fn(gate_proj(x)) * up_proj(x)` of the model's forward to two elementwise
+ * kernels; this entry point and the next replace those and their autograd.
+ * gate, up, out of `dtype` (AXN_BF16 or AXN_F32), row stride ld; N % 8 == 0,
+ * ld % 8 == 0, pointers 16-byte aligned.  Computed in fp32, rounded once.
+ * out may alias gate or up. */
+AXN_API int axn_swiglu_fwd(const void* gate, const void* up, void* out, int dtype,
+                   int64_t M, int64_t N, int64_t ld, void* stream);
+
+/* Backward of the above:
+ *   dgate = dout * up * silu'(gate),  dup = dout * silu(gate),
+ *   silu'(x) = s (1 + x (1 - s)),  s = 1 / (1 + exp(-x)).
+ * dgate may alias gate and dup may alias up (each element is read before the
+ * element at the same position is written). */
+AXN_API int axn_swiglu_bwd(const void* dout, const void* gate, const void* up,
+                   void* dgate, void* dup, int dtype, int64_t M, int64_t N,
+                   int64_t ld, void* stream);
 
 /* fp32 variants of the three GEMMs for full-precision layers (the reference's
  * own tests run the layer in fp32: axonn/tests/test_intra_layer_fc.py:25).

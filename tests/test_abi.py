@@ -74,6 +74,19 @@ def test_gemm_argument_errors():
     assert lib.axn_gemm_dgrad_f32(ctypes.c_void_p(0x1002), A, A, 4, 4, 4, None) == nv.AXN_EALIGN
 
 
+def test_swiglu_argument_errors():
+    lib = nv.load()
+    f, b = lib.axn_swiglu_fwd, lib.axn_swiglu_bwd
+    assert f(None, A, A, nv.BF16, 8, 8, 8, None) == nv.AXN_EINVAL
+    assert f(A, A, A, nv.F16, 8, 8, 8, None) == nv.AXN_EINVAL
+    assert f(A, A, A, nv.BF16, 8, 12, 16, None) == nv.AXN_ESHAPE
+    assert f(A, A, A, nv.BF16, 8, 8, 4, None) == nv.AXN_EALIGN          # ld < N
+    assert f(ctypes.c_void_p(0x1008), A, A, nv.BF16, 8, 8, 8, None) == nv.AXN_EALIGN
+    assert b(A, A, A, A, None, nv.BF16, 8, 8, 8, None) == nv.AXN_EINVAL
+    assert b(A, A, A, A, A, nv.F32, 0, 8, 8, None) == nv.AXN_EINVAL
+    assert "axn_swiglu_bwd" in _err()
+
+
 def test_elementwise_argument_errors():
     lib = nv.load()
     f = lib.axn_dgelu_dbias

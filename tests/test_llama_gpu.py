@@ -1,0 +1,140 @@
+"""Parity of the Llama MLP block (patched Hugging Face LlamaMLP on the kernels)
+and of the SwiGLU kernels with the CPU oracle.
+
+Tolerances: the SwiGLU kernels compute in fp32 and round once, so against the
+float64 oracle on the same inputs the bf16 result is within one bf16 rounding
+(checked elementwise) and the fp32 result within 1e-6 relative.  The block's
+outputs and gradients, which pass through three bf16 GEMMs, use the GEMM bar:
+normwise 1e-2 against the float64 oracle fed the same bf16 weights and inputs.
+"""
+
+import numpy as np
+import pytest
+import torch
+
+from axonn_amd import _native as nv
+from oracle import llama as om
+
+pytestmark = pytest.mark.gpu
+
+
+def np64(t):
+    return t.detach().float().cpu().numpy().astype(np.float64)
+
+
+def rel(a, b):
+    a, b = np.asarray(a, np.float64), np.asarray(b, np.float64)
+    return float(np.linalg.norm(a - b) / max(np.linalg.norm(b), 1e-300))
+
+
+@pytest.mark.parametrize("M,N", [(1, 8), (37, 520), (256, 1024)])
+def test_swiglu_kernels_match_oracle_elementwise(M, N):
+    from axonn_amd import ops
+
+    g = torch.Generator().manual_seed(M * 1000 + N)
+    gate = (torch.randn(M, N, generator=g) * 3).bfloat16()
+    up = torch.randn(M, N, generator=g).bfloat16()
+    dout = torch.randn(M, N, generator=g).bfloat16()
+    want = om.swiglu_forward(np64(gate), np64(up))
+    out = ops.swiglu_fwd(gate.cuda(), up.cuda())
+    assert np.all(np.abs(np64(out) - want) <= 2.0 ** -8 * np.abs(want) + 1e-30)
+    wdg, wdu = om.swiglu_backward(np64(dout), np64(gate), np64(up))
+    dg, du = ops.swiglu_bwd(dout.cuda(), gate.cuda(), up.cuda())
+    assert np.all(np.abs(np64(dg) - wdg) <= 2.0 ** -8 * np.abs(wdg) + 1e-6)
+    assert np.all(np.abs(np64(du) - wdu) <= 2.0 ** -8 * np.abs(wdu) + 1e-6)
+    # fp32 storage: only the fp32 arithmetic error is left
+    o32 = ops.swiglu_fwd(gate.float().cuda(), up.float().cuda())
+    assert rel(o32.cpu().numpy(), want) < 1e-6
+    dg32, du32 = ops.swiglu_bwd(dout.float().cuda(), gate.float().cuda(), up.float().cuda())
+    assert rel(dg32.cpu().numpy(), wdg) < 1e-6 and rel(du32.cpu().numpy(), wdu) < 1e-6
+
+
+def test_swiglu_tails_and_special_values():
+    from axonn_amd import ops
+
+    # the hardware exp / reciprocal pair is good to a few 1e-7 relative; below -88 the
+    # exponential overflows and the result is the limit 0 instead of a value under 1e-36
+    gate = torch.tensor([[-200.0, -90.0, -30.0, -1e-3, 0.0, 1e-3, 30.0, 200.0]] * 2)
+    up = torch.full_like(gate, 1.5)
+    out = ops.swiglu_fwd(gate.cuda(), up.cuda()).cpu().numpy()
+    want = om.swiglu_forward(gate.numpy(), up.numpy())
+    assert np.all(np.isfinite(out)) and np.allclose(out, want, rtol=5e-6, atol=1e-30)
+    dg, du = ops.swiglu_bwd(torch.ones_like(gate).cuda(), gate.cuda(), up.cuda())
+    wdg, wdu = om.swiglu_backward(np.ones(gate.shape), gate.numpy(), up.numpy())
+    assert np.all(np.isfinite(dg.cpu().numpy())) and np.allclose(dg.cpu().numpy(), wdg, rtol=5e-6, atol=1e-30)
+    assert np.allclose(du.cpu().numpy(), wdu, rtol=5e-6, atol=1e-30)
+
+
+def test_swiglu_rejects_bad_arguments():
+    from axonn_amd import ops
+
+    a = torch.zeros(4, 12, device="cuda", dtype=torch.bfloat16)
+    with pytest.raises(ValueError):
+        ops.swiglu_fwd(a, a)                       # 12 columns: not a multiple of 8
+    b = torch.zeros(4, 16, device="cuda", dtype=torch.bfloat16)
+    with pytest.raises(ValueError):
+        ops.swiglu_fwd(b, b.float())
+    with pytest.raises(TypeError):
+        ops.swiglu_fwd(b.half(), b.half())
+    with pytest.raises(RuntimeError):
+        ops.swiglu_fwd(b.cpu(), b.cpu())
+
+
+@pytest.mark.parametrize("M,H,I", [(48, 64, 160), (512, 256, 768)])
+def test_patched_llama_mlp_block_matches_oracle(M, H, I):
+    """LlamaMLP built inside `parallelize` has the three projections on the GEMM
+    kernels and the fused SwiGLU between them; forward and backward against the
+    oracle block with bf16 storage between the stages."""
+    from transformers import LlamaConfig
+    from transformers.models.llama.modeling_llama import LlamaMLP
+
+    import axonn_amd.axonn as ax
+    from axonn_amd.intra_layer import Linear
+    from axonn_amd.models.transformers import parallelize
+
+    ax.init(1, 1, 1, 1)
+    cfg = LlamaConfig(hidden_size=H, intermediate_size=I, num_attention_heads=4, num_key_value_heads=2,
+                      num_hidden_layers=1, vocab_size=32)
+    original_forward = LlamaMLP.forward
+    with parallelize(cfg):
+        mlp = LlamaMLP(cfg)
+    assert LlamaMLP.forward is original_forward          # the patch is undone on exit
+    assert isinstance(mlp.gate_proj, Linear) and mlp.gate_proj.weight.dim() == 1
+    from axonn_amd.models.transformers.modify_llama import modified_mlp_forward
+    mlp.forward = modified_mlp_forward.__get__(mlp)      # the instance keeps the fused forward
+    mlp = mlp.cuda().bfloat16()
+    g = torch.Generator(device="cuda").manual_seed(M)
+    x = torch.randn(M, H, generator=g, device="cuda").bfloat16().requires_grad_(True)
+    dy = (torch.randn(M, H, generator=g, device="cuda") * 0.1).bfloat16()
+    y = mlp(x)
+    y.backward(dy)
+    wg, wu, wd = (np64(p).reshape(-1) for p in (mlp.gate_proj.weight, mlp.up_proj.weight, mlp.down_proj.weight))
+    fwd = om.llama_mlp_forward(np64(x), wg, wu, wd, H, I, store="bf16")
+    bwd = om.llama_mlp_backward(np64(x), wg, wu, wd, H, I, np64(dy), fwd, store="bf16")
+    assert rel(np64(y), fwd["out"]) < 1e-2
+    assert rel(np64(x.grad), bwd["dx"]) < 1e-2
+    for key, lin in (("dw_gate", mlp.gate_proj), ("dw_up", mlp.up_proj), ("dw_down", mlp.down_proj)):
+        assert rel(np64(lin.weight.grad), bwd[key]) < 1e-2
+    # and the same block on Hugging Face's own forward (two elementwise kernels of torch)
+    with torch.no_grad():
+        y_ref = mlp.down_proj(torch.nn.functional.silu(mlp.gate_proj(x)) * mlp.up_proj(x))
+    assert rel(np64(y), np64(y_ref)) < 1e-2
+
+
+def test_patched_attention_projections_are_linear_layers():
+    from transformers import LlamaConfig
+    from transformers.models.llama.modeling_llama import LlamaAttention
+
+    import axonn_amd.axonn as ax
+    from axonn_amd.intra_layer import Linear
+    from axonn_amd.models.transformers import parallelize
+
+    ax.init(1, 1, 1, 1)
+    cfg = LlamaConfig(hidden_size=64, intermediate_size=128, num_attention_heads=4, num_key_value_heads=2,
+                      num_hidden_layers=1, vocab_size=32)
+    with parallelize(cfg):
+        attn = LlamaAttention(cfg, 0)
+    for name, shape in (("q_proj", (64, 64)), ("k_proj", (32, 64)), ("v_proj", (32, 64)), ("o_proj", (64, 64))):
+        lin = getattr(attn, name)
+        assert isinstance(lin, Linear) and lin.weight.numel() == shape[0] * shape[1]
+    assert not isinstance(LlamaAttention(cfg, 0).q_proj, Linear)

@@ -382,3 +382,56 @@ def test_torch_cpu_mlp_step_matches_numpy_oracle():
     assert np.allclose(bw2["dw"].reshape(D, Hd), res["grads"][2].numpy(), rtol=1e-4, atol=1e-7)
     p1, _, _ = oo.adam_update(w1.numpy(), res["grads"][0].numpy(), 0 * w1.numpy(), 0 * w1.numpy(), 1)
     assert np.allclose(p1, res["params"][0].numpy(), rtol=1e-6, atol=0)
+
+
+# ---- Llama MLP block (oracle/llama.py) ------------------------------------------
+def test_silu_swiglu_pinned_by_torch_closed_forms_and_finite_differences():
+    from oracle import llama as om
+
+    x = np.linspace(-30.0, 30.0, 2001)
+    t = torch.tensor(x, dtype=torch.float64, requires_grad=True)
+    y = torch.nn.functional.silu(t)
+    y.sum().backward()
+    assert np.allclose(om.silu(x), y.detach().numpy(), rtol=1e-13, atol=1e-300)
+    assert np.allclose(om.dsilu(x), t.grad.numpy(), rtol=1e-12, atol=1e-15)
+    # closed forms: silu(0) = 0, silu'(0) = 1/2, silu(x) - silu(-x) = x, silu -> x / 0 in the tails
+    assert om.silu(np.array([0.0]))[0] == 0.0 and om.dsilu(np.array([0.0]))[0] == 0.5
+    assert np.allclose(om.silu(x) - om.silu(-x), x, atol=1e-13)
+    assert abs(om.silu(np.array([40.0]))[0] - 40.0) < 1e-12 and abs(om.silu(np.array([-745.0]))[0]) < 1e-300
+    h = 1e-6
+    fd = (om.silu(x + h) - om.silu(x - h)) / (2 * h)
+    assert np.allclose(om.dsilu(x), fd, atol=1e-8)
+    # swiglu backward against autograd, and a dropped-factor check: dgate must depend on up
+    g = torch.randn(7, 16, dtype=torch.float64, requires_grad=True)
+    u = torch.randn(7, 16, dtype=torch.float64, requires_grad=True)
+    d = torch.randn(7, 16, dtype=torch.float64)
+    (torch.nn.functional.silu(g) * u).backward(d)
+    dg, du = om.swiglu_backward(d.numpy(), g.detach().numpy(), u.detach().numpy())
+    assert np.allclose(dg, g.grad.numpy(), rtol=1e-12) and np.allclose(du, u.grad.numpy(), rtol=1e-12)
+    assert not np.allclose(dg, om.swiglu_backward(d.numpy(), g.detach().numpy(), 2 * u.detach().numpy())[0])
+
+
+def test_llama_mlp_oracle_matches_hugging_face_block_with_autograd():
+    """The unpatched Hugging Face LlamaMLP in float64 on the CPU is the library
+    routine the oracle's block must equal, forward and backward."""
+    from transformers import LlamaConfig
+    from transformers.models.llama.modeling_llama import LlamaMLP
+    from oracle import llama as om
+
+    torch.manual_seed(3)
+    H, I, M = 24, 56, 10
+    cfg = LlamaConfig(hidden_size=H, intermediate_size=I, num_attention_heads=4, num_key_value_heads=2,
+                      num_hidden_layers=1, vocab_size=32)
+    mlp = LlamaMLP(cfg).double()
+    x = torch.randn(M, H, dtype=torch.float64, requires_grad=True)
+    dy = torch.randn(M, H, dtype=torch.float64)
+    y = mlp(x)
+    y.backward(dy)
+    wg, wu, wd = (p.detach().numpy().reshape(-1) for p in
+                  (mlp.gate_proj.weight, mlp.up_proj.weight, mlp.down_proj.weight))
+    fwd = om.llama_mlp_forward(x.detach().numpy(), wg, wu, wd, H, I)
+    bwd = om.llama_mlp_backward(x.detach().numpy(), wg, wu, wd, H, I, dy.numpy(), fwd)
+    assert np.allclose(fwd["out"], y.detach().numpy(), rtol=1e-12, atol=1e-14)
+    assert np.allclose(bwd["dx"], x.grad.numpy(), rtol=1e-11, atol=1e-14)
+    for key, lin in (("dw_gate", mlp.gate_proj), ("dw_up", mlp.up_proj), ("dw_down", mlp.down_proj)):
+        assert np.allclose(bwd[key].reshape(lin.weight.shape), lin.weight.grad.numpy(), rtol=1e-11, atol=1e-14)
