@@ -40,8 +40,8 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 # file, scaled by what the same counters read for the 1 GiB copy below
 # (profiles/gemm_adam_llama_set_pmc.txt has the runs and the arithmetic).  The
 # counters sit between L2 and the fabric, so hits in the memory-side cache are included.
-TRAFFIC_BYTES_PER_LAUNCH = {"fwd": 634480098, "dgrad": 594794773, "wgrad": 702799177}
-ADAM_TRAFFIC_BYTES_PER_STEP = 39819558462   # scan + update, 1.3e9 elements
+TRAFFIC_BYTES_PER_LAUNCH = {"fwd": 634514096, "dgrad": 591325408, "wgrad": 694834872}
+ADAM_TRAFFIC_BYTES_PER_STEP = 39818024670   # scan + update, 1.3e9 elements
 
 LLAMA_SET = [  # (name, M, N, K), gate and up are two layers of one shape
     ("qkv", 4096, 6144, 4096),
@@ -177,10 +177,10 @@ def main():
                 "tflops": tot_fl / (tot_ms * 1e-3) / 1e12, "total_ms": tot_ms,
             }
         dom = max(kinds, key=lambda k: kinds[k]["total_ms"])
-        # template arguments: <A contraction-contiguous, B contraction-contiguous, epilogue, fp32 out>
-        kernel_names = {"fwd": "gemm_bf16_solo_kernel<true, true, 0, false> (Y = X W^T)",
-                        "dgrad": "gemm_bf16_solo_kernel<true, false, 0, false> (dX = dY W)",
-                        "wgrad": "gemm_bf16_solo_kernel<false, false, 0, false> (dW = dY^T X)"}
+        # template arguments: <tile, A contraction-contiguous, B contraction-contiguous, epilogue, fp32 out>
+        kernel_names = {"fwd": "gemm_bf16_solo_kernel<256, true, true, 0, false> (Y = X W^T)",
+                        "dgrad": "gemm_bf16_solo_kernel<256, true, false, 0, false> (dX = dY W)",
+                        "wgrad": "gemm_bf16_solo_kernel<256, false, false, 0, false> (dW = dY^T X)"}
         roofline = {
             "bound": "mfma", "kernel": kernel_names[dom],
             "achieved": round(kinds[dom]["tflops"], 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
