@@ -14,8 +14,9 @@
 // Workgroup b finds its tensor by binary search in that prefix sum (scalar
 // loads from the argument block) and owns one chunk of consecutive elements of it.
 // Tensors are views into flat buffers at arbitrary element offsets
-// (axonn/utils.py:11-30), so each tensor starts with a scalar "head" of up to 7
-// elements after which every pointer of the tensor is 16-byte aligned; the
+// (axonn/utils.py:11-30), so each tensor starts with a scalar "head" of up to 63
+// elements after which every pointer of the tensor is 16-byte aligned (and on a
+// cache line when the buffers allow it); the
 // body is then moved as 16-byte vectors, 8 elements per lane per step.  A
 // tensor whose pointers cannot be aligned by one common head is processed with
 // scalar accesses.
@@ -505,6 +506,17 @@ int common_head(const void* const* ptrs, const int* elem_sizes, int count) {
     if (ptrs[i] == nullptr) continue;
     const uintptr_t a = (uintptr_t)ptrs[i] + (uintptr_t)best * elem_sizes[i];
     if (a % 16 != 0) return -1;
+  }
+  // Prefer a head after which every pointer sits on a 128-byte cache line, so that
+  // the chunks of different workgroups do not share lines (views at one common
+  // element offset into line-aligned flat buffers always have one, of at most 63
+  // elements).  Steps of 8 elements keep the 16-byte alignment found above.
+  for (int h = best; h < 64; h += 8) {
+    bool all = true;
+    for (int i = 0; i < count && all; ++i)
+      if (ptrs[i] != nullptr)
+        all = ((uintptr_t)ptrs[i] + (uintptr_t)h * elem_sizes[i]) % 128 == 0;
+    if (all) return h;
   }
   return best;
 }
