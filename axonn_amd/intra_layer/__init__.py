@@ -9,6 +9,7 @@ from .fully_connected import Linear, AsyncLinear, FusedLinear  # noqa: F401
 from .communication import Drop, Gather  # noqa: F401
 from .gradient_normalization import clip_grad_norm_  # noqa: F401
 from .overlap_communication import optimize_communication  # noqa: F401
+from .automatic_parallelism import auto_parallelize  # noqa: F401
 from .overlap_communication import (  # noqa: F401
     overlap_all_gathers_for_checkpointed_forward,
 )

@@ -164,3 +164,35 @@ def test_package_exports():
     from axonn_amd.intra_layer import AsyncLinear, Drop, Gather, no_grad_sync, sync_gradients  # noqa: F401
 
     assert axonn_amd.config.G_intra == 1
+
+
+def test_auto_parallelize_swaps_nn_linear_inside_the_context_only():
+    import torch.nn as nn
+
+    import axonn_amd.axonn as ax
+    from axonn_amd.intra_layer import Linear, auto_parallelize
+    from axonn_amd.intra_layer.automatic_parallelism import is_parallelizable_linear
+
+    ax.init(1, 1, 1, 1)
+    original = nn.Linear
+    with auto_parallelize():
+        a = nn.Linear(16, 24)
+        b = nn.Linear(16, 8, bias=False, dtype=torch.bfloat16)
+
+        class Net(nn.Module):            # a model declared inside picks the layer up unchanged
+            def __init__(self):
+                super().__init__()
+                self.fc = nn.Linear(8, 8)
+
+        net = Net()
+    assert nn.Linear is original and isinstance(nn.Linear(4, 4), original)
+    assert isinstance(a, Linear) and a.weight.shape == (16 * 24,) and a.bias is not None
+    assert isinstance(b, Linear) and b.bias is None and b.weight.dtype == torch.bfloat16
+    assert isinstance(net.fc, Linear)
+    assert is_parallelizable_linear(16, 24)
+    try:
+        with auto_parallelize():
+            raise RuntimeError("boom")
+    except RuntimeError:
+        pass
+    assert nn.Linear is original     # restored on error as well

@@ -138,3 +138,62 @@ def test_patched_attention_projections_are_linear_layers():
         lin = getattr(attn, name)
         assert isinstance(lin, Linear) and lin.weight.numel() == shape[0] * shape[1]
     assert not isinstance(LlamaAttention(cfg, 0).q_proj, Linear)
+
+
+def test_tiny_llama_model_under_parallelize_matches_its_torch_twin():
+    """A 2-layer LlamaForCausalLM built inside `parallelize` (all 7 projections of
+    each layer on the GEMM kernels, the fused SwiGLU in the MLP) against the same
+    model built from torch.nn.Linear with the same weights: logits, loss and the
+    gradients of every projection, bf16 on the GPU, normwise 2e-2 (two models in
+    bf16 differ by rounding in every layer; the oracle-level bar is applied to the
+    block in the test above)."""
+    from transformers import LlamaConfig, LlamaForCausalLM
+
+    import axonn_amd.axonn as ax
+    from axonn_amd.intra_layer import Linear
+    from axonn_amd.models.transformers import parallelize
+
+    ax.init(1, 1, 1, 1)
+    cfg = LlamaConfig(hidden_size=256, intermediate_size=512, num_attention_heads=4, num_key_value_heads=2,
+                      num_hidden_layers=2, vocab_size=128, max_position_embeddings=64,
+                      architectures=["LlamaForCausalLM"])
+    cfg._attn_implementation = "eager"
+    torch.manual_seed(0)
+    ref = LlamaForCausalLM(cfg)
+    with parallelize(cfg):
+        ours = LlamaForCausalLM(cfg)
+    n_lin = sum(isinstance(m, Linear) for m in ours.modules())
+    assert n_lin == 2 * 7
+    missing = ours.load_state_dict(ref.state_dict(), strict=True)   # 2-D weights into the flat parameters
+    assert not missing.missing_keys and not missing.unexpected_keys
+    ref, ours = ref.cuda().bfloat16(), ours.cuda().bfloat16()
+    ids = torch.randint(0, 128, (4, 32), generator=torch.Generator().manual_seed(1)).cuda()
+    out_r = ref(input_ids=ids, labels=ids)
+    out_o = ours(input_ids=ids, labels=ids)
+    assert rel(np64(out_o.logits), np64(out_r.logits)) < 2e-2
+    assert abs(out_o.loss.item() - out_r.loss.item()) < 2e-2 * abs(out_r.loss.item())
+    out_r.loss.backward()
+    out_o.loss.backward()
+    for (name, p_r), (_, p_o) in zip(ref.named_parameters(), ours.named_parameters()):
+        assert rel(np64(p_o.grad).reshape(-1), np64(p_r.grad).reshape(-1)) < 5e-2, name
+
+
+def test_auto_parallelize_builds_hugging_face_mlp_on_the_kernels():
+    from transformers import LlamaConfig
+    from transformers.models.llama.modeling_llama import LlamaMLP
+
+    import axonn_amd.axonn as ax
+    from axonn_amd.intra_layer import Linear, auto_parallelize
+
+    ax.init(1, 1, 1, 1)
+    cfg = LlamaConfig(hidden_size=128, intermediate_size=256, num_attention_heads=4, num_key_value_heads=2,
+                      num_hidden_layers=1, vocab_size=32)
+    with auto_parallelize():
+        mlp = LlamaMLP(cfg)
+    assert all(isinstance(getattr(mlp, n), Linear) for n in ("gate_proj", "up_proj", "down_proj"))
+    mlp = mlp.cuda().bfloat16()
+    x = torch.randn(64, 128, generator=torch.Generator().manual_seed(2)).cuda().bfloat16()
+    y = mlp(x)
+    wg, wu, wd = (np64(p).reshape(-1) for p in (mlp.gate_proj.weight, mlp.up_proj.weight, mlp.down_proj.weight))
+    fwd = om.llama_mlp_forward(np64(x), wg, wu, wd, 128, 256, store="bf16")
+    assert rel(np64(y), fwd["out"]) < 1e-2
