@@ -348,3 +348,28 @@ def test_full_size_shapes_sampled_oracle_and_properties(name):
     # (d) determinism: the same call gives the same bits
     y3, _ = ops.gemm_fwd(X, W)
     assert torch.equal(y3, y)
+
+
+def test_operand_of_two_gibibytes_takes_the_64_bit_path():
+    """The tile kernels address an operand with 32-bit byte offsets; an operand of
+    2 GiB or more must go to the kernel with 64-bit addressing and still be right
+    in its last rows."""
+    from axonn_amd import ops
+
+    M, K, N = 32768, 32768, 256          # X is exactly 2^31 bytes
+    g = torch.Generator(device="cuda").manual_seed(5)
+    X = torch.empty(M, K, dtype=torch.bfloat16, device="cuda")
+    for r in range(0, M, 4096):          # filled in slabs: no 4 GiB fp32 temporary
+        X[r:r + 4096] = torch.randn(4096, K, generator=g, device="cuda").bfloat16()
+    W = (torch.randn(N, K, generator=g, device="cuda") * 0.02).bfloat16()
+    y, _ = ops.gemm_fwd(X, W)
+    rows = torch.cat([torch.arange(0, 64), torch.arange(M // 2 - 32, M // 2 + 32), torch.arange(M - 64, M)]).cuda()
+    ref = X[rows].float() @ W.float().t()
+    assert rel(np64(y[rows]), np64(ref)) < BF16_TOL
+    dY = torch.randn(M, N, generator=g, device="cuda").bfloat16()
+    dw = ops.gemm_wgrad(dY, X, out_dtype=torch.float32)       # X as the 2 GiB contraction-strided operand
+    cols = torch.arange(K - 128, K, device="cuda")
+    refw = dY.float().t() @ X[:, cols].float()
+    assert rel(np64(dw[:, cols]), np64(refw)) < 1e-4
+    del X
+    torch.cuda.empty_cache()
