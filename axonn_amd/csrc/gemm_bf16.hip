@@ -20,8 +20,8 @@
 //   * Workgroup ids are remapped so that each of the 8 XCDs (private L2 each)
 //     works on a compact block of neighbouring tiles.
 //
-// gemm_bf16_solo_kernel (whole 256 x 256 tiles, contraction % 64 == 0, at least
-// 192 tiles): 4 waves, one per SIMD, 128 x 128 per wave on v_mfma_f32_16x16x32_bf16;
+// gemm_bf16_solo_kernel (whole 256 x 256 tiles, contraction % 64 == 0, more than
+// 128 tiles): 4 waves, one per SIMD, 128 x 128 per wave on v_mfma_f32_16x16x32_bf16;
 // operand tiles go global -> LDS directly (buffer loads to LDS, 16 bytes per
 // lane, no registers) into a ring of five 64-deep tiles; each wave pipelines its
 // LDS fragment reads and its share of the copies between its own MFMAs.
@@ -739,8 +739,8 @@ int launch_solo(const GemmArgs& in, hipStream_t stream) {
   return AXN_OK;
 }
 
-// Kernel selection.  Problems made of whole 256 x 256 tiles, at least 192 of
-// them (3/4 of the CUs), take the one-wave-per-SIMD kernel at that tile size;
+// Kernel selection.  Problems made of whole 256 x 256 tiles, more than 128 of
+// them (half of the CUs), take the one-wave-per-SIMD kernel at that tile size;
 // other problems made of whole 128 x 128 tiles take it at 128 x 128; ragged
 // shapes, and operands too large for 32-bit byte offsets, take the
 // register-staged kernel.
@@ -755,7 +755,9 @@ int launch_shape(const GemmArgs& g, hipStream_t stream) {
   const int64_t a_span = (int64_t)(AK ? g.M : g.Kc) * g.lda * 2;
   const int64_t b_span = (int64_t)(BKM ? g.N : g.Kc) * g.ldb * 2;
   const bool small_spans = a_span < (1LL << 31) && b_span < (1LL << 31);
-  if (small_spans && whole256 && tiles256 >= 192)
+  // Up to 128 large tiles the small tile wins: four times as many workgroups, two per CU, still
+  // fit in one round.  Beyond that its second round costs more than the idle CUs of the large one.
+  if (small_spans && whole256 && tiles256 > 128)
     return launch_solo<256, AK, BKM, EPI, OUT_F32>(g, stream);
   if (small_spans && whole128 && tiles128 < (1LL << 31))
     return launch_solo<128, AK, BKM, EPI, OUT_F32>(g, stream);

@@ -222,7 +222,7 @@ def test_fp32_gemms_match_oracle(M, N, K):
 @pytest.mark.parametrize("M,N,K", [(128, 128, 64), (256, 384, 192), (512, 256, 320), (4096, 3072, 128),
                                    (4096, 3072, 320)])
 def test_tile_kernels_every_output_block_with_epilogues(M, N, K):
-    """Whole-tile shapes on the one-wave-per-SIMD kernel (128 x 128 tiles below 192
+    """Whole-tile shapes on the one-wave-per-SIMD kernel (128 x 128 tiles up to 128
     tiles of 256 x 256, else 256 x 256), checked element by element so that a single
     wrong 16 x 16 accumulator block shows (a block copied out of its registers before
     its last MFMA had finished once passed the normwise checks of other shapes)."""
@@ -258,7 +258,7 @@ def test_tile_kernels_every_output_block_with_epilogues(M, N, K):
 # ---- the 256 x 256-tile kernel: few and many contraction stages, all layouts/epilogues ----
 @pytest.mark.parametrize("K", [64, 128, 192, 256, 448])
 def test_tile256_kernel_short_contractions(K):
-    """Shapes of >= 192 whole 256 x 256 tiles take the one-wave-per-SIMD kernel; it
+    """Shapes of more than 128 whole 256 x 256 tiles take the one-wave-per-SIMD kernel; it
     walks the contraction in stages of 64 and copies two stages ahead, so K = 64 and
     128 exercise the start-up and drain paths alone (1 and 2 stages), 192 and 256 a
     single or two steady-state stages, and 448 the steady state proper."""
