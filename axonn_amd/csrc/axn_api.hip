@@ -237,6 +237,93 @@ int axn_swiglu_bwd(const void* dout, const void* gate, const void* up, void* dga
   return launch_swiglu_bwd(dout, gate, up, dgate, dup, dtype, M, N, ld, (hipStream_t)stream);
 }
 
+static int elem_bytes_of(int dtype) { return dtype == AXN_F32 ? 4 : 2; }
+
+static int check_embedding(const char* name, int64_t T, int64_t V, int64_t H) {
+  REQUIRE(T >= 0 && V >= 1 && H >= 1, AXN_EINVAL, "%s: T must be >= 0, V and H >= 1", name);
+  REQUIRE(T < (1LL << 31) && V < (1LL << 31) - 1, AXN_ELIMIT,
+          "%s: T and V must be below 2^31", name);
+  return AXN_OK;
+}
+
+static int check_rows16(const char* name, const char* what, int dtype, int64_t H, int64_t ld) {
+  const int per = 16 / elem_bytes_of(dtype);
+  REQUIRE(H % per == 0, AXN_ESHAPE, "%s: H must be a multiple of %d for %s", name, per, what);
+  REQUIRE(ld >= H && ld % per == 0, AXN_EALIGN, "%s: ld of %s must be >= H and a multiple of %d",
+          name, what, per);
+  return AXN_OK;
+}
+
+int axn_embedding_fwd(const int64_t* ids, const void* W, void* out, int dtype, int64_t T,
+                      int64_t V, int64_t H, int64_t ldw, int64_t ldo, int32_t* status,
+                      void* stream) {
+  const char* name = "axn_embedding_fwd";
+  REQUIRE(W && ((ids && out) || T == 0), AXN_EINVAL, "%s: null pointer", name);
+  REQUIRE(dtype == AXN_BF16 || dtype == AXN_F16 || dtype == AXN_F32, AXN_EINVAL,
+          "%s: unknown dtype %d", name, dtype);
+  int rc = check_embedding(name, T, V, H);
+  if (rc) return rc;
+  if ((rc = check_rows16(name, "W", dtype, H, ldw))) return rc;
+  if ((rc = check_rows16(name, "out", dtype, H, ldo))) return rc;
+  REQUIRE(aligned16(W) && aligned16(out), AXN_EALIGN, "%s: pointers must be 16-byte aligned", name);
+  if (T == 0) return AXN_OK;
+  return launch_embedding_fwd(ids, W, out, elem_bytes_of(dtype), T, V, H, ldw, ldo, (int*)status,
+                              (hipStream_t)stream);
+}
+
+size_t axn_embedding_workspace_bytes(int64_t T, int64_t V) {
+  return embedding_workspace_bytes(T, V);
+}
+
+int axn_embedding_bwd(const int64_t* ids, const void* dY, void* dW, int dy_dtype, int dw_dtype,
+                      int64_t T, int64_t V, int64_t H, int64_t lddy, int64_t lddw,
+                      int64_t padding_idx, int scale_grad_by_freq, int beta, void* workspace,
+                      size_t workspace_bytes, void* stream) {
+  const char* name = "axn_embedding_bwd";
+  REQUIRE(dW && ((ids && dY) || T == 0), AXN_EINVAL, "%s: null pointer", name);
+  REQUIRE((dy_dtype == AXN_BF16 || dy_dtype == AXN_F32) &&
+              (dw_dtype == AXN_BF16 || dw_dtype == AXN_F32),
+          AXN_EINVAL, "%s: dtypes must be bf16 or fp32", name);
+  int rc = check_embedding(name, T, V, H);
+  if (rc) return rc;
+  if ((rc = check_rows16(name, "dY", dy_dtype, H, lddy))) return rc;
+  if ((rc = check_rows16(name, "dW", dw_dtype, H, lddw))) return rc;
+  REQUIRE(padding_idx >= -1 && padding_idx < V, AXN_EINVAL,
+          "%s: padding_idx must be -1 or a row of the table", name);
+  REQUIRE(beta == 0 || beta == 1, AXN_EINVAL, "%s: beta must be 0 or 1", name);
+  REQUIRE((T == 0 || aligned16(dY)) && aligned16(dW), AXN_EALIGN,
+          "%s: pointers must be 16-byte aligned", name);
+  REQUIRE(workspace != nullptr && workspace_bytes >= embedding_workspace_bytes(T, V), AXN_EINVAL,
+          "%s: workspace too small (%zu bytes given, %zu needed)", name, workspace_bytes,
+          embedding_workspace_bytes(T, V));
+  REQUIRE(aligned16(workspace), AXN_EALIGN, "%s: workspace must be 16-byte aligned", name);
+  return launch_embedding_bwd(ids, dY, dW, dy_dtype, dw_dtype, T, V, H, lddy, lddw, padding_idx,
+                              scale_grad_by_freq != 0, beta, workspace, workspace_bytes,
+                              (hipStream_t)stream);
+}
+
+int axn_embedding_renorm(const int64_t* ids, void* W, int dtype, int64_t T, int64_t V, int64_t H,
+                         int64_t ldw, float max_norm, float norm_type, void* workspace,
+                         size_t workspace_bytes, void* stream) {
+  const char* name = "axn_embedding_renorm";
+  REQUIRE(W && (ids || T == 0), AXN_EINVAL, "%s: null pointer", name);
+  REQUIRE(dtype == AXN_BF16 || dtype == AXN_F32, AXN_EINVAL, "%s: dtype must be bf16 or fp32",
+          name);
+  int rc = check_embedding(name, T, V, H);
+  if (rc) return rc;
+  if ((rc = check_rows16(name, "W", dtype, H, ldw))) return rc;
+  REQUIRE(max_norm > 0.0f && norm_type > 0.0f, AXN_EINVAL,
+          "%s: max_norm and norm_type must be positive", name);
+  REQUIRE(aligned16(W), AXN_EALIGN, "%s: pointers must be 16-byte aligned", name);
+  REQUIRE(workspace != nullptr && workspace_bytes >= embedding_workspace_bytes(T, V), AXN_EINVAL,
+          "%s: workspace too small (%zu bytes given, %zu needed)", name, workspace_bytes,
+          embedding_workspace_bytes(T, V));
+  REQUIRE(aligned16(workspace), AXN_EALIGN, "%s: workspace must be 16-byte aligned", name);
+  if (T == 0) return AXN_OK;
+  return launch_embedding_renorm(ids, W, dtype, T, V, H, ldw, max_norm, norm_type, workspace,
+                                 workspace_bytes, (hipStream_t)stream);
+}
+
 int axn_gemm_fwd_f32(const float* X, const float* W, const float* bias, float* Y,
                      float* Zsave, int64_t M, int64_t N, int64_t K, int epilogue,
                      void* stream) {

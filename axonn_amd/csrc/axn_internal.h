@@ -94,6 +94,19 @@ int launch_swiglu_fwd(const void* gate, const void* up, void* out, int dtype, in
 int launch_swiglu_bwd(const void* dout, const void* gate, const void* up, void* dgate, void* dup,
                       int dtype, int64_t M, int64_t N, int64_t ld, hipStream_t stream);
 
+// ---- embedding table: row gather, dense weight gradient, max_norm -------------------
+size_t embedding_workspace_bytes(int64_t T, int64_t V);
+int launch_embedding_fwd(const int64_t* ids, const void* W, void* out, int elem_bytes, int64_t T,
+                         int64_t V, int64_t H, int64_t ldw, int64_t ldo, int* status,
+                         hipStream_t stream);
+int launch_embedding_bwd(const int64_t* ids, const void* dY, void* dW, int dy_dtype, int dw_dtype,
+                         int64_t T, int64_t V, int64_t H, int64_t lddy, int64_t lddw,
+                         int64_t padding_idx, int scale_by_freq, int beta, void* ws,
+                         size_t ws_bytes, hipStream_t stream);
+int launch_embedding_renorm(const int64_t* ids, void* W, int dtype, int64_t T, int64_t V,
+                            int64_t H, int64_t ldw, float max_norm, float norm_type, void* ws,
+                            size_t ws_bytes, hipStream_t stream);
+
 // ---- multi-tensor optimizer ------------------------------------------------
 size_t mt_scan_workspace_bytes(int64_t n, int64_t total);
 int launch_mt_scan(const void* const* h_g, const int64_t* h_sizes, int64_t n,

@@ -18,7 +18,7 @@ LIB_DIR = os.path.join(os.path.dirname(HERE), "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libaxn_gfx950.so")
 OBJ_DIR = os.path.join(HERE, "build")
 
-SOURCES = ["axn_api.hip", "gemm_bf16.hip", "gemm_f32.hip", "elementwise.hip", "optim.hip"]
+SOURCES = ["axn_api.hip", "gemm_bf16.hip", "gemm_f32.hip", "elementwise.hip", "embedding.hip", "optim.hip"]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 

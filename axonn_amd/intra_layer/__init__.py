@@ -6,6 +6,7 @@ from contextlib import contextmanager
 import torch
 
 from .fully_connected import Linear, AsyncLinear, FusedLinear  # noqa: F401
+from .embedding import Embedding  # noqa: F401
 from .communication import Drop, Gather  # noqa: F401
 from .gradient_normalization import clip_grad_norm_  # noqa: F401
 from .overlap_communication import optimize_communication  # noqa: F401

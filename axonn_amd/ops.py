@@ -226,6 +226,92 @@ def swiglu_bwd(dout, gate, up):
     return dgate, dup
 
 
+# ------------------------------------------------------------- embedding -----
+def _embedding_table(name, w):
+    if w.dim() != 2:
+        raise ValueError("%s: 2-D table expected, got %s" % (name, tuple(w.shape)))
+    per = 16 // w.element_size()
+    if w.shape[1] % per:
+        raise ValueError("%s: embedding width must be a multiple of %d for %s, got %d"
+                         % (name, per, w.dtype, w.shape[1]))
+    if w.stride(1) != 1 or w.stride(0) % per or w.data_ptr() % 16:
+        raise ValueError("%s: rows must be contiguous and 16-byte aligned" % name)
+
+
+def _embedding_ids(ids):
+    if ids.dtype not in (torch.int64, torch.int32):
+        raise TypeError("embedding: int64 or int32 indices expected, got %s" % ids.dtype)
+    return ids.reshape(-1).to(torch.int64).contiguous()
+
+
+def _embedding_workspace(T, V, device):
+    nbytes = nv.load().axn_embedding_workspace_bytes(T, V)
+    return torch.empty(nbytes, dtype=torch.uint8, device=device), nbytes
+
+
+def embedding_fwd(ids, weight, status=None):
+    """weight[ids]: rows of the table gathered into ids.shape + (H,).  `status`, a
+    device int32 scalar, is set to 1 if an id lies outside the table (such a token
+    reads as zeros)."""
+    _require_gpu(ids, weight)
+    _embedding_table("embedding_fwd", weight)
+    flat = _embedding_ids(ids)
+    V, H = weight.shape
+    out = torch.empty((flat.numel(), H), dtype=weight.dtype, device=weight.device)
+    nv.call("axn_embedding_fwd", nv.ptr(flat), nv.ptr(weight), nv.ptr(out),
+            nv.dtype_code(weight.dtype), flat.numel(), V, H, weight.stride(0), H,
+            nv.ptr(status) if status is not None else None, nv.current_stream())
+    return out.view(*ids.shape, H)
+
+
+def embedding_bwd(ids, dy, num_embeddings, padding_idx=None, scale_grad_by_freq=False, out=None,
+                  accumulate=False, out_dtype=None):
+    """Dense gradient of the table: row v receives the sum of the dy rows of the tokens
+    with id v, added in token order (deterministic).  With `out` and accumulate=True the
+    sum is added to out."""
+    _require_gpu(ids, dy)
+    flat = _embedding_ids(ids)
+    H = dy.shape[-1]
+    dy2 = dy.reshape(-1, H)
+    if dy2.dtype not in (torch.bfloat16, torch.float32):
+        raise TypeError("embedding_bwd: bf16 or fp32 gradient expected, got %s" % dy2.dtype)
+    if dy2.shape[0] != flat.numel():
+        raise ValueError("embedding_bwd: %d tokens but %d gradient rows"
+                         % (flat.numel(), dy2.shape[0]))
+    if dy2.stride(1) != 1 or dy2.stride(0) != H or dy2.data_ptr() % 16:
+        dy2 = dy2.contiguous().clone()
+    if out is None:
+        if accumulate:
+            raise ValueError("embedding_bwd: accumulate needs out")
+        out = torch.empty((num_embeddings, H), dtype=out_dtype or dy2.dtype, device=dy2.device)
+    _embedding_table("embedding_bwd", out)
+    if tuple(out.shape) != (num_embeddings, H):
+        raise ValueError("embedding_bwd: out is %s, expected %s"
+                         % (tuple(out.shape), (num_embeddings, H)))
+    ws, nbytes = _embedding_workspace(flat.numel(), num_embeddings, dy2.device)
+    nv.call("axn_embedding_bwd", nv.ptr(flat), nv.ptr(dy2), nv.ptr(out), nv.dtype_code(dy2.dtype),
+            nv.dtype_code(out.dtype), flat.numel(), num_embeddings, H, H, out.stride(0),
+            -1 if padding_idx is None else padding_idx, int(bool(scale_grad_by_freq)),
+            int(bool(accumulate)), nv.ptr(ws), nbytes, nv.current_stream())
+    return out
+
+
+def embedding_renorm_(weight, ids, max_norm, norm_type=2.0):
+    """In place: every row of the table that ids names and whose norm exceeds max_norm is
+    scaled to max_norm (torch.embedding_renorm_)."""
+    _require_gpu(ids, weight)
+    _embedding_table("embedding_renorm_", weight)
+    if weight.dtype not in (torch.bfloat16, torch.float32):
+        raise TypeError("embedding_renorm_: bf16 or fp32 table expected, got %s" % weight.dtype)
+    flat = _embedding_ids(ids)
+    V, H = weight.shape
+    ws, nbytes = _embedding_workspace(flat.numel(), V, weight.device)
+    nv.call("axn_embedding_renorm", nv.ptr(flat), nv.ptr(weight), nv.dtype_code(weight.dtype),
+            flat.numel(), V, H, weight.stride(0), float(max_norm), float(norm_type), nv.ptr(ws),
+            nbytes, nv.current_stream())
+    return weight
+
+
 # ---------------------------------------------------------- multi-tensor -----
 class ScanResult:
     """Device-resident axn_scan_result (32 bytes) with typed views."""

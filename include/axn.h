@@ -30,7 +30,7 @@
 extern "C" {
 #endif
 
-#define AXN_ABI_VERSION 2
+#define AXN_ABI_VERSION 3
 
 #if defined(__GNUC__)
 #define AXN_API __attribute__((visibility("default")))
@@ -134,6 +134,51 @@ AXN_API int axn_swiglu_fwd(const void* gate, const void* up, void* out, int dtyp
 AXN_API int axn_swiglu_bwd(const void* dout, const void* gate, const void* up,
                    void* dgate, void* dup, int dtype, int64_t M, int64_t N,
                    int64_t ld, void* stream);
+
+/* ------------------------------------------------------------------------
+ * Embedding table.  T = tokens, V = rows of the (local) table, H = (local)
+ * embedding width.  ids are int64 as torch hands them over.  Rows are moved
+ * in 16-byte vectors: H and every ld a multiple of 16 / sizeof(element)
+ * (4 for fp32, 8 for bf16), pointers 16-byte aligned.  T may be 0.
+ * T < 2^31, V < 2^31 - 1.
+ * ------------------------------------------------------------------------ */
+
+/* Forward.  Replaces the gather of `F.embedding(x, weight, ...)`
+ * (axonn/intra_layer/embedding.py:164-172): out[t, :] = W[ids[t], :].
+ * W [V,H] and out [T,H] of `dtype` (any axn_dtype; rows are copied verbatim).
+ * torch raises a device-side assertion for an id outside [0, V); here such a
+ * token reads as a row of zeros and, if `status` (device int32, may be NULL) is
+ * given, *status is set to 1 - it is never cleared by the call. */
+AXN_API int axn_embedding_fwd(const int64_t* ids, const void* W, void* out, int dtype,
+                      int64_t T, int64_t V, int64_t H, int64_t ldw, int64_t ldo,
+                      int32_t* status, void* stream);
+
+/* Workspace of the two entry points below (token positions sorted by id). */
+AXN_API size_t axn_embedding_workspace_bytes(int64_t T, int64_t V);
+
+/* Backward.  Replaces the autograd of the same F.embedding call
+ * (torch's embedding_dense_backward; sparse gradients are not supported):
+ *   dW[v, :] = beta * dW[v, :] + sum_{t : ids[t] == v} s_v * dY[t, :]
+ * with s_v = 1, or 1 / #{t : ids[t] == v} when scale_grad_by_freq is set;
+ * row `padding_idx` (-1: none) receives no gradient.  beta = 0 writes every
+ * row of dW (zeros where no token points), so dW needs no clearing.
+ * dY [T,H] of dy_dtype, dW [V,H] of dw_dtype (each AXN_BF16 or AXN_F32).
+ * Terms are added in fp32 in ascending token order: the result is
+ * deterministic and equals a sequential loop over the tokens.  Ids outside
+ * [0, V) are skipped. */
+AXN_API int axn_embedding_bwd(const int64_t* ids, const void* dY, void* dW, int dy_dtype,
+                      int dw_dtype, int64_t T, int64_t V, int64_t H, int64_t lddy,
+                      int64_t lddw, int64_t padding_idx, int scale_grad_by_freq,
+                      int beta, void* workspace, size_t workspace_bytes, void* stream);
+
+/* max_norm of F.embedding (torch.embedding_renorm_, applied to the table in
+ * place before the lookup): every row named by at least one id whose
+ * norm_type-norm exceeds max_norm is scaled by max_norm / (norm + 1e-7).
+ * W [V,H] of dtype AXN_BF16 or AXN_F32; max_norm > 0, norm_type > 0. */
+AXN_API int axn_embedding_renorm(const int64_t* ids, void* W, int dtype, int64_t T,
+                         int64_t V, int64_t H, int64_t ldw, float max_norm,
+                         float norm_type, void* workspace, size_t workspace_bytes,
+                         void* stream);
 
 /* fp32 variants of the three GEMMs for full-precision layers (the reference's
  * own tests run the layer in fp32: axonn/tests/test_intra_layer_fc.py:25).

@@ -42,6 +42,12 @@ def test_workspace_queries():
     assert lib.axn_mt_scan_workspace_bytes(-1, 5) == 0
     assert lib.axn_dgelu_dbias_workspace_bytes(8192, 5120) == 64 * 5120 * 4
     assert lib.axn_dgelu_dbias_workspace_bytes(0, 8) == 0
+    # embedding: four int32 arrays over the tokens, one over the rows, the sort's own storage
+    T, V = 16384, 128256
+    need = lib.axn_embedding_workspace_bytes(T, V)
+    assert 4 * T * 4 + V * 4 + 16 * T <= need <= 4 * T * 4 + V * 4 + 16 * T + (8 << 20)
+    assert lib.axn_embedding_workspace_bytes(0, V) >= V * 4
+    assert lib.axn_embedding_workspace_bytes(T, 0) == 0 and lib.axn_embedding_workspace_bytes(-1, V) == 0
 
 
 def _err():
@@ -85,6 +91,37 @@ def test_swiglu_argument_errors():
     assert b(A, A, A, A, None, nv.BF16, 8, 8, 8, None) == nv.AXN_EINVAL
     assert b(A, A, A, A, A, nv.F32, 0, 8, 8, None) == nv.AXN_EINVAL
     assert "axn_swiglu_bwd" in _err()
+
+
+def test_embedding_argument_errors():
+    lib = nv.load()
+    f, b, r = lib.axn_embedding_fwd, lib.axn_embedding_bwd, lib.axn_embedding_renorm
+    big = 1 << 30
+    assert f(A, None, A, nv.F32, 4, 16, 8, 8, 8, None, None) == nv.AXN_EINVAL
+    assert f(None, A, A, nv.F32, 4, 16, 8, 8, 8, None, None) == nv.AXN_EINVAL  # ids missing
+    assert f(A, A, A, 7, 4, 16, 8, 8, 8, None, None) == nv.AXN_EINVAL
+    assert f(A, A, A, nv.F32, -1, 16, 8, 8, 8, None, None) == nv.AXN_EINVAL
+    assert f(A, A, A, nv.F32, 4, 16, 6, 8, 8, None, None) == nv.AXN_ESHAPE      # fp32 rows of 24 bytes
+    assert f(A, A, A, nv.BF16, 4, 16, 12, 16, 16, None, None) == nv.AXN_ESHAPE  # bf16 rows of 24 bytes
+    assert f(A, A, A, nv.F32, 4, 16, 8, 4, 8, None, None) == nv.AXN_EALIGN      # ldw < H
+    assert f(A, A, A, nv.F32, 4, 16, 8, 8, 10, None, None) == nv.AXN_EALIGN
+    assert f(A, ctypes.c_void_p(0x1004), A, nv.F32, 4, 16, 8, 8, 8, None, None) == nv.AXN_EALIGN
+    assert f(A, A, A, nv.F32, 1 << 31, 16, 8, 8, 8, None, None) == nv.AXN_ELIMIT
+    assert "axn_embedding_fwd" in _err()
+    assert b(A, A, None, nv.F32, nv.F32, 4, 16, 8, 8, 8, -1, 0, 0, A, big, None) == nv.AXN_EINVAL
+    assert b(A, A, A, nv.F16, nv.F32, 4, 16, 8, 8, 8, -1, 0, 0, A, big, None) == nv.AXN_EINVAL
+    assert b(A, A, A, nv.BF16, nv.F32, 4, 16, 12, 16, 12, -1, 0, 0, A, big, None) == nv.AXN_ESHAPE
+    assert b(A, A, A, nv.F32, nv.F32, 4, 16, 8, 8, 8, 16, 0, 0, A, big, None) == nv.AXN_EINVAL  # padding row
+    assert b(A, A, A, nv.F32, nv.F32, 4, 16, 8, 8, 8, -2, 0, 0, A, big, None) == nv.AXN_EINVAL
+    assert b(A, A, A, nv.F32, nv.F32, 4, 16, 8, 8, 8, -1, 0, 2, A, big, None) == nv.AXN_EINVAL  # beta
+    assert b(A, A, A, nv.F32, nv.F32, 4, 16, 8, 8, 8, -1, 0, 0, A, 64, None) == nv.AXN_EINVAL
+    assert "workspace" in _err()
+    assert b(A, A, A, nv.F32, nv.F32, 4, 16, 8, 8, 8, -1, 0, 0, None, big, None) == nv.AXN_EINVAL
+    assert r(A, None, nv.F32, 4, 16, 8, 8, 1.0, 2.0, A, big, None) == nv.AXN_EINVAL
+    assert r(A, A, nv.F16, 4, 16, 8, 8, 1.0, 2.0, A, big, None) == nv.AXN_EINVAL
+    assert r(A, A, nv.F32, 4, 16, 8, 8, 0.0, 2.0, A, big, None) == nv.AXN_EINVAL
+    assert r(A, A, nv.F32, 4, 16, 8, 8, 1.0, -1.0, A, big, None) == nv.AXN_EINVAL
+    assert r(A, A, nv.F32, 4, 16, 8, 8, 1.0, 2.0, A, 16, None) == nv.AXN_EINVAL
 
 
 def test_elementwise_argument_errors():

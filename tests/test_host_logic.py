@@ -196,3 +196,58 @@ def test_auto_parallelize_swaps_nn_linear_inside_the_context_only():
     except RuntimeError:
         pass
     assert nn.Linear is original     # restored on error as well
+
+
+def test_embedding_parameters_state_dict_and_no_cpu_fallback():
+    """The reference's layout: a flat [V * H] weight, tags for gradient sync and clipping,
+    a loader that takes torch.nn.Embedding's 2-D weight or its own 1-D shard
+    (axonn/intra_layer/embedding.py:139-148, :191-222; its test loads both ways,
+    axonn/tests/test_intra_layer_emb.py:46-49)."""
+    from axonn_amd.intra_layer import Embedding
+
+    torch.manual_seed(2)
+    V, H = 50, 16
+    layer = Embedding(V, H, padding_idx=-3)
+    assert layer.weight.shape == (V * H,) and layer.weight.is_tensor_parallel
+    assert layer.weight.needs_depth_parallel_gradient_sync is False
+    assert layer.padding_idx == V - 3 and layer.get_output_feature_size() == H
+    table = layer.weight.detach().view(V, H)
+    assert not table[V - 3].any() and table[0].any() and table[V - 2].any()
+    assert abs(float(table.std()) - 1.0) < 0.1  # normal(0, 1) default
+    ref = torch.nn.Embedding(V, H)
+    layer.load_state_dict(ref.state_dict())
+    assert torch.equal(layer.weight.view(V, H), ref.weight)
+    layer.load_state_dict(layer.state_dict())
+    assert torch.equal(layer.weight.view(V, H), ref.weight)
+    with pytest.raises(AssertionError, match="neither a full checkpoint nor a sharded"):
+        layer.load_state_dict({"weight": torch.zeros(H, V)})
+    with pytest.raises(AssertionError, match="Padding_idx"):
+        Embedding(V, H, padding_idx=V)
+    with pytest.raises(AssertionError, match="_weight"):
+        Embedding(V, H, _weight=torch.zeros(V, H))
+    assert Embedding(V, H, _freeze=True).weight.requires_grad is False
+    with pytest.raises(RuntimeError, match="GPU only"):
+        layer(torch.zeros(2, 3, dtype=torch.long))
+    with pytest.raises(NotImplementedError, match="sparse"):
+        Embedding(V, H, sparse=True)(torch.zeros(2, 3, dtype=torch.long))
+
+
+def test_checkpoint_round_trip_under_the_rank_prefix(tmp_path):
+    """axonn/checkpoint.py:11-27: one file per tensor-parallel rank, under a folder named
+    after its grid coordinates."""
+    from axonn_amd import checkpoint
+
+    assert checkpoint.get_prefix_for_checkpoint() == "tp_row_0_col_0_depth_0"
+    layer = Linear(16, 8)
+    state = {"model": layer.state_dict(), "step": 7}
+    checkpoint.save(state, str(tmp_path), "ckpt")
+    assert (tmp_path / "tp_row_0_col_0_depth_0" / "ckpt.pt").exists()
+    with pytest.raises(ValueError, match="already exists"):
+        checkpoint.save(state, str(tmp_path), "ckpt", overwrite=False)
+    loaded = checkpoint.load({}, str(tmp_path), "ckpt")
+    assert loaded["step"] == 7 and torch.equal(loaded["model"]["weight"], layer.weight)
+    other = Linear(16, 8)
+    other.load_state_dict(loaded["model"])
+    assert torch.equal(other.weight, layer.weight)
+    with pytest.raises(AssertionError, match="does not exist"):
+        checkpoint.load({}, str(tmp_path / "missing"), "ckpt")

@@ -435,3 +435,87 @@ def test_llama_mlp_oracle_matches_hugging_face_block_with_autograd():
     assert np.allclose(bwd["dx"], x.grad.numpy(), rtol=1e-11, atol=1e-14)
     for key, lin in (("dw_gate", mlp.gate_proj), ("dw_up", mlp.up_proj), ("dw_down", mlp.down_proj)):
         assert np.allclose(bwd[key].reshape(lin.weight.shape), lin.weight.grad.numpy(), rtol=1e-11, atol=1e-14)
+
+
+# ------------------------------------------------------------------ embedding
+@pytest.mark.parametrize("padding_idx", [None, 3])
+@pytest.mark.parametrize("scale", [False, True])
+def test_embedding_oracle_matches_torch_cpu_embedding_and_autograd(padding_idx, scale):
+    """torch's CPU F.embedding and its autograd are the library routines the reference
+    calls (axonn/intra_layer/embedding.py:164-172); ids repeat heavily (V = 11, T = 60)."""
+    from oracle import embedding as oe
+
+    torch.manual_seed(5)
+    V, H, T = 11, 8, 60
+    W = torch.randn(V, H, requires_grad=True)
+    ids = torch.randint(0, V, (4, 15))
+    dY = torch.randn(4, 15, H)
+    out = torch.nn.functional.embedding(ids, W, padding_idx=padding_idx, scale_grad_by_freq=scale)
+    out.backward(dY)
+    assert np.array_equal(oe.embedding_forward(ids.numpy(), W.detach().numpy()), out.detach().numpy())
+    dW = oe.embedding_backward(ids.numpy(), dY.numpy(), V, padding_idx, scale)
+    assert dW.dtype == np.float32
+    # torch sums in another order: a few fp32 roundings of sums of up to 12 terms
+    assert np.allclose(dW, W.grad.numpy(), rtol=2e-6, atol=2e-6)
+    d64 = oe.embedding_backward_f64(ids.numpy(), dY.numpy(), V, padding_idx, scale)
+    assert np.allclose(dW, d64, rtol=2e-6, atol=2e-6)
+    assert np.allclose(W.grad.numpy(), d64, rtol=2e-6, atol=2e-6)
+    if padding_idx is not None:
+        assert not dW[padding_idx].any() and (ids == padding_idx).any()
+
+
+def test_embedding_oracle_closed_forms():
+    from oracle import embedding as oe
+
+    rng = np.random.default_rng(0)
+    V, H = 9, 4
+    W = rng.standard_normal((V, H)).astype(np.float32)
+    perm = rng.permutation(V)
+    dY = rng.standard_normal((V, H)).astype(np.float32)
+    # a permutation of the rows: the gradient is dY put back in place, exactly
+    dW = oe.embedding_backward(perm, dY, V)
+    assert np.array_equal(dW[perm], dY)
+    assert np.array_equal(oe.embedding_forward(perm, W), W[perm])
+    # one id repeated: the sequential fp32 sum, term by term
+    rep = np.full(7, 2)
+    dY7 = rng.standard_normal((7, H)).astype(np.float32)
+    acc = np.zeros(H, np.float32)
+    for t in range(7):
+        acc = acc + dY7[t]
+    dW = oe.embedding_backward(rep, dY7, V)
+    assert np.array_equal(dW[2], acc) and not dW[[0, 1, 3, 4, 5, 6, 7, 8]].any()
+    # scale by frequency: the mean of the rows; the order of summation shows in the last bit only
+    dWs = oe.embedding_backward(rep, dY7, V, scale_grad_by_freq=True)
+    assert np.allclose(dWs[2], dY7.astype(np.float64).mean(axis=0), rtol=1e-6, atol=1e-7)
+    # ids outside the table: zeros forward, skipped backward
+    bad = np.array([1, -1, V, 4])
+    out = oe.embedding_forward(bad, W)
+    assert np.array_equal(out[0], W[1]) and not out[1].any() and not out[2].any()
+    dWb = oe.embedding_backward(bad, dY[:4], V)
+    assert np.array_equal(dWb[1], dY[0]) and np.array_equal(dWb[4], dY[3]) and dWb.sum() == (dY[0] + dY[3]).sum()
+    # accumulate: touched rows get sum + old, the others keep old
+    old = rng.standard_normal((V, H)).astype(np.float32)
+    acc2 = oe.embedding_backward(np.array([5, 5]), dY[:2], V, accumulate_into=old)
+    assert np.array_equal(acc2[5], (dY[0] + dY[1]) + old[5])
+    mask = np.ones(V, bool)
+    mask[5] = False
+    assert np.array_equal(acc2[mask], old[mask])
+
+
+@pytest.mark.parametrize("norm_type", [1.0, 2.0, 3.0])
+def test_embedding_renorm_oracle_matches_torch(norm_type):
+    from oracle import embedding as oe
+
+    torch.manual_seed(11)
+    V, H = 13, 16
+    W = torch.randn(V, H, dtype=torch.float64)
+    W[4] *= 0.01  # a row already inside the ball stays as it is
+    ids = torch.tensor([[1, 4, 4, 7], [7, 7, 12, 1]])
+    ref = W.clone()
+    torch.embedding_renorm_(ref, ids, 1.5, norm_type)
+    got = oe.embedding_renorm(W.numpy(), ids.numpy(), 1.5, norm_type)
+    assert np.allclose(got, ref.numpy(), rtol=1e-12, atol=1e-14)
+    untouched = [0, 2, 3, 5, 6, 8, 9, 10, 11]
+    assert np.array_equal(got[untouched], W.numpy()[untouched]) and np.array_equal(got[4], W.numpy()[4])
+    norms = np.linalg.norm(got[[1, 7, 12]], ord=norm_type, axis=1)
+    assert np.all(norms <= 1.5) and np.all(norms > 1.5 * (1 - 1e-6))
