@@ -123,69 +123,91 @@ struct Vec<uint16_t> {
   }
 };
 
-// One wave per (row, 64 x VEC columns).  VEC is the smaller of the two types'
-// 16-byte vectors, so both sides move at least 8 bytes per lane.
-template <typename TY, typename TW>
+// Loads VEC consecutive elements as fp32 (VEC = 4 or 8), 16 bytes per instruction
+// where the type allows.  Gradient rows are read once: non-temporal.
+template <int VEC>
+__device__ __forceinline__ void load_row_piece(const float* p, float (&x)[VEC]) {
+#pragma unroll
+  for (int h = 0; h < VEC / 4; ++h) {
+    const f32x4 v = __builtin_nontemporal_load((const f32x4*)p + h);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) x[4 * h + e] = v[e];
+  }
+}
+template <int VEC>
+__device__ __forceinline__ void load_row_piece(const uint16_t* p, float (&x)[VEC]) {
+  typedef __bf16 bf16xv __attribute__((ext_vector_type(VEC)));
+  const bf16xv v = __builtin_nontemporal_load((const bf16xv*)p);
+#pragma unroll
+  for (int e = 0; e < VEC; ++e) x[e] = (float)v[e];
+}
+template <int VEC>
+__device__ __forceinline__ void add_old(const float* p, float (&x)[VEC]) {
+  const f32x4 v = *(const f32x4*)p;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) x[e] += v[e];
+}
+template <int VEC>
+__device__ __forceinline__ void add_old(const uint16_t* p, float (&x)[VEC]) {
+  const bf16x8 v = *(const bf16x8*)p;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) x[e] += (float)v[e];
+}
+
+// One wave per (row, U x 64 x VEC columns): VEC = one 16-byte store of the dW type
+// per lane, U such pieces per lane, 64 x VEC columns apart, so that a wave has U
+// independent loads in flight per gradient row and U KiB of stores behind one
+// look-up of row_start (with one piece per wave the 8192 resident waves of the chip
+// covered 8 MB per memory latency: 4.2 TB/s on a gradient that is mostly zeros).
+template <typename TY, typename TW, int U>
 __global__ void __launch_bounds__(64 * WAVES_PER_BLOCK)
     embedding_bwd_kernel(const int* __restrict__ keys, const int* __restrict__ vals,
                          const int* __restrict__ row_start, const TY* __restrict__ dY, TW* dW,
                          int64_t T, int64_t V, int64_t H, int64_t lddy, int64_t lddw,
                          int units_per_row, int64_t padding_idx, int scale_by_freq, int beta) {
-  constexpr int VEC = 4;
+  constexpr int VEC = 16 / (int)sizeof(TW);
   const int lane = threadIdx.x & 63;
   const int64_t unit = (int64_t)blockIdx.x * WAVES_PER_BLOCK + (threadIdx.x >> 6);
   const int64_t row = unit / units_per_row;
   if (row >= V) return;
-  const int64_t col = ((unit % units_per_row) * 64 + lane) * VEC;
-  if (col >= H) return;
-  float acc[VEC] = {0.f, 0.f, 0.f, 0.f};
+  const int64_t col0 = ((unit % units_per_row) * U * 64 + lane) * VEC;
+  float acc[U][VEC];
+#pragma unroll
+  for (int u = 0; u < U; ++u)
+#pragma unroll
+    for (int q = 0; q < VEC; ++q) acc[u][q] = 0.f;
   const int s = row_start[row];
   if (s >= 0 && row != padding_idx) {
-    int e = s + 1;
     float inv = 1.0f;
     if (scale_by_freq) {
+      int e = s + 1;
       while (e < T && keys[e] == (int)row) ++e;
       inv = 1.0f / (float)(e - s);
     }
     for (int j = s; j < T; ++j) {
       if (j != s && keys[j] != (int)row) break;
-      const TY* src = dY + (int64_t)vals[j] * lddy + col;
-      float g[VEC];
-      if constexpr (sizeof(TY) == 4) {
-        const f32x4 v = __builtin_nontemporal_load((const f32x4*)src);
+      const TY* src = dY + (int64_t)vals[j] * lddy + col0;
+      float g[U][VEC];
 #pragma unroll
-        for (int q = 0; q < VEC; ++q) g[q] = v[q];
-      } else {
-        typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
-        const bf16x4 v = __builtin_nontemporal_load((const bf16x4*)src);
+      for (int u = 0; u < U; ++u)
+        if (col0 + u * 64 * VEC < H) load_row_piece<VEC>(src + u * 64 * VEC, g[u]);
 #pragma unroll
-        for (int q = 0; q < VEC; ++q) g[q] = (float)v[q];
-      }
+      for (int u = 0; u < U; ++u)
+        if (col0 + u * 64 * VEC < H) {
 #pragma unroll
-      for (int q = 0; q < VEC; ++q) acc[q] = scale_by_freq ? __fmaf_rn(g[q], inv, acc[q]) : acc[q] + g[q];
+          for (int q = 0; q < VEC; ++q)
+            acc[u][q] = scale_by_freq ? __fmaf_rn(g[u][q], inv, acc[u][q]) : acc[u][q] + g[u][q];
+        }
     }
   } else if (beta != 0) {
     return;  // nothing to add to this row
   }
-  TW* dst = dW + row * lddw + col;
-  if constexpr (sizeof(TW) == 4) {
-    if (beta != 0) {
-      const f32x4 old = *(const f32x4*)dst;
+  TW* dst = dW + row * lddw + col0;
 #pragma unroll
-      for (int q = 0; q < VEC; ++q) acc[q] += old[q];
-    }
-    __builtin_nontemporal_store(f32x4{acc[0], acc[1], acc[2], acc[3]}, (f32x4*)dst);
-  } else {
-    typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
-    if (beta != 0) {
-      const bf16x4 old = *(const bf16x4*)dst;
-#pragma unroll
-      for (int q = 0; q < VEC; ++q) acc[q] += (float)old[q];
-    }
-    bf16x4 v;
-#pragma unroll
-    for (int q = 0; q < VEC; ++q) v[q] = (__bf16)acc[q];
-    __builtin_nontemporal_store(v, (bf16x4*)dst);
+  for (int u = 0; u < U; ++u) {
+    if (col0 + u * 64 * VEC >= H) break;
+    if (beta != 0) add_old<VEC>(dst + u * 64 * VEC, acc[u]);
+    Vec<TW>::store(dst + u * 64 * VEC, acc[u]);
   }
 }
 
@@ -341,7 +363,11 @@ int launch_embedding_bwd(const int64_t* ids, const void* dY, void* dW, int dy_dt
               embedding_workspace_bytes(T, V));
     return AXN_EINVAL;
   }
-  const int upr = (int)((H / 4 + 63) / 64);
+  // pieces of 64 lanes x one 16-byte dW vector per row; up to 4 of them per wave
+  const int vec = dw_dtype == AXN_F32 ? 4 : 8;
+  const int64_t pieces = (H / vec + 63) / 64;
+  const int U = pieces >= 4 ? 4 : pieces >= 2 ? 2 : 1;
+  const int upr = (int)((pieces + U - 1) / U);
   const int64_t blocks = (V * upr + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK;
   if (blocks >= (1LL << 31)) {
     set_error("embedding_bwd: too many rows x columns (%lld blocks)", (long long)blocks);
@@ -351,10 +377,19 @@ int launch_embedding_bwd(const int64_t* ids, const void* dY, void* dW, int dy_dt
   int rc = sort_token_positions(ids, T, V, w, &keys, &vals, stream);
   if (rc) return rc;
   const dim3 grid((unsigned)blocks), block(64 * WAVES_PER_BLOCK);
-#define AXN_EMB_BWD(TY, TW)                                                                     \
-  hipLaunchKernelGGL((embedding_bwd_kernel<TY, TW>), grid, block, 0, stream, keys, vals,        \
+#define AXN_EMB_BWD_U(TY, TW, UU)                                                               \
+  hipLaunchKernelGGL((embedding_bwd_kernel<TY, TW, UU>), grid, block, 0, stream, keys, vals,    \
                      w.row_start, (const TY*)dY, (TW*)dW, T, V, H, lddy, lddw, upr, padding_idx, \
                      scale_by_freq, beta)
+#define AXN_EMB_BWD(TY, TW)                 \
+  do {                                      \
+    if (U == 4)                             \
+      AXN_EMB_BWD_U(TY, TW, 4);             \
+    else if (U == 2)                        \
+      AXN_EMB_BWD_U(TY, TW, 2);             \
+    else                                    \
+      AXN_EMB_BWD_U(TY, TW, 1);             \
+  } while (0)
   if (dy_dtype == AXN_F32 && dw_dtype == AXN_F32)
     AXN_EMB_BWD(float, float);
   else if (dy_dtype == AXN_F32)
@@ -363,6 +398,7 @@ int launch_embedding_bwd(const int64_t* ids, const void* dY, void* dW, int dy_dt
     AXN_EMB_BWD(uint16_t, float);
   else
     AXN_EMB_BWD(uint16_t, uint16_t);
+#undef AXN_EMB_BWD_U
 #undef AXN_EMB_BWD
   AXN_HIP_TRY(hipGetLastError());
   return AXN_OK;

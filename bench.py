@@ -15,7 +15,8 @@ keys of the one JSON line:
             64 ragged tensors, GB/s at 30 algorithmic bytes per element, and the
             overflow (skip) variant
   shapes    the 12B-style MLP shard with fused bias + GELU, the skinny
-            decode-like shard, and the Llama MLP block with the one-pass SwiGLU
+            decode-like shard, the Llama MLP block with the one-pass SwiGLU, and the
+            embedding lookup and its weight gradient at the Llama-3 vocabulary
   cpu_baseline  the torch-CPU restatement of the same layer math on the host cores
 
 Every GEMM launch of the timed region is bracketed by HIP events on the launch
@@ -286,6 +287,33 @@ def main():
             "swiglu_fwd_gbs": round(6.0 * Mt * I / t_sw / 1e9, 1),
             "swiglu_bwd_gbs": round(10.0 * Mt * I / t_swb / 1e9, 1)}
         del x, wg, wu, wd, dy, gt, up, act, dact, dgt, dup, y, dx1, dx2, dwg, dwu, dwd
+        torch.cuda.empty_cache()
+
+        # Embedding of the Llama-3 vocabulary at the largest shape of the reference's own
+        # test of the layer (B 8, S 2048, H 2048, V 128256, fp32): row gather forward and
+        # the dense weight gradient (sort of the token positions + one pass that writes
+        # every row of dW once).
+        Te, He, Ve = 8 * 2048, 2048, 128256
+        g = torch.Generator(device="cuda").manual_seed(13)
+        table = torch.randn(Ve, He, generator=g, device="cuda")
+        ids = torch.randint(0, Ve, (Te,), generator=g, device="cuda")
+        dye = torch.randn(Te, He, generator=g, device="cuda") * 1e-3
+        oute = torch.empty(Te, He, device="cuda")
+        dtab = torch.empty(Ve, He, device="cuda")
+        ws_bytes = lib.axn_embedding_workspace_bytes(Te, Ve)
+        wse = torch.empty(ws_bytes, dtype=torch.uint8, device="cuda")
+        t_ef = time_loop(lambda: nv.check(lib.axn_embedding_fwd(
+            P(ids), P(table), P(oute), nv.F32, Te, Ve, He, He, He, None, stream)), 20)
+        t_eb = time_loop(lambda: nv.check(lib.axn_embedding_bwd(
+            P(ids), P(dye), P(dtab), nv.F32, nv.F32, Te, Ve, He, He, He, -1, 0, 0, P(wse), ws_bytes,
+            stream)), 20)
+        fwd_bytes = 8.0 * Te * He + 8.0 * Te            # rows in, rows out, ids
+        bwd_bytes = 4.0 * Te * He + 4.0 * Ve * He + 8.0 * Te  # dY in, every dW row out, ids
+        shapes["embedding_16384x2048x128256_f32"] = {
+            "fwd_us": round(t_ef * 1e6, 1), "fwd_gbs": round(fwd_bytes / t_ef / 1e9, 1),
+            "bwd_us": round(t_eb * 1e6, 1), "bwd_gbs": round(bwd_bytes / t_eb / 1e9, 1),
+            "bwd_frac_hbm": round(bwd_bytes / t_eb / 1e9 / PEAK_HBM_GBS, 4)}
+        del table, ids, dye, oute, dtab, wse
         torch.cuda.empty_cache()
 
     adam = None
