@@ -115,15 +115,16 @@ int axn_abi_version(void) { return AXN_ABI_VERSION; }
 
 const char* axn_last_error(void) { return g_err; }
 
-int axn_gemm_fwd(const void* X, const void* W, const float* bias, void* Y,
-                 void* Zsave, int64_t M, int64_t N, int64_t K, int64_t ldx,
-                 int64_t ldw, int64_t ldy, int epilogue, void* stream) {
-  int rc = check_gemm("axn_gemm_fwd", X, W, Y, M, N, K, ldx, ldw, ldy, K, K, N);
+// The 16-bit GEMM entry points: `half` selects IEEE half instead of bfloat16.
+static int gemm_fwd_16(const char* name, bool half, const void* X, const void* W,
+                       const float* bias, void* Y, void* Zsave, int64_t M, int64_t N, int64_t K,
+                       int64_t ldx, int64_t ldw, int64_t ldy, int epilogue, void* stream) {
+  int rc = check_gemm(name, X, W, Y, M, N, K, ldx, ldw, ldy, K, K, N);
   if (rc) return rc;
-  rc = check_epilogue("axn_gemm_fwd", epilogue, bias);
+  rc = check_epilogue(name, epilogue, bias);
   if (rc) return rc;
-  REQUIRE(Zsave == nullptr || aligned16(Zsave), AXN_EALIGN,
-          "axn_gemm_fwd: Zsave must be 16-byte aligned");
+  REQUIRE(Zsave == nullptr || aligned16(Zsave), AXN_EALIGN, "%s: Zsave must be 16-byte aligned",
+          name);
   GemmArgs g = {};
   g.A = (const uint16_t*)X;
   g.B = (const uint16_t*)W;
@@ -137,13 +138,14 @@ int axn_gemm_fwd(const void* X, const void* W, const float* bias, void* Y,
   g.ldb = ldw;
   g.ldc = ldy;
   g.beta = 0;
-  return launch_gemm_bf16(GEMM_NT, g, epilogue, false, (hipStream_t)stream);
+  return half ? launch_gemm_f16(GEMM_NT, g, epilogue, false, (hipStream_t)stream)
+              : launch_gemm_bf16(GEMM_NT, g, epilogue, false, (hipStream_t)stream);
 }
 
-int axn_gemm_dgrad(const void* dY, const void* W, void* dX, int64_t M, int64_t N,
-                   int64_t K, int64_t lddy, int64_t ldw, int64_t lddx,
-                   void* stream) {
-  int rc = check_gemm("axn_gemm_dgrad", dY, W, dX, M, N, K, lddy, ldw, lddx, N, K, K);
+static int gemm_dgrad_16(const char* name, bool half, const void* dY, const void* W, void* dX,
+                         int64_t M, int64_t N, int64_t K, int64_t lddy, int64_t ldw,
+                         int64_t lddx, void* stream) {
+  int rc = check_gemm(name, dY, W, dX, M, N, K, lddy, ldw, lddx, N, K, K);
   if (rc) return rc;
   GemmArgs g = {};
   g.A = (const uint16_t*)dY;  // [M][N]: rows of the output, contraction contiguous
@@ -156,17 +158,18 @@ int axn_gemm_dgrad(const void* dY, const void* W, void* dX, int64_t M, int64_t N
   g.ldb = ldw;
   g.ldc = lddx;
   g.beta = 0;
-  return launch_gemm_bf16(GEMM_NN, g, AXN_EPI_NONE, false, (hipStream_t)stream);
+  return half ? launch_gemm_f16(GEMM_NN, g, AXN_EPI_NONE, false, (hipStream_t)stream)
+              : launch_gemm_bf16(GEMM_NN, g, AXN_EPI_NONE, false, (hipStream_t)stream);
 }
 
-int axn_gemm_wgrad(const void* dY, const void* X, void* dW, int64_t M, int64_t N,
-                   int64_t K, int64_t lddy, int64_t ldx, int64_t lddw, int beta,
-                   int dw_dtype, void* stream) {
-  int rc = check_gemm("axn_gemm_wgrad", dY, X, dW, M, N, K, lddy, ldx, lddw, N, K, K);
+static int gemm_wgrad_16(const char* name, bool half, const void* dY, const void* X, void* dW,
+                         int64_t M, int64_t N, int64_t K, int64_t lddy, int64_t ldx,
+                         int64_t lddw, int beta, int dw_dtype, void* stream) {
+  int rc = check_gemm(name, dY, X, dW, M, N, K, lddy, ldx, lddw, N, K, K);
   if (rc) return rc;
-  REQUIRE(beta == 0 || beta == 1, AXN_EINVAL, "axn_gemm_wgrad: beta must be 0 or 1");
-  REQUIRE(dw_dtype == AXN_BF16 || dw_dtype == AXN_F32, AXN_EINVAL,
-          "axn_gemm_wgrad: dW must be bf16 or fp32");
+  REQUIRE(beta == 0 || beta == 1, AXN_EINVAL, "%s: beta must be 0 or 1", name);
+  REQUIRE(dw_dtype == (half ? AXN_F16 : AXN_BF16) || dw_dtype == AXN_F32, AXN_EINVAL,
+          "%s: dW must be %s or fp32", name, half ? "fp16" : "bf16");
   GemmArgs g = {};
   g.A = (const uint16_t*)dY;  // [M][N]: contraction-major, output rows = N
   g.B = (const uint16_t*)X;   // [M][K]: contraction-major, output cols = K
@@ -178,8 +181,49 @@ int axn_gemm_wgrad(const void* dY, const void* X, void* dW, int64_t M, int64_t N
   g.ldb = ldx;
   g.ldc = lddw;
   g.beta = beta;
-  return launch_gemm_bf16(GEMM_TN, g, AXN_EPI_NONE, dw_dtype == AXN_F32,
-                          (hipStream_t)stream);
+  return half ? launch_gemm_f16(GEMM_TN, g, AXN_EPI_NONE, dw_dtype == AXN_F32,
+                                (hipStream_t)stream)
+              : launch_gemm_bf16(GEMM_TN, g, AXN_EPI_NONE, dw_dtype == AXN_F32,
+                                 (hipStream_t)stream);
+}
+
+int axn_gemm_fwd(const void* X, const void* W, const float* bias, void* Y,
+                 void* Zsave, int64_t M, int64_t N, int64_t K, int64_t ldx,
+                 int64_t ldw, int64_t ldy, int epilogue, void* stream) {
+  return gemm_fwd_16("axn_gemm_fwd", false, X, W, bias, Y, Zsave, M, N, K, ldx, ldw, ldy,
+                     epilogue, stream);
+}
+
+int axn_gemm_dgrad(const void* dY, const void* W, void* dX, int64_t M, int64_t N,
+                   int64_t K, int64_t lddy, int64_t ldw, int64_t lddx,
+                   void* stream) {
+  return gemm_dgrad_16("axn_gemm_dgrad", false, dY, W, dX, M, N, K, lddy, ldw, lddx, stream);
+}
+
+int axn_gemm_wgrad(const void* dY, const void* X, void* dW, int64_t M, int64_t N,
+                   int64_t K, int64_t lddy, int64_t ldx, int64_t lddw, int beta,
+                   int dw_dtype, void* stream) {
+  return gemm_wgrad_16("axn_gemm_wgrad", false, dY, X, dW, M, N, K, lddy, ldx, lddw, beta,
+                       dw_dtype, stream);
+}
+
+int axn_gemm_fwd_f16(const void* X, const void* W, const float* bias, void* Y,
+                     void* Zsave, int64_t M, int64_t N, int64_t K, int64_t ldx,
+                     int64_t ldw, int64_t ldy, int epilogue, void* stream) {
+  return gemm_fwd_16("axn_gemm_fwd_f16", true, X, W, bias, Y, Zsave, M, N, K, ldx, ldw, ldy,
+                     epilogue, stream);
+}
+
+int axn_gemm_dgrad_f16(const void* dY, const void* W, void* dX, int64_t M, int64_t N,
+                       int64_t K, int64_t lddy, int64_t ldw, int64_t lddx, void* stream) {
+  return gemm_dgrad_16("axn_gemm_dgrad_f16", true, dY, W, dX, M, N, K, lddy, ldw, lddx, stream);
+}
+
+int axn_gemm_wgrad_f16(const void* dY, const void* X, void* dW, int64_t M, int64_t N,
+                       int64_t K, int64_t lddy, int64_t ldx, int64_t lddw, int beta,
+                       int dw_dtype, void* stream) {
+  return gemm_wgrad_16("axn_gemm_wgrad_f16", true, dY, X, dW, M, N, K, lddy, ldx, lddw, beta,
+                       dw_dtype, stream);
 }
 
 size_t axn_dgelu_dbias_workspace_bytes(int64_t M, int64_t N) {
@@ -191,8 +235,8 @@ int axn_dgelu_dbias(const void* dY, const void* Z, void* dZ, int dtype,
                     void* workspace, size_t workspace_bytes, void* stream) {
   const char* name = "axn_dgelu_dbias";
   REQUIRE(dY != nullptr, AXN_EINVAL, "%s: dY is null", name);
-  REQUIRE(dtype == AXN_BF16 || dtype == AXN_F32, AXN_EINVAL,
-          "%s: dtype must be bf16 or fp32", name);
+  REQUIRE(dtype == AXN_BF16 || dtype == AXN_F16 || dtype == AXN_F32, AXN_EINVAL,
+          "%s: unknown dtype %d", name, dtype);
   REQUIRE(M >= 1 && N >= 1, AXN_EINVAL, "%s: M and N must be >= 1", name);
   REQUIRE(N % 8 == 0, AXN_ESHAPE, "%s: N must be a multiple of 8", name);
   REQUIRE(ld >= N && ld % 8 == 0, AXN_EALIGN,
@@ -208,7 +252,8 @@ int axn_dgelu_dbias(const void* dY, const void* Z, void* dZ, int dtype,
 }
 
 static int check_swiglu(const char* name, int dtype, int64_t M, int64_t N, int64_t ld) {
-  REQUIRE(dtype == AXN_BF16 || dtype == AXN_F32, AXN_EINVAL, "%s: dtype must be bf16 or fp32", name);
+  REQUIRE(dtype == AXN_BF16 || dtype == AXN_F16 || dtype == AXN_F32, AXN_EINVAL,
+          "%s: unknown dtype %d", name, dtype);
   REQUIRE(M >= 1 && N >= 1, AXN_EINVAL, "%s: M and N must be >= 1", name);
   REQUIRE(N % 8 == 0, AXN_ESHAPE, "%s: N must be a multiple of 8", name);
   REQUIRE(ld >= N && ld % 8 == 0, AXN_EALIGN, "%s: ld must be >= N and a multiple of 8", name);

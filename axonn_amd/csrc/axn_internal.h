@@ -76,6 +76,9 @@ enum GemmLayout { GEMM_NT = 0, GEMM_NN = 1, GEMM_TN = 2 };
 
 int launch_gemm_bf16(GemmLayout layout, const GemmArgs& args, int epilogue,
                      bool out_f32, hipStream_t stream);
+// The same kernels on IEEE half operands (v_mfma_f32_16x16x32_f16, half outputs).
+int launch_gemm_f16(GemmLayout layout, const GemmArgs& args, int epilogue, bool out_f32,
+                    hipStream_t stream);
 
 // ---- fp32 GEMM (full-precision layers) --------------------------------------
 int launch_gemm_f32(GemmLayout layout, const float* A, const float* B, float* C,

@@ -19,6 +19,7 @@ namespace axn {
 namespace {
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 
 constexpr int EW_TX = 64;          // lanes along columns (8 columns each)
@@ -29,6 +30,11 @@ constexpr int EW_BAND = 128;       // rows per workgroup
 // 8 consecutive columns as floats, for bf16 (16 bytes) and fp32 (32 bytes) rows.
 __device__ __forceinline__ void load8(const uint16_t* p, float (&x)[8]) {
   const bf16x8 v = *(const bf16x8*)p;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) x[e] = (float)v[e];
+}
+__device__ __forceinline__ void load8(const _Float16* p, float (&x)[8]) {
+  const f16x8 v = *(const f16x8*)p;
 #pragma unroll
   for (int e = 0; e < 8; ++e) x[e] = (float)v[e];
 }
@@ -49,6 +55,15 @@ __device__ __forceinline__ void store8(uint16_t* p, float (&x)[8]) {
     x[e] = (float)v[e];
   }
   *(bf16x8*)p = v;
+}
+__device__ __forceinline__ void store8(_Float16* p, float (&x)[8]) {
+  f16x8 v;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    v[e] = (_Float16)x[e];
+    x[e] = (float)v[e];
+  }
+  *(f16x8*)p = v;
 }
 __device__ __forceinline__ void store8(float* p, float (&x)[8]) {
   *(f32x4*)p = f32x4{x[0], x[1], x[2], x[3]};
@@ -182,6 +197,9 @@ int launch_swiglu_fwd(const void* gate, const void* up, void* out, int dtype, in
   if (dtype == AXN_F32)
     hipLaunchKernelGGL(swiglu_fwd_kernel<float>, grid, block, 0, stream, (const float*)gate,
                        (const float*)up, (float*)out, M, N, ld);
+  else if (dtype == AXN_F16)
+    hipLaunchKernelGGL(swiglu_fwd_kernel<_Float16>, grid, block, 0, stream, (const _Float16*)gate,
+                       (const _Float16*)up, (_Float16*)out, M, N, ld);
   else
     hipLaunchKernelGGL(swiglu_fwd_kernel<uint16_t>, grid, block, 0, stream, (const uint16_t*)gate,
                        (const uint16_t*)up, (uint16_t*)out, M, N, ld);
@@ -200,6 +218,10 @@ int launch_swiglu_bwd(const void* dout, const void* gate, const void* up, void* 
   if (dtype == AXN_F32)
     hipLaunchKernelGGL(swiglu_bwd_kernel<float>, grid, block, 0, stream, (const float*)dout,
                        (const float*)gate, (const float*)up, (float*)dgate, (float*)dup, M, N, ld);
+  else if (dtype == AXN_F16)
+    hipLaunchKernelGGL(swiglu_bwd_kernel<_Float16>, grid, block, 0, stream, (const _Float16*)dout,
+                       (const _Float16*)gate, (const _Float16*)up, (_Float16*)dgate,
+                       (_Float16*)dup, M, N, ld);
   else
     hipLaunchKernelGGL(swiglu_bwd_kernel<uint16_t>, grid, block, 0, stream, (const uint16_t*)dout,
                        (const uint16_t*)gate, (const uint16_t*)up, (uint16_t*)dgate,
@@ -240,6 +262,14 @@ int launch_dgelu_dbias(const void* dY, const void* Z, void* dZ, int dtype,
     else
       hipLaunchKernelGGL((dgelu_dbias_kernel<float, false>), grid, block, 0, stream,
                          y, z, (float*)dZ, partial, M, N, ld);
+  } else if (dtype == AXN_F16) {
+    const _Float16 *y = (const _Float16*)dY, *z = (const _Float16*)Z;
+    if (Z != nullptr)
+      hipLaunchKernelGGL((dgelu_dbias_kernel<_Float16, true>), grid, block, 0, stream, y, z,
+                         (_Float16*)dZ, partial, M, N, ld);
+    else
+      hipLaunchKernelGGL((dgelu_dbias_kernel<_Float16, false>), grid, block, 0, stream, y, z,
+                         (_Float16*)dZ, partial, M, N, ld);
   } else {
     const uint16_t *y = (const uint16_t*)dY, *z = (const uint16_t*)Z;
     if (Z != nullptr)

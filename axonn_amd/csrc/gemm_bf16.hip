@@ -39,6 +39,7 @@ namespace {
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
 typedef __attribute__((ext_vector_type(4))) short s16x4;
 typedef __attribute__((ext_vector_type(8))) short s16x8;
 typedef __attribute__((ext_vector_type(16))) float f32x16;
@@ -171,8 +172,11 @@ struct OperandTile {
 // Epilogue of 8 consecutive columns of one output row, held in fp32: bias,
 // exact GELU with optional save of the pre-activation, accumulation into the
 // existing output (beta), conversion and one 16- or 32-byte store.
-template <int EPI, bool OUT_F32>
+// HALF: the 16-bit storage type is IEEE half instead of bfloat16.
+template <int EPI, bool OUT_F32, bool HALF>
 __device__ __forceinline__ void store_row8(float (&v)[8], const GemmArgs& g, int row, int col) {
+  using lp = std::conditional_t<HALF, _Float16, __bf16>;
+  using lpx8 = std::conditional_t<HALF, f16x8, bf16x8>;
   const int64_t o = (int64_t)row * g.ldc + col;
   if (EPI == AXN_EPI_BIAS || EPI == AXN_EPI_BIAS_GELU) {
     const f32x4 b0 = *(const f32x4*)(g.bias + col);
@@ -185,10 +189,10 @@ __device__ __forceinline__ void store_row8(float (&v)[8], const GemmArgs& g, int
   }
   if (EPI == AXN_EPI_BIAS_GELU || EPI == AXN_EPI_GELU) {
     if (g.Z != nullptr) {
-      bf16x8 z;
+      lpx8 z;
 #pragma unroll
-      for (int e = 0; e < 8; ++e) z[e] = (__bf16)v[e];
-      *(bf16x8*)(g.Z + o) = z;
+      for (int e = 0; e < 8; ++e) z[e] = (lp)v[e];
+      *(lpx8*)(g.Z + o) = z;
     }
 #pragma unroll
     for (int e = 0; e < 8; ++e) v[e] = gelu_exact(v[e]);
@@ -205,14 +209,14 @@ __device__ __forceinline__ void store_row8(float (&v)[8], const GemmArgs& g, int
   } else {
     uint16_t* C = (uint16_t*)g.C + o;
     if (g.beta) {
-      const bf16x8 old = *(const bf16x8*)C;
+      const lpx8 old = *(const lpx8*)C;
 #pragma unroll
       for (int e = 0; e < 8; ++e) v[e] += (float)old[e];
     }
-    bf16x8 y;
+    lpx8 y;
 #pragma unroll
-    for (int e = 0; e < 8; ++e) y[e] = (__bf16)v[e];
-    *(bf16x8*)C = y;
+    for (int e = 0; e < 8; ++e) y[e] = (lp)v[e];
+    *(lpx8*)C = y;
   }
 }
 
@@ -223,7 +227,7 @@ __device__ __forceinline__ void store_row8(float (&v)[8], const GemmArgs& g, int
 // a per-wave LDS buffer (32 rows x 64 fp32 columns, padded) so that every lane
 // then owns 8 consecutive columns of one row.  The caller must have made sure
 // that no wave still reads operand tiles from LDS.
-template <int FM, int FN, int EPI, bool OUT_F32, bool EDGE>
+template <int FM, int FN, int EPI, bool OUT_F32, bool EDGE, bool HALF>
 __device__ __forceinline__ void store_tile(const f32x16 (&acc)[FM][FN], const GemmArgs& g,
                                            char* lds, int wave, int lane, int row0,
                                            int col0) {
@@ -257,7 +261,7 @@ __device__ __forceinline__ void store_tile(const f32x16 (&acc)[FM][FN], const Ge
         const int row = row0 + i * 32 + r;
         const int col = col0 + jp * EPC + c;
         if (EDGE && (row >= g.M || col >= g.N)) continue;
-        store_row8<EPI, OUT_F32>(v, g, row, col);
+        store_row8<EPI, OUT_F32, HALF>(v, g, row, col);
       }
     }
   }
@@ -438,8 +442,8 @@ __device__ __forceinline__ void wait_vmcnt() {
 // TILE = 128 is the same schedule on a 128 x 128 tile for problems that do not
 // fill the chip with 256 x 256 tiles: 64 x 64 per wave (4 x 4 blocks, 16 MFMAs per
 // step, 4 copies per tile and wave), an 80 KiB ring, two workgroups per CU.
-template <int TILE, bool A_KMAJOR, bool B_KMAJOR, int EPI, bool OUT_F32>
-__global__ void __launch_bounds__(256) gemm_bf16_solo_kernel(const GemmArgs g) {
+template <int TILE, bool A_KMAJOR, bool B_KMAJOR, int EPI, bool OUT_F32, bool HALF>
+__device__ __forceinline__ void solo_gemm(const GemmArgs& g) {
   constexpr int BM = TILE, BN = TILE, WTM = TILE / 2, WTN = TILE / 2, FR = TILE / 32;
   constexpr int PK = 64, NSLOT = 5;
   constexpr int NM = FR * FR;           // MFMAs per step
@@ -561,9 +565,15 @@ __global__ void __launch_bounds__(256) gemm_bf16_solo_kernel(const GemmArgs g) {
         // (transposed) fragments through AGPRs and spills.  No MFMA hazard can arise:
         // fragments come from LDS behind s_waitcnt, and an accumulator is touched
         // again only NM - 1 (at least 15) independent MFMAs later.
-        asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0"
-                     : "+a"(acc[i][j])
-                     : "v"(fb[j]), "v"(fa[i]));
+        // (fragments are opaque 16-byte registers: the mnemonic alone names the type)
+        if constexpr (HALF)
+          asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0"
+                       : "+a"(acc[i][j])
+                       : "v"(fb[j]), "v"(fa[i]));
+        else
+          asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0"
+                       : "+a"(acc[i][j])
+                       : "v"(fb[j]), "v"(fa[i]));
         if constexpr (m < NM / 2 && m % READ_EVERY == 0) {
           if constexpr (ST == 0) read(std::integral_constant<int, 1>{},
                                       std::integral_constant<int, m / READ_EVERY>{}, sa, sb);
@@ -606,17 +616,25 @@ __global__ void __launch_bounds__(256) gemm_bf16_solo_kernel(const GemmArgs g) {
     for (int t = 0; t < FR / 2; ++t) {
       const f32x4 lo = acc[i][2 * t], hi = acc[i][2 * t + 1];
       float v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-      store_row8<EPI, OUT_F32>(v, g, orow + 16 * i, ocol + 32 * t);
+      store_row8<EPI, OUT_F32, HALF>(v, g, orow + 16 * i, ocol + 32 * t);
     }
+}
+
+template <int TILE, bool A_KMAJOR, bool B_KMAJOR, int EPI, bool OUT_F32>
+__global__ void __launch_bounds__(256) gemm_bf16_solo_kernel(const GemmArgs g) {
+  solo_gemm<TILE, A_KMAJOR, B_KMAJOR, EPI, OUT_F32, false>(g);
+}
+template <int TILE, bool A_KMAJOR, bool B_KMAJOR, int EPI, bool OUT_F32>
+__global__ void __launch_bounds__(256) gemm_f16_solo_kernel(const GemmArgs g) {
+  solo_gemm<TILE, A_KMAJOR, B_KMAJOR, EPI, OUT_F32, true>(g);
 }
 
 // ---------------------------------------------------------------------------
 // Register-staged kernel.
 // ---------------------------------------------------------------------------
 template <int BM, int BN, int WAVES_M, int WAVES_N, bool A_KMAJOR, bool B_KMAJOR,
-          int EPI, bool OUT_F32, bool EDGE>
-__global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
-    gemm_bf16_kernel(const GemmArgs g) {
+          int EPI, bool OUT_F32, bool EDGE, bool HALF>
+__device__ __forceinline__ void staged_gemm(const GemmArgs& g) {
   constexpr int NT = WAVES_M * WAVES_N * 64;
   constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N;
   constexpr int FM = WTM / 32, FN = WTN / 32;
@@ -670,8 +688,13 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
     for (int i = 0; i < FM; ++i)
 #pragma unroll
       for (int j = 0; j < FN; ++j)
-        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[buf][j], fa[buf][i],
-                                                            acc[i][j], 0, 0, 0);
+        if constexpr (HALF)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
+              __builtin_bit_cast(f16x8, fb[buf][j]), __builtin_bit_cast(f16x8, fa[buf][i]),
+              acc[i][j], 0, 0, 0);
+        else
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[buf][j], fa[buf][i],
+                                                              acc[i][j], 0, 0, 0);
   };
 
   read_frags(0, lds, lds + TA::BYTES, 0);
@@ -700,18 +723,32 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
     if (more) read_frags(0, nA, nA + TA::BYTES, 0);
   }
 
-  store_tile<FM, FN, EPI, OUT_F32, EDGE>(acc, g, lds, wave, lane, m0 + wm * WTM, n0 + wn * WTN);
+  store_tile<FM, FN, EPI, OUT_F32, EDGE, HALF>(acc, g, lds, wave, lane, m0 + wm * WTM,
+                                               n0 + wn * WTN);
+}
+
+template <int BM, int BN, int WAVES_M, int WAVES_N, bool A_KMAJOR, bool B_KMAJOR,
+          int EPI, bool OUT_F32, bool EDGE>
+__global__ void __launch_bounds__(WAVES_M* WAVES_N * 64) gemm_bf16_kernel(const GemmArgs g) {
+  staged_gemm<BM, BN, WAVES_M, WAVES_N, A_KMAJOR, B_KMAJOR, EPI, OUT_F32, EDGE, false>(g);
+}
+template <int BM, int BN, int WAVES_M, int WAVES_N, bool A_KMAJOR, bool B_KMAJOR,
+          int EPI, bool OUT_F32, bool EDGE>
+__global__ void __launch_bounds__(WAVES_M* WAVES_N * 64) gemm_f16_kernel(const GemmArgs g) {
+  staged_gemm<BM, BN, WAVES_M, WAVES_N, A_KMAJOR, B_KMAJOR, EPI, OUT_F32, EDGE, true>(g);
 }
 
 template <int BM, int BN, int WAVES_M, int WAVES_N, bool AK, bool BKM, int EPI,
-          bool OUT_F32, bool EDGE>
+          bool OUT_F32, bool EDGE, bool HALF>
 int launch_cfg(const GemmArgs& in, hipStream_t stream) {
   GemmArgs g = in;
   g.tiles_m = (g.M + BM - 1) / BM;
   g.tiles_n = (g.N + BN - 1) / BN;
   constexpr int NT = WAVES_M * WAVES_N * 64;
   constexpr size_t lds = 2 * (size_t)(BM + BN) * BK * 2;
-  auto kern = gemm_bf16_kernel<BM, BN, WAVES_M, WAVES_N, AK, BKM, EPI, OUT_F32, EDGE>;
+  void (*kern)(const GemmArgs) =
+      gemm_bf16_kernel<BM, BN, WAVES_M, WAVES_N, AK, BKM, EPI, OUT_F32, EDGE>;
+  if constexpr (HALF) kern = gemm_f16_kernel<BM, BN, WAVES_M, WAVES_N, AK, BKM, EPI, OUT_F32, EDGE>;
   AXN_HIP_TRY(hipFuncSetAttribute((const void*)kern,
                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
   const long long nwg = (long long)g.tiles_m * g.tiles_n;
@@ -724,14 +761,15 @@ int launch_cfg(const GemmArgs& in, hipStream_t stream) {
   return AXN_OK;
 }
 
-template <int TILE, bool AK, bool BKM, int EPI, bool OUT_F32>
+template <int TILE, bool AK, bool BKM, int EPI, bool OUT_F32, bool HALF>
 int launch_solo(const GemmArgs& in, hipStream_t stream) {
   GemmArgs g = in;
   g.tiles_m = g.M / TILE;
   g.tiles_n = g.N / TILE;
   // ring of 5 operand tiles: 160 KiB (all of a CU's LDS) or 80 KiB (two workgroups per CU)
   constexpr size_t lds = 5 * TILE * 64 * 2;
-  auto kern = gemm_bf16_solo_kernel<TILE, AK, BKM, EPI, OUT_F32>;
+  void (*kern)(const GemmArgs) = gemm_bf16_solo_kernel<TILE, AK, BKM, EPI, OUT_F32>;
+  if constexpr (HALF) kern = gemm_f16_solo_kernel<TILE, AK, BKM, EPI, OUT_F32>;
   AXN_HIP_TRY(hipFuncSetAttribute((const void*)kern,
                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
   hipLaunchKernelGGL(kern, dim3((unsigned)(g.tiles_m * g.tiles_n)), dim3(256), lds, stream, g);
@@ -744,7 +782,7 @@ int launch_solo(const GemmArgs& in, hipStream_t stream) {
 // other problems made of whole 128 x 128 tiles take it at 128 x 128; ragged
 // shapes, and operands too large for 32-bit byte offsets, take the
 // register-staged kernel.
-template <bool AK, bool BKM, int EPI, bool OUT_F32>
+template <bool AK, bool BKM, int EPI, bool OUT_F32, bool HALF>
 int launch_shape(const GemmArgs& g, hipStream_t stream) {
   const bool deep = g.Kc % 64 == 0;
   const bool whole256 = (g.M % 256 == 0) && (g.N % 256 == 0) && deep;
@@ -758,41 +796,54 @@ int launch_shape(const GemmArgs& g, hipStream_t stream) {
   // Up to 128 large tiles the small tile wins: four times as many workgroups, two per CU, still
   // fit in one round.  Beyond that its second round costs more than the idle CUs of the large one.
   if (small_spans && whole256 && tiles256 > 128)
-    return launch_solo<256, AK, BKM, EPI, OUT_F32>(g, stream);
+    return launch_solo<256, AK, BKM, EPI, OUT_F32, HALF>(g, stream);
   if (small_spans && whole128 && tiles128 < (1LL << 31))
-    return launch_solo<128, AK, BKM, EPI, OUT_F32>(g, stream);
-  if (whole128) return launch_cfg<128, 128, 2, 2, AK, BKM, EPI, OUT_F32, false>(g, stream);
-  return launch_cfg<128, 128, 2, 2, AK, BKM, EPI, OUT_F32, true>(g, stream);
+    return launch_solo<128, AK, BKM, EPI, OUT_F32, HALF>(g, stream);
+  if (whole128) return launch_cfg<128, 128, 2, 2, AK, BKM, EPI, OUT_F32, false, HALF>(g, stream);
+  return launch_cfg<128, 128, 2, 2, AK, BKM, EPI, OUT_F32, true, HALF>(g, stream);
 }
 
 }  // namespace
 
-int launch_gemm_bf16(GemmLayout layout, const GemmArgs& g, int epilogue,
-                     bool out_f32, hipStream_t stream) {
+namespace {
+template <bool HALF>
+int launch_layout(GemmLayout layout, const GemmArgs& g, int epilogue, bool out_f32,
+                  hipStream_t stream) {
   switch (layout) {
     case GEMM_NT:
       if (out_f32) break;
       switch (epilogue) {
         case AXN_EPI_NONE:
-          return launch_shape<true, true, AXN_EPI_NONE, false>(g, stream);
+          return launch_shape<true, true, AXN_EPI_NONE, false, HALF>(g, stream);
         case AXN_EPI_BIAS:
-          return launch_shape<true, true, AXN_EPI_BIAS, false>(g, stream);
+          return launch_shape<true, true, AXN_EPI_BIAS, false, HALF>(g, stream);
         case AXN_EPI_BIAS_GELU:
-          return launch_shape<true, true, AXN_EPI_BIAS_GELU, false>(g, stream);
+          return launch_shape<true, true, AXN_EPI_BIAS_GELU, false, HALF>(g, stream);
         case AXN_EPI_GELU:
-          return launch_shape<true, true, AXN_EPI_GELU, false>(g, stream);
+          return launch_shape<true, true, AXN_EPI_GELU, false, HALF>(g, stream);
       }
       break;
     case GEMM_NN:
       if (out_f32 || epilogue != AXN_EPI_NONE) break;
-      return launch_shape<true, false, AXN_EPI_NONE, false>(g, stream);
+      return launch_shape<true, false, AXN_EPI_NONE, false, HALF>(g, stream);
     case GEMM_TN:
       if (epilogue != AXN_EPI_NONE) break;
-      return out_f32 ? launch_shape<false, false, AXN_EPI_NONE, true>(g, stream)
-                     : launch_shape<false, false, AXN_EPI_NONE, false>(g, stream);
+      return out_f32 ? launch_shape<false, false, AXN_EPI_NONE, true, HALF>(g, stream)
+                     : launch_shape<false, false, AXN_EPI_NONE, false, HALF>(g, stream);
   }
   set_error("gemm: unsupported layout/epilogue/output combination");
   return AXN_EINVAL;
+}
+}  // namespace
+
+int launch_gemm_bf16(GemmLayout layout, const GemmArgs& g, int epilogue,
+                     bool out_f32, hipStream_t stream) {
+  return launch_layout<false>(layout, g, epilogue, out_f32, stream);
+}
+
+int launch_gemm_f16(GemmLayout layout, const GemmArgs& g, int epilogue, bool out_f32,
+                    hipStream_t stream) {
+  return launch_layout<true>(layout, g, epilogue, out_f32, stream);
 }
 
 }  // namespace axn

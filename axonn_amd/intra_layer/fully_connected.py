@@ -10,7 +10,7 @@ autograd function and its argument list (:96-108), autocast behaviour
 (:32-54), and `skip_bias_add` (:345-346).
 
 What differs: `Y = X W^T`, `dX = dY W` and `dW = dY^T X` (:118, :140, :147-151)
-run as bf16 MFMA kernels (fp32 kernels for fp32 layers); the bias add (:348)
+run as bf16 or fp16 MFMA kernels (fp32 kernels for fp32 layers); the bias add (:348)
 and, on request, the GELU that callers place after the layer are fused into the
 forward kernel's epilogue; with `optimize_communication(overlap_reduce_scatter=
 True)` the weight gradient is accumulated into `weight.grad` by the wgrad kernel
@@ -79,10 +79,8 @@ def _weight_grad(grad_2d, input_2d, original_weight):
     """dW = dY^T X in the parameter's dtype, flat, either returned to autograd or
     - under overlap_reduce_scatter - accumulated straight into weight.grad."""
     out_dtype = original_weight.dtype
-    if out_dtype not in (torch.float32, torch.bfloat16) or (
-        grad_2d.dtype == torch.float32 and out_dtype != torch.float32
-    ):
-        out_dtype = grad_2d.dtype
+    if out_dtype not in (torch.float32, grad_2d.dtype):
+        out_dtype = grad_2d.dtype  # the kernels write dW in the operands' type or in fp32
     if overlap_communication.OVERLAP_REDUCE_SCATTER:
         grad = original_weight.grad
         fusable = (

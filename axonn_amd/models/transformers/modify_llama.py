@@ -66,7 +66,7 @@ def modified_mlp_init(self, config):
 def modified_mlp_forward(self, x):
     gate, up = self.gate_proj(x), self.up_proj(x)
     if getattr(self, "_axonn_fused_swiglu", False) and gate.is_cuda and gate.dtype == up.dtype \
-            and gate.dtype in (torch.bfloat16, torch.float32):
+            and gate.dtype in (torch.bfloat16, torch.float16, torch.float32):
         return self.down_proj(swiglu(gate, up))
     return self.down_proj(self.act_fn(gate) * up)
 

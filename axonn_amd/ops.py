@@ -50,8 +50,12 @@ def _prep_bf16(t):
 
 
 # ------------------------------------------------------------------ GEMMs ----
+# 16-bit operand types of the MFMA kernels -> suffix of their entry points
+_GEMM16 = {torch.bfloat16: "", torch.float16: "_f16"}
+
+
 def gemm_fwd(x, w, bias=None, activation=None, save_z=False):
-    """Y = act(X W^T + b).  x [M,K], w [N,K]; bf16 or fp32 (both the same).
+    """Y = act(X W^T + b).  x [M,K], w [N,K]; bf16, fp16 or fp32 (both the same).
     Returns (y, z) with z the saved pre-activation (None unless activation and
     save_z)."""
     _require_gpu(x, w, bias)
@@ -67,12 +71,12 @@ def gemm_fwd(x, w, bias=None, activation=None, save_z=False):
         if bias.numel() != N:
             raise ValueError("bias has %d elements, expected %d" % (bias.numel(), N))
     want_z = activation is not None and save_z
-    if x.dtype == torch.bfloat16:
+    if x.dtype in _GEMM16:
         x, ldx = _prep_bf16(x)
         w, ldw = _prep_bf16(w)
-        y = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
+        y = torch.empty((M, N), dtype=x.dtype, device=x.device)
         z = torch.empty_like(y) if want_z else None
-        nv.call("axn_gemm_fwd", nv.ptr(x), nv.ptr(w), nv.ptr(bias), nv.ptr(y), nv.ptr(z),
+        nv.call("axn_gemm_fwd" + _GEMM16[x.dtype], nv.ptr(x), nv.ptr(w), nv.ptr(bias), nv.ptr(y), nv.ptr(z),
                 M, N, K, ldx, ldw, N, epi, nv.current_stream())
     elif x.dtype == torch.float32:
         x, w = x.contiguous(), w.contiguous()
@@ -81,7 +85,7 @@ def gemm_fwd(x, w, bias=None, activation=None, save_z=False):
         nv.call("axn_gemm_fwd_f32", nv.ptr(x), nv.ptr(w), nv.ptr(bias), nv.ptr(y), nv.ptr(z),
                 M, N, K, epi, nv.current_stream())
     else:
-        raise TypeError("the Linear kernels take bf16 or fp32 operands, got %s" % x.dtype)
+        raise TypeError("the Linear kernels take bf16, fp16 or fp32 operands, got %s" % x.dtype)
     return y, z
 
 
@@ -92,11 +96,11 @@ def gemm_dgrad(dy, w):
         raise TypeError("grad_output is %s but weight is %s" % (dy.dtype, w.dtype))
     M, N = dy.shape
     K = w.shape[1]
-    if dy.dtype == torch.bfloat16:
+    if dy.dtype in _GEMM16:
         dy, lddy = _prep_bf16(dy)
         w, ldw = _prep_bf16(w)
-        dx = torch.empty((M, K), dtype=torch.bfloat16, device=dy.device)
-        nv.call("axn_gemm_dgrad", nv.ptr(dy), nv.ptr(w), nv.ptr(dx), M, N, K, lddy, ldw, K,
+        dx = torch.empty((M, K), dtype=dy.dtype, device=dy.device)
+        nv.call("axn_gemm_dgrad" + _GEMM16[dy.dtype], nv.ptr(dy), nv.ptr(w), nv.ptr(dx), M, N, K, lddy, ldw, K,
                 nv.current_stream())
     elif dy.dtype == torch.float32:
         dy, w = dy.contiguous(), w.contiguous()
@@ -104,7 +108,7 @@ def gemm_dgrad(dy, w):
         nv.call("axn_gemm_dgrad_f32", nv.ptr(dy), nv.ptr(w), nv.ptr(dx), M, N, K,
                 nv.current_stream())
     else:
-        raise TypeError("the Linear kernels take bf16 or fp32 operands, got %s" % dy.dtype)
+        raise TypeError("the Linear kernels take bf16, fp16 or fp32 operands, got %s" % dy.dtype)
     return dx
 
 
@@ -124,14 +128,14 @@ def gemm_wgrad(dy, x, out=None, accumulate=False, out_dtype=None):
         raise ValueError("accumulate=True needs `out`")
     if out_dtype is None:
         out_dtype = dy.dtype
-    if dy.dtype == torch.bfloat16:
-        if out_dtype not in (torch.bfloat16, torch.float32):
-            raise TypeError("dW must be bf16 or fp32, got %s" % out_dtype)
+    if dy.dtype in _GEMM16:
+        if out_dtype not in (dy.dtype, torch.float32):
+            raise TypeError("dW must be %s or fp32, got %s" % (dy.dtype, out_dtype))
         dy, lddy = _prep_bf16(dy)
         x, ldx = _prep_bf16(x)
         if out is None:
             out = torch.empty((N, K), dtype=out_dtype, device=dy.device)
-        nv.call("axn_gemm_wgrad", nv.ptr(dy), nv.ptr(x), nv.ptr(out), M, N, K, lddy, ldx, K,
+        nv.call("axn_gemm_wgrad" + _GEMM16[dy.dtype], nv.ptr(dy), nv.ptr(x), nv.ptr(out), M, N, K, lddy, ldx, K,
                 1 if accumulate else 0, nv.dtype_code(out_dtype), nv.current_stream())
     elif dy.dtype == torch.float32:
         if out_dtype != torch.float32:
@@ -142,7 +146,7 @@ def gemm_wgrad(dy, x, out=None, accumulate=False, out_dtype=None):
         nv.call("axn_gemm_wgrad_f32", nv.ptr(dy), nv.ptr(x), nv.ptr(out), M, N, K,
                 1 if accumulate else 0, nv.current_stream())
     else:
-        raise TypeError("the Linear kernels take bf16 or fp32 operands, got %s" % dy.dtype)
+        raise TypeError("the Linear kernels take bf16, fp16 or fp32 operands, got %s" % dy.dtype)
     return out
 
 
@@ -150,8 +154,8 @@ def dgelu_dbias(dy, z=None, want_dbias=True, dbias_out=None, accumulate=False):
     """dZ = dY * gelu'(Z) (when z is given) and dbias = column sums of dZ (fp32).
     Returns (dz, dbias); dz is dy itself when z is None."""
     _require_gpu(dy, z, dbias_out)
-    if dy.dtype not in (torch.bfloat16, torch.float32):
-        raise TypeError("bf16 or fp32 expected, got %s" % dy.dtype)
+    if dy.dtype not in (torch.bfloat16, torch.float16, torch.float32):
+        raise TypeError("bf16, fp16 or fp32 expected, got %s" % dy.dtype)
     dy, ld = _rows(dy)
     if dy.data_ptr() % 16 or ld % 8:
         dy = dy.contiguous().clone()
@@ -190,8 +194,8 @@ def _same_2d(name, ref, *others):
 
 def _swiglu_operands(name, tensors):
     ref = tensors[0]
-    if ref.dtype not in (torch.bfloat16, torch.float32):
-        raise TypeError("%s: bf16 or fp32 expected, got %s" % (name, ref.dtype))
+    if ref.dtype not in (torch.bfloat16, torch.float16, torch.float32):
+        raise TypeError("%s: bf16, fp16 or fp32 expected, got %s" % (name, ref.dtype))
     if ref.dim() != 2 or ref.shape[1] % 8:
         raise ValueError("%s: 2-D operands with a multiple of 8 columns expected, got %s"
                          % (name, tuple(ref.shape)))

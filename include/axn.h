@@ -30,7 +30,7 @@
 extern "C" {
 #endif
 
-#define AXN_ABI_VERSION 3
+#define AXN_ABI_VERSION 4
 
 #if defined(__GNUC__)
 #define AXN_API __attribute__((visibility("default")))
@@ -104,7 +104,7 @@ AXN_API int axn_gemm_wgrad(const void* dY, const void* X, void* dW, int64_t M,
  *   dZ = dY * gelu'(Z)   (Z = NULL: dZ is not written, dbias = colsum(dY))
  *   dbias[n] = beta * dbias[n] + sum_m dZ[m,n]        (dbias NULL: skipped)
  * Replaces what autograd derives from `x + bias` (fully_connected.py:348)
- * and from the caller's nn.GELU.  dY, Z, dZ are of `dtype` (AXN_BF16 or
+ * and from the caller's nn.GELU.  dY, Z, dZ are of `dtype` (AXN_BF16, AXN_F16 or
  * AXN_F32), row stride ld; dbias is fp32.  N % 8 == 0, pointers 16-byte
  * aligned, ld % 8 == 0.  Deterministic: column partial sums go through
  * `workspace` (axn_dgelu_dbias_workspace_bytes, needed only when dbias is
@@ -114,13 +114,28 @@ AXN_API int axn_dgelu_dbias(const void* dY, const void* Z, void* dZ, int dtype,
                     void* workspace, size_t workspace_bytes, void* stream);
 AXN_API size_t axn_dgelu_dbias_workspace_bytes(int64_t M, int64_t N);
 
+/* The three GEMMs on IEEE half operands (the reference's default mixed
+ * precision is fp16 autocast with a loss scaler: axonn/axonn.py:21-67,
+ * axonn/inter_layer.py:274-302).  Same arguments, requirements and kernels as
+ * axn_gemm_fwd / _dgrad / _wgrad with every bf16 operand and result fp16
+ * instead; fp32 accumulate; dw_dtype AXN_F16 or AXN_F32. */
+AXN_API int axn_gemm_fwd_f16(const void* X, const void* W, const float* bias, void* Y,
+                     void* Zsave, int64_t M, int64_t N, int64_t K, int64_t ldx,
+                     int64_t ldw, int64_t ldy, int epilogue, void* stream);
+AXN_API int axn_gemm_dgrad_f16(const void* dY, const void* W, void* dX, int64_t M,
+                       int64_t N, int64_t K, int64_t lddy, int64_t ldw, int64_t lddx,
+                       void* stream);
+AXN_API int axn_gemm_wgrad_f16(const void* dY, const void* X, void* dW, int64_t M,
+                       int64_t N, int64_t K, int64_t lddy, int64_t ldx, int64_t lddw,
+                       int beta, int dw_dtype, void* stream);
+
 /* SwiGLU activation of the Llama MLP, one pass over [M,N]:
  *   out = silu(gate) * up,  silu(x) = x / (1 + exp(-x)).
  * The reference's Llama patch (axonn/models/transformers/modify_llama.py:76-95)
  * replaces gate_proj / up_proj / down_proj by its Linear and leaves
  * `act_fn(gate_proj(x)) * up_proj(x)` of the model's forward to two elementwise
  * kernels; this entry point and the next replace those and their autograd.
- * gate, up, out of `dtype` (AXN_BF16 or AXN_F32), row stride ld; N % 8 == 0,
+ * gate, up, out of `dtype` (AXN_BF16, AXN_F16 or AXN_F32), row stride ld; N % 8 == 0,
  * ld % 8 == 0, pointers 16-byte aligned.  Computed in fp32, rounded once.
  * out may alias gate or up. */
 AXN_API int axn_swiglu_fwd(const void* gate, const void* up, void* out, int dtype,

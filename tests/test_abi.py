@@ -75,6 +75,12 @@ def test_gemm_argument_errors():
     assert lib.axn_gemm_dgrad(A, A, None, 8, 8, 8, 8, 8, 8, None) == nv.AXN_EINVAL
     assert lib.axn_gemm_wgrad(A, A, A, 8, 8, 8, 8, 8, 8, 2, nv.BF16, None) == nv.AXN_EINVAL
     assert lib.axn_gemm_wgrad(A, A, A, 8, 8, 8, 8, 8, 8, 0, nv.F16, None) == nv.AXN_EINVAL
+    # the fp16 entry points share the checks; dW there is fp16 or fp32, never bf16
+    assert lib.axn_gemm_fwd_f16(A, A, None, A, None, 8, 12, 8, 8, 8, 16, 0, None) == nv.AXN_ESHAPE
+    assert "axn_gemm_fwd_f16" in _err()
+    assert lib.axn_gemm_dgrad_f16(A, None, A, 8, 8, 8, 8, 8, 8, None) == nv.AXN_EINVAL
+    assert lib.axn_gemm_wgrad_f16(A, A, A, 8, 8, 8, 8, 8, 8, 0, nv.BF16, None) == nv.AXN_EINVAL
+    assert "fp16 or fp32" in _err()
     assert lib.axn_gemm_fwd_f32(A, None, None, A, None, 4, 4, 4, 0, None) == nv.AXN_EINVAL
     assert lib.axn_gemm_wgrad_f32(A, A, A, 4, 4, 4, 3, None) == nv.AXN_EINVAL
     assert lib.axn_gemm_dgrad_f32(ctypes.c_void_p(0x1002), A, A, 4, 4, 4, None) == nv.AXN_EALIGN
@@ -84,7 +90,7 @@ def test_swiglu_argument_errors():
     lib = nv.load()
     f, b = lib.axn_swiglu_fwd, lib.axn_swiglu_bwd
     assert f(None, A, A, nv.BF16, 8, 8, 8, None) == nv.AXN_EINVAL
-    assert f(A, A, A, nv.F16, 8, 8, 8, None) == nv.AXN_EINVAL
+    assert f(A, A, A, 7, 8, 8, 8, None) == nv.AXN_EINVAL
     assert f(A, A, A, nv.BF16, 8, 12, 16, None) == nv.AXN_ESHAPE
     assert f(A, A, A, nv.BF16, 8, 8, 4, None) == nv.AXN_EALIGN          # ld < N
     assert f(ctypes.c_void_p(0x1008), A, A, nv.BF16, 8, 8, 8, None) == nv.AXN_EALIGN
@@ -130,7 +136,7 @@ def test_elementwise_argument_errors():
     assert f(None, None, None, nv.BF16, A, 8, 8, 8, 0, A, 1024, None) == nv.AXN_EINVAL
     assert f(A, A, None, nv.BF16, A, 8, 8, 8, 0, A, 1024, None) == nv.AXN_EINVAL  # Z without dZ
     assert f(A, None, None, nv.BF16, None, 8, 8, 8, 0, A, 1024, None) == nv.AXN_EINVAL  # nothing to do
-    assert f(A, None, None, nv.F16, A, 8, 8, 8, 0, A, 1024, None) == nv.AXN_EINVAL
+    assert f(A, None, None, 7, A, 8, 8, 8, 0, A, 1024, None) == nv.AXN_EINVAL
     assert f(A, None, None, nv.BF16, A, 8, 12, 16, 0, A, 1024, None) == nv.AXN_ESHAPE
     assert f(A, None, None, nv.BF16, A, 8, 8, 8, 0, A, 4, None) == nv.AXN_EINVAL  # workspace too small
     assert "workspace" in _err()

@@ -194,8 +194,10 @@ def test_unsupported_shapes_raise():
     with pytest.raises(nv.AxnError, match="multiples of 8") as e:
         ops.gemm_fwd(X, W)
     assert e.value.code == nv.AXN_ESHAPE
-    with pytest.raises(TypeError):
+    with pytest.raises(nv.AxnError, match="axn_gemm_fwd_f16: N and K must be multiples of 8"):
         ops.gemm_fwd(X.half(), W.half())
+    with pytest.raises(TypeError, match="bf16, fp16 or fp32"):
+        ops.gemm_fwd(X.double(), W.double())
     with pytest.raises(TypeError):
         ops.gemm_fwd(X, W.float())
 

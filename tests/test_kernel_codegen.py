@@ -26,10 +26,11 @@ def gemm_asm(tmp_path_factory):
     subprocess.run(cmd, check=True, capture_output=True, timeout=900)
     text = out.read_text()
     kernels = {}
-    for m in re.finditer(r"^(_ZN3axn\S*gemm_bf16_solo_kernel\S*):", text, re.M):
+    for m in re.finditer(r"^(_ZN3axn\S*gemm_(?:bf16|f16)_solo_kernel\S*):", text, re.M):
         end = text.index(".end_amdhsa_kernel", m.end())
         kernels[m.group(1)] = text[m.end():end]
-    assert len(kernels) >= 14, sorted(kernels)   # 7 layout/epilogue/output variants x 2 tile sizes
+    # 7 layout/epilogue/output variants x 2 tile sizes x 2 element types
+    assert len(kernels) >= 28, sorted(kernels)
     return kernels
 
 
@@ -71,7 +72,8 @@ def test_main_loop_mfma_operands_have_fixed_register_classes(gemm_asm):
     """Accumulators in AGPRs, fragments in VGPRs, for every MFMA of every variant."""
     for name, body in gemm_asm.items():
         for s in _instructions(body):
-            if s.startswith("v_mfma_f32_16x16x32_bf16"):
+            if s.startswith("v_mfma_f32_16x16x32_"):
+                assert s.split()[0].endswith("_f16" if "gemm_f16_solo" in name else "_bf16"), (name, s)
                 ops = [o.strip() for o in s.split(None, 1)[1].split(",")]
                 assert ops[0].startswith("a[") and ops[3].startswith("a[") and ops[0] == ops[3], (name, s)
                 assert ops[1].startswith("v[") and ops[2].startswith("v["), (name, s)

@@ -75,7 +75,7 @@ def test_swiglu_rejects_bad_arguments():
     with pytest.raises(ValueError):
         ops.swiglu_fwd(b, b.float())
     with pytest.raises(TypeError):
-        ops.swiglu_fwd(b.half(), b.half())
+        ops.swiglu_fwd(b.double(), b.double())
     with pytest.raises(RuntimeError):
         ops.swiglu_fwd(b.cpu(), b.cpu())
 
