@@ -83,16 +83,12 @@ __global__ void __launch_bounds__(256)
 }
 
 // ---- backward ------------------------------------------------------------------
+// One 16-byte vector of a table row as fp32 values.
 template <typename T>
 struct Vec;
 template <>
 struct Vec<float> {
   static constexpr int N = 4;
-  static __device__ __forceinline__ void load(const float* p, float (&x)[4]) {
-    const f32x4 v = __builtin_nontemporal_load((const f32x4*)p);
-#pragma unroll
-    for (int e = 0; e < 4; ++e) x[e] = v[e];
-  }
   static __device__ __forceinline__ void load_cached(const float* p, float (&x)[4]) {
     const f32x4 v = *(const f32x4*)p;
 #pragma unroll
@@ -105,11 +101,6 @@ struct Vec<float> {
 template <>
 struct Vec<uint16_t> {
   static constexpr int N = 8;
-  static __device__ __forceinline__ void load(const uint16_t* p, float (&x)[8]) {
-    const bf16x8 v = __builtin_nontemporal_load((const bf16x8*)p);
-#pragma unroll
-    for (int e = 0; e < 8; ++e) x[e] = (float)v[e];
-  }
   static __device__ __forceinline__ void load_cached(const uint16_t* p, float (&x)[8]) {
     const bf16x8 v = *(const bf16x8*)p;
 #pragma unroll

@@ -106,7 +106,34 @@ def optimizer_cases():
     np.savez_compressed(os.path.join(HERE, "optimizer_f32.npz"), **out)
 
 
+def embedding_cases():
+    """torch's CPU F.embedding (the call at axonn/intra_layer/embedding.py:164-172) and its
+    autograd in float64 on fp32-representable inputs, ids drawn as the reference's test
+    draws them (randint over the vocabulary; here a small one, so that ids repeat), with
+    each flag of the call exercised once."""
+    g = torch.Generator().manual_seed(2024)
+    V, H, B, S = 97, 24, 4, 50
+    out = {}
+    W = torch.randn(V, H, generator=g).double()
+    ids = torch.randint(0, V, (B, S), generator=g)
+    dY = (torch.randn(B, S, H, generator=g) * 0.01).double()
+    out["ids"], out["W"], out["dY"] = ids.numpy(), W.numpy().astype(np.float32), dY.numpy().astype(np.float32)
+    for tag, kw in (("plain", {}), ("pad", {"padding_idx": 5}),
+                    ("freq", {"padding_idx": 5, "scale_grad_by_freq": True})):
+        w = W.clone().requires_grad_(True)
+        y = torch.nn.functional.embedding(ids, w, **kw)
+        y.backward(dY)
+        out[tag + "_Y"] = y.detach().numpy()
+        out[tag + "_dW"] = w.grad.numpy()
+    w = W.clone()
+    torch.nn.functional.embedding(ids[:1, :20], w, max_norm=3.0, norm_type=2.0)
+    out["renorm_ids"] = ids[:1, :20].numpy()
+    out["renorm_W"] = w.numpy()
+    np.savez_compressed(os.path.join(HERE, "embedding_f64.npz"), **out)
+
+
 if __name__ == "__main__":
     linear_cases()
     optimizer_cases()
+    embedding_cases()
     print("wrote", sorted(f for f in os.listdir(HERE) if f.endswith(".npz")))

@@ -181,3 +181,60 @@ def test_hip_optimizer_reproduces_golden(opt):
         # the low-precision copy is exactly the rounding of the master weights
         want_bits = ol.bf16_bits(got)
         assert np.array_equal(flat_pl.view(torch.int16).cpu().numpy().view(np.uint16), want_bits)
+
+
+# ------------------------------------------------------------------ embedding
+@pytest.fixture(scope="module")
+def emb(golden_dir):
+    return np.load(os.path.join(golden_dir, "embedding_f64.npz"))
+
+
+EMB_CASES = [("plain", None, False), ("pad", 5, False), ("freq", 5, True)]
+
+
+@pytest.mark.parametrize("tag,padding_idx,scale", EMB_CASES)
+def test_oracle_embedding_reproduces_golden(emb, tag, padding_idx, scale):
+    """The fixture holds torch's float64 results; the oracle adds in fp32 in token order,
+    so it agrees to fp32 rounding of sums of at most 8 terms of size 0.01."""
+    from oracle import embedding as oe
+
+    V = emb["W"].shape[0]
+    assert np.array_equal(oe.embedding_forward(emb["ids"], emb["W"]), emb[tag + "_Y"].astype(np.float32))
+    dW = oe.embedding_backward(emb["ids"], emb["dY"], V, padding_idx, scale)
+    assert np.allclose(dW, emb[tag + "_dW"], rtol=1e-6, atol=1e-9)
+    assert np.allclose(oe.embedding_backward_f64(emb["ids"], emb["dY"], V, padding_idx, scale),
+                       emb[tag + "_dW"], rtol=1e-12, atol=1e-15)
+    if padding_idx is not None:
+        assert (emb["ids"] == padding_idx).any() and not emb[tag + "_dW"][padding_idx].any()
+
+
+def test_oracle_embedding_renorm_reproduces_golden(emb):
+    from oracle import embedding as oe
+
+    got = oe.embedding_renorm(emb["W"], emb["renorm_ids"], 3.0, 2.0)
+    assert np.allclose(got, emb["renorm_W"], rtol=1e-12, atol=1e-15)
+    assert not np.array_equal(got, emb["W"].astype(np.float64))  # some rows were clipped
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("tag,padding_idx,scale", EMB_CASES)
+def test_hip_embedding_reproduces_golden(emb, tag, padding_idx, scale):
+    from axonn_amd import ops
+
+    V = emb["W"].shape[0]
+    ids = torch.from_numpy(emb["ids"]).cuda()
+    W = torch.from_numpy(emb["W"]).cuda()
+    dY = torch.from_numpy(emb["dY"]).cuda()
+    y = ops.embedding_fwd(ids, W)
+    assert np.array_equal(y.cpu().numpy(), emb[tag + "_Y"].astype(np.float32))
+    dW = ops.embedding_bwd(ids, dY, V, padding_idx=padding_idx, scale_grad_by_freq=scale)
+    assert np.allclose(dW.cpu().numpy(), emb[tag + "_dW"], rtol=1e-6, atol=1e-9)
+
+
+@pytest.mark.gpu
+def test_hip_embedding_renorm_reproduces_golden(emb):
+    from axonn_amd import ops
+
+    W = torch.from_numpy(emb["W"].copy()).cuda()
+    ops.embedding_renorm_(W, torch.from_numpy(emb["renorm_ids"]).cuda(), 3.0, 2.0)
+    assert np.allclose(W.cpu().numpy(), emb["renorm_W"], rtol=2e-6, atol=1e-9)

@@ -251,3 +251,15 @@ def test_checkpoint_round_trip_under_the_rank_prefix(tmp_path):
     assert torch.equal(other.weight, layer.weight)
     with pytest.raises(AssertionError, match="does not exist"):
         checkpoint.load({}, str(tmp_path / "missing"), "ckpt")
+
+
+def test_bench_refuses_more_than_one_gpu():
+    import os
+    import subprocess
+    import sys
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    proc = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"],
+                          capture_output=True, text=True, timeout=120)
+    assert proc.returncode != 0
+    assert "ONE GPU" in proc.stderr and proc.stdout.strip() == ""
