@@ -222,10 +222,10 @@ def test_fp32_gemms_match_oracle(M, N, K):
 
 
 @pytest.mark.parametrize("M,N,K", [(128, 128, 64), (256, 384, 192), (512, 256, 320), (4096, 3072, 128),
-                                   (4096, 3072, 320)])
+                                   (4096, 3072, 320), (4608, 4096, 64)])
 def test_tile_kernels_every_output_block_with_epilogues(M, N, K):
     """Whole-tile shapes on the one-wave-per-SIMD kernel (128 x 128 tiles up to 128
-    tiles of 256 x 256, else 256 x 256), checked element by element so that a single
+    tiles of 256 x 256 and from 257 to 320 of them, else 256 x 256), checked element by element so that a single
     wrong 16 x 16 accumulator block shows (a block copied out of its registers before
     its last MFMA had finished once passed the normwise checks of other shapes)."""
     from axonn_amd import ops
