@@ -226,6 +226,91 @@ int axn_gemm_wgrad_f16(const void* dY, const void* X, void* dW, int64_t M, int64
                        dw_dtype, stream);
 }
 
+// ---- split-contraction variants --------------------------------------------------
+static void fill_gemm_args(GemmArgs& g, int op, const void* a, const void* b, void* c, int64_t M,
+                           int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc) {
+  g.A = (const uint16_t*)a;
+  g.B = (const uint16_t*)b;
+  g.C = c;
+  g.lda = lda;
+  g.ldb = ldb;
+  g.ldc = ldc;
+  if (op == AXN_GEMM_FWD) {  // Y[M,N] = X[M,K] W[N,K]^T
+    g.M = (int)M, g.N = (int)N, g.Kc = (int)K;
+  } else if (op == AXN_GEMM_DGRAD) {  // dX[M,K] = dY[M,N] W[N,K]
+    g.M = (int)M, g.N = (int)K, g.Kc = (int)N;
+  } else {  // dW[N,K] = dY[M,N]^T X[M,K]
+    g.M = (int)N, g.N = (int)K, g.Kc = (int)M;
+  }
+}
+
+static const GemmLayout kLayoutOfOp[3] = {GEMM_NT, GEMM_NN, GEMM_TN};
+
+size_t axn_gemm_workspace_bytes(int op, int64_t M, int64_t N, int64_t K) {
+  if (op < AXN_GEMM_FWD || op > AXN_GEMM_WGRAD || M < 1 || N < 1 || K < 1 || M > 0x7fffffff ||
+      N > 0x7fffffff || K > 0x7fffffff)
+    return 0;
+  GemmArgs g = {};
+  // dense operands: the leading dimensions are the row lengths
+  fill_gemm_args(g, op, nullptr, nullptr, nullptr, M, N, K, op == AXN_GEMM_FWD ? K : N, K,
+                 op == AXN_GEMM_FWD ? N : K);
+  const int s = gemm_splits(kLayoutOfOp[op], g);
+  return s > 1 ? (size_t)s * (size_t)g.M * (size_t)g.N * sizeof(float) : 0;
+}
+
+static int gemm_ws(const char* name, int op, const void* a, const void* b, void* c, int dtype,
+                   int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc, int beta,
+                   int out_dtype, void* workspace, size_t workspace_bytes, void* stream) {
+  REQUIRE(dtype == AXN_BF16 || dtype == AXN_F16, AXN_EINVAL, "%s: dtype must be bf16 or fp16", name);
+  const bool half = dtype == AXN_F16;
+  int rc;
+  if (op == AXN_GEMM_FWD)
+    rc = check_gemm(name, a, b, c, M, N, K, lda, ldb, ldc, K, K, N);
+  else
+    rc = check_gemm(name, a, b, c, M, N, K, lda, ldb, ldc, N, K, K);
+  if (rc) return rc;
+  REQUIRE(beta == 0 || beta == 1, AXN_EINVAL, "%s: beta must be 0 or 1", name);
+  REQUIRE(out_dtype == dtype || (op == AXN_GEMM_WGRAD && out_dtype == AXN_F32), AXN_EINVAL,
+          "%s: unsupported output type", name);
+  GemmArgs g = {};
+  fill_gemm_args(g, op, a, b, c, M, N, K, lda, ldb, ldc);
+  g.beta = beta;
+  const GemmLayout layout = kLayoutOfOp[op];
+  const int splits = (workspace != nullptr) ? gemm_splits(layout, g) : 1;
+  if (splits > 1) {
+    const size_t need = (size_t)splits * (size_t)g.M * (size_t)g.N * sizeof(float);
+    REQUIRE(workspace_bytes >= need, AXN_EINVAL,
+            "%s: workspace too small (%zu bytes given, %zu needed)", name, workspace_bytes, need);
+    REQUIRE(aligned16(workspace), AXN_EALIGN, "%s: workspace must be 16-byte aligned", name);
+    return launch_gemm_splitk(layout, g, half, out_dtype, splits, (float*)workspace,
+                              (hipStream_t)stream);
+  }
+  return half ? launch_gemm_f16(layout, g, AXN_EPI_NONE, out_dtype == AXN_F32, (hipStream_t)stream)
+              : launch_gemm_bf16(layout, g, AXN_EPI_NONE, out_dtype == AXN_F32,
+                                 (hipStream_t)stream);
+}
+
+int axn_gemm_fwd_ws(const void* X, const void* W, void* Y, int dtype, int64_t M, int64_t N,
+                    int64_t K, int64_t ldx, int64_t ldw, int64_t ldy, void* workspace,
+                    size_t workspace_bytes, void* stream) {
+  return gemm_ws("axn_gemm_fwd_ws", AXN_GEMM_FWD, X, W, Y, dtype, M, N, K, ldx, ldw, ldy, 0, dtype,
+                 workspace, workspace_bytes, stream);
+}
+
+int axn_gemm_dgrad_ws(const void* dY, const void* W, void* dX, int dtype, int64_t M, int64_t N,
+                      int64_t K, int64_t lddy, int64_t ldw, int64_t lddx, void* workspace,
+                      size_t workspace_bytes, void* stream) {
+  return gemm_ws("axn_gemm_dgrad_ws", AXN_GEMM_DGRAD, dY, W, dX, dtype, M, N, K, lddy, ldw, lddx, 0,
+                 dtype, workspace, workspace_bytes, stream);
+}
+
+int axn_gemm_wgrad_ws(const void* dY, const void* X, void* dW, int dtype, int64_t M, int64_t N,
+                      int64_t K, int64_t lddy, int64_t ldx, int64_t lddw, int beta, int dw_dtype,
+                      void* workspace, size_t workspace_bytes, void* stream) {
+  return gemm_ws("axn_gemm_wgrad_ws", AXN_GEMM_WGRAD, dY, X, dW, dtype, M, N, K, lddy, ldx, lddw,
+                 beta, dw_dtype, workspace, workspace_bytes, stream);
+}
+
 size_t axn_dgelu_dbias_workspace_bytes(int64_t M, int64_t N) {
   return dgelu_dbias_workspace_bytes(M, N);
 }

@@ -67,6 +67,10 @@ struct GemmArgs {
   int64_t lda, ldb, ldc;
   int tiles_m, tiles_n;
   int beta;  // 0: C = AB ; 1: C += AB
+  // Split of the contraction over workgroups (splits > 1): workgroup id / tiles is the
+  // split, which covers k_split contraction elements and writes its fp32 partial
+  // product to C + split * M * ldc.  0 or 1: no split.
+  int splits, k_split;
 };
 
 enum GemmLayout { GEMM_NT = 0, GEMM_NN = 1, GEMM_TN = 2 };
@@ -79,6 +83,14 @@ int launch_gemm_bf16(GemmLayout layout, const GemmArgs& args, int epilogue,
 // The same kernels on IEEE half operands (v_mfma_f32_16x16x32_f16, half outputs).
 int launch_gemm_f16(GemmLayout layout, const GemmArgs& args, int epilogue, bool out_f32,
                     hipStream_t stream);
+// Split-contraction variant for problems with few output tiles: the number of splits
+// chosen for an [M x N] output over a contraction of Kc (1 = do not split), and the
+// launch: partial products in fp32 to `ws` (splits * M * N floats), then one pass that
+// adds them in split order, adds the old output if args.beta, and stores args.C in
+// out_dtype.  No epilogue.
+int gemm_splits(GemmLayout layout, const GemmArgs& args);
+int launch_gemm_splitk(GemmLayout layout, const GemmArgs& args, bool half, int out_dtype,
+                       int splits, float* ws, hipStream_t stream);
 
 // ---- fp32 GEMM (full-precision layers) --------------------------------------
 int launch_gemm_f32(GemmLayout layout, const float* A, const float* B, float* C,

@@ -462,8 +462,13 @@ __device__ __forceinline__ void solo_gemm(const GemmArgs& g) {
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave >> 1, wn = wave & 1;
 
+  int pid = blockIdx.x, split = 0;
+  if (g.splits > 1) {
+    split = pid / (g.tiles_m * g.tiles_n);
+    pid -= split * (g.tiles_m * g.tiles_n);
+  }
   int tm, tn;
-  tile_of_workgroup(blockIdx.x, g.tiles_m, g.tiles_n, tm, tn);
+  tile_of_workgroup(pid, g.tiles_m, g.tiles_n, tm, tn);
   const int m0 = tm * BM, n0 = tn * BN;
 
   f32x4 acc[FR][FR];
@@ -472,7 +477,7 @@ __device__ __forceinline__ void solo_gemm(const GemmArgs& g) {
 #pragma unroll
     for (int j = 0; j < FR; ++j) acc[i][j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
 
-  const int KP = g.Kc / PK;  // stages
+  const int KP = (g.splits > 1 ? g.k_split : g.Kc) / PK;  // stages of this workgroup
   const uint32_t a_bytes = (uint32_t)((int64_t)(A_KMAJOR ? g.M : g.Kc) * g.lda * 2);
   const uint32_t b_bytes = (uint32_t)((int64_t)(B_KMAJOR ? g.N : g.Kc) * g.ldb * 2);
   const __amdgpu_buffer_rsrc_t ra_rsrc =
@@ -484,7 +489,8 @@ __device__ __forceinline__ void solo_gemm(const GemmArgs& g) {
   const uint32_t vb = OB::dma_offset(g.ldb, n0, wave, lane, b_is);
   const uint32_t a_step = (uint32_t)((A_KMAJOR ? (int64_t)PK : (int64_t)PK * g.lda) * 2);
   const uint32_t b_step = (uint32_t)((B_KMAJOR ? (int64_t)PK : (int64_t)PK * g.ldb) * 2);
-  uint32_t ka = 0, kb = 0;  // byte offsets of the next A / B tile to copy
+  // byte offsets of the next A / B tile to copy
+  uint32_t ka = (uint32_t)split * (uint32_t)KP * a_step, kb = (uint32_t)split * (uint32_t)KP * b_step;
   uint32_t wslot = 0;       // ring slot (byte offset) the next copied tile takes
 
   const uint32_t lds0 = (uint32_t)(uintptr_t)LDS_PTR(char, lds);
@@ -610,13 +616,15 @@ __device__ __forceinline__ void solo_gemm(const GemmArgs& g) {
   // instruction.
   const int orow = m0 + wm * WTM + (lane & 15);
   const int ocol = n0 + wn * WTN + 8 * (lane >> 4);
+  GemmArgs go = g;  // a split writes its own fp32 partial product
+  if (OUT_F32 && g.splits > 1) go.C = (float*)g.C + (int64_t)split * g.M * g.ldc;
 #pragma unroll
   for (int i = 0; i < FR; ++i)
 #pragma unroll
     for (int t = 0; t < FR / 2; ++t) {
       const f32x4 lo = acc[i][2 * t], hi = acc[i][2 * t + 1];
       float v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-      store_row8<EPI, OUT_F32, HALF>(v, g, orow + 16 * i, ocol + 32 * t);
+      store_row8<EPI, OUT_F32, HALF>(v, go, orow + 16 * i, ocol + 32 * t);
     }
 }
 
@@ -772,7 +780,9 @@ int launch_solo(const GemmArgs& in, hipStream_t stream) {
   if constexpr (HALF) kern = gemm_f16_solo_kernel<TILE, AK, BKM, EPI, OUT_F32>;
   AXN_HIP_TRY(hipFuncSetAttribute((const void*)kern,
                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-  hipLaunchKernelGGL(kern, dim3((unsigned)(g.tiles_m * g.tiles_n)), dim3(256), lds, stream, g);
+  const int splits = g.splits > 1 ? g.splits : 1;
+  hipLaunchKernelGGL(kern, dim3((unsigned)(g.tiles_m * g.tiles_n * splits)), dim3(256), lds, stream,
+                     g);
   AXN_HIP_TRY(hipGetLastError());
   return AXN_OK;
 }
@@ -810,6 +820,53 @@ int launch_shape(const GemmArgs& g, hipStream_t stream) {
 }  // namespace
 
 namespace {
+
+// Sum of the fp32 partial products of a split contraction, in split order, plus the
+// old output if beta; one 16-byte store (two for fp32) of 8 columns per lane.
+template <typename LP>
+__global__ void __launch_bounds__(256)
+    splitk_reduce_kernel(const float* __restrict__ ws, LP* out, int64_t M, int64_t N, int64_t ld,
+                         int splits, int beta) {
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int64_t per_row = N / 8;
+  if (idx >= M * per_row) return;
+  const int64_t row = idx / per_row, col = (idx - row * per_row) * 8;
+  const float* p = ws + row * N + col;
+  f32x4 a0 = __builtin_nontemporal_load((const f32x4*)p);
+  f32x4 a1 = __builtin_nontemporal_load((const f32x4*)(p + 4));
+  for (int s = 1; s < splits; ++s) {
+    p += M * N;
+    a0 += __builtin_nontemporal_load((const f32x4*)p);
+    a1 += __builtin_nontemporal_load((const f32x4*)(p + 4));
+  }
+  LP* o = out + row * ld + col;
+  if constexpr (sizeof(LP) == 4) {
+    if (beta) {
+      a0 += *(const f32x4*)o;
+      a1 += *(const f32x4*)(o + 4);
+    }
+    *(f32x4*)o = a0;
+    *(f32x4*)(o + 4) = a1;
+  } else {
+    typedef LP lpx8 __attribute__((ext_vector_type(8)));
+    float v[8] = {a0[0], a0[1], a0[2], a0[3], a1[0], a1[1], a1[2], a1[3]};
+    if (beta) {
+      const lpx8 old = *(const lpx8*)o;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v[e] += (float)old[e];
+    }
+    lpx8 y;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) y[e] = (LP)v[e];
+    *(lpx8*)o = y;
+  }
+}
+
+template <bool AK, bool BKM, bool HALF>
+int launch_split(const GemmArgs& g, hipStream_t stream) {
+  return launch_solo<128, AK, BKM, AXN_EPI_NONE, true, HALF>(g, stream);
+}
+
 template <bool HALF>
 int launch_layout(GemmLayout layout, const GemmArgs& g, int epilogue, bool out_f32,
                   hipStream_t stream) {
@@ -848,6 +905,63 @@ int launch_gemm_bf16(GemmLayout layout, const GemmArgs& g, int epilogue,
 int launch_gemm_f16(GemmLayout layout, const GemmArgs& g, int epilogue, bool out_f32,
                     hipStream_t stream) {
   return launch_layout<true>(layout, g, epilogue, out_f32, stream);
+}
+
+// Few output tiles leave most CUs without work: 128 x 128 tiles times splits of the
+// contraction, up to two workgroups per CU (512), each split at least 512 deep.
+// Only below 129 tiles: with a workgroup on every second CU or more, the second pass
+// costs more than the split gains (measured at 256 tiles: 35 -> 44 us).
+int gemm_splits(GemmLayout layout, const GemmArgs& g) {
+  if (g.M % 128 || g.N % 128 || g.Kc % 64) return 1;
+  const bool ak = layout != GEMM_TN, bkm = layout == GEMM_NT;
+  const int64_t a_span = (int64_t)(ak ? g.M : g.Kc) * g.lda * 2;
+  const int64_t b_span = (int64_t)(bkm ? g.N : g.Kc) * g.ldb * 2;
+  if (a_span >= (1LL << 31) || b_span >= (1LL << 31)) return 1;
+  const long long tiles = (long long)(g.M / 128) * (g.N / 128);
+  if (tiles > 128) return 1;
+  for (int s = 8; s >= 2; s >>= 1)
+    if (tiles * s <= 512 && g.Kc % (64 * s) == 0 && g.Kc / s >= 512) return s;
+  return 1;
+}
+
+int launch_gemm_splitk(GemmLayout layout, const GemmArgs& in, bool half, int out_dtype,
+                       int splits, float* ws, hipStream_t stream) {
+  GemmArgs g = in;
+  g.C = ws;
+  g.ldc = g.N;
+  g.beta = 0;
+  g.bias = nullptr;
+  g.Z = nullptr;
+  g.splits = splits;
+  g.k_split = g.Kc / splits;
+  int rc;
+  switch (layout) {
+    case GEMM_NT:
+      rc = half ? launch_split<true, true, true>(g, stream)
+                : launch_split<true, true, false>(g, stream);
+      break;
+    case GEMM_NN:
+      rc = half ? launch_split<true, false, true>(g, stream)
+                : launch_split<true, false, false>(g, stream);
+      break;
+    default:
+      rc = half ? launch_split<false, false, true>(g, stream)
+                : launch_split<false, false, false>(g, stream);
+  }
+  if (rc) return rc;
+  const int64_t lanes = (int64_t)in.M * (in.N / 8);
+  const dim3 grid((unsigned)((lanes + 255) / 256)), block(256);
+  if (out_dtype == AXN_F32)
+    hipLaunchKernelGGL(splitk_reduce_kernel<float>, grid, block, 0, stream, ws, (float*)in.C,
+                       (int64_t)in.M, (int64_t)in.N, in.ldc, splits, in.beta);
+  else if (out_dtype == AXN_F16)
+    hipLaunchKernelGGL(splitk_reduce_kernel<_Float16>, grid, block, 0, stream, ws, (_Float16*)in.C,
+                       (int64_t)in.M, (int64_t)in.N, in.ldc, splits, in.beta);
+  else
+    hipLaunchKernelGGL(splitk_reduce_kernel<__bf16>, grid, block, 0, stream, ws, (__bf16*)in.C,
+                       (int64_t)in.M, (int64_t)in.N, in.ldc, splits, in.beta);
+  AXN_HIP_TRY(hipGetLastError());
+  return AXN_OK;
 }
 
 }  // namespace axn

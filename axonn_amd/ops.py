@@ -52,6 +52,16 @@ def _prep_bf16(t):
 # ------------------------------------------------------------------ GEMMs ----
 # 16-bit operand types of the MFMA kernels -> suffix of their entry points
 _GEMM16 = {torch.bfloat16: "", torch.float16: "_f16"}
+GEMM_FWD, GEMM_DGRAD, GEMM_WGRAD = 0, 1, 2
+
+
+def _split_workspace(op, M, N, K, device):
+    """Workspace for a GEMM whose contraction the library would split over workgroups
+    (few output tiles), or (None, 0)."""
+    nbytes = nv.load().axn_gemm_workspace_bytes(op, M, N, K)
+    if nbytes == 0:
+        return None, 0
+    return torch.empty(nbytes, dtype=torch.uint8, device=device), nbytes
 
 
 def gemm_fwd(x, w, bias=None, activation=None, save_z=False):
@@ -75,6 +85,12 @@ def gemm_fwd(x, w, bias=None, activation=None, save_z=False):
         x, ldx = _prep_bf16(x)
         w, ldw = _prep_bf16(w)
         y = torch.empty((M, N), dtype=x.dtype, device=x.device)
+        ws, ws_bytes = _split_workspace(GEMM_FWD, M, N, K, x.device) if epi == nv.EPI_NONE \
+            else (None, 0)
+        if ws is not None:
+            nv.call("axn_gemm_fwd_ws", nv.ptr(x), nv.ptr(w), nv.ptr(y), nv.dtype_code(x.dtype),
+                    M, N, K, ldx, ldw, N, nv.ptr(ws), ws_bytes, nv.current_stream())
+            return y, None
         z = torch.empty_like(y) if want_z else None
         nv.call("axn_gemm_fwd" + _GEMM16[x.dtype], nv.ptr(x), nv.ptr(w), nv.ptr(bias), nv.ptr(y), nv.ptr(z),
                 M, N, K, ldx, ldw, N, epi, nv.current_stream())
@@ -100,6 +116,12 @@ def gemm_dgrad(dy, w):
         dy, lddy = _prep_bf16(dy)
         w, ldw = _prep_bf16(w)
         dx = torch.empty((M, K), dtype=dy.dtype, device=dy.device)
+        ws, ws_bytes = _split_workspace(GEMM_DGRAD, M, N, K, dy.device)
+        if ws is not None:
+            nv.call("axn_gemm_dgrad_ws", nv.ptr(dy), nv.ptr(w), nv.ptr(dx),
+                    nv.dtype_code(dy.dtype), M, N, K, lddy, ldw, K, nv.ptr(ws), ws_bytes,
+                    nv.current_stream())
+            return dx
         nv.call("axn_gemm_dgrad" + _GEMM16[dy.dtype], nv.ptr(dy), nv.ptr(w), nv.ptr(dx), M, N, K, lddy, ldw, K,
                 nv.current_stream())
     elif dy.dtype == torch.float32:
@@ -135,6 +157,12 @@ def gemm_wgrad(dy, x, out=None, accumulate=False, out_dtype=None):
         x, ldx = _prep_bf16(x)
         if out is None:
             out = torch.empty((N, K), dtype=out_dtype, device=dy.device)
+        ws, ws_bytes = _split_workspace(GEMM_WGRAD, M, N, K, dy.device)
+        if ws is not None:
+            nv.call("axn_gemm_wgrad_ws", nv.ptr(dy), nv.ptr(x), nv.ptr(out),
+                    nv.dtype_code(dy.dtype), M, N, K, lddy, ldx, K, 1 if accumulate else 0,
+                    nv.dtype_code(out_dtype), nv.ptr(ws), ws_bytes, nv.current_stream())
+            return out
         nv.call("axn_gemm_wgrad" + _GEMM16[dy.dtype], nv.ptr(dy), nv.ptr(x), nv.ptr(out), M, N, K, lddy, ldx, K,
                 1 if accumulate else 0, nv.dtype_code(out_dtype), nv.current_stream())
     elif dy.dtype == torch.float32:

@@ -30,7 +30,7 @@
 extern "C" {
 #endif
 
-#define AXN_ABI_VERSION 4
+#define AXN_ABI_VERSION 5
 
 #if defined(__GNUC__)
 #define AXN_API __attribute__((visibility("default")))
@@ -128,6 +128,31 @@ AXN_API int axn_gemm_dgrad_f16(const void* dY, const void* W, void* dX, int64_t 
 AXN_API int axn_gemm_wgrad_f16(const void* dY, const void* X, void* dW, int64_t M,
                        int64_t N, int64_t K, int64_t lddy, int64_t ldx, int64_t lddw,
                        int beta, int dw_dtype, void* stream);
+
+/* Variants of the three GEMMs that may split the contraction over workgroups.
+ * A problem with few output tiles (a short batch, a narrow shard) leaves most of
+ * the 256 CUs without work; with a workspace the library cuts the contraction
+ * into 2, 4 or 8 parts, writes fp32 partial products and adds them in a fixed
+ * order in a second pass (deterministic).  No reference counterpart: torch picks
+ * such kernels inside its GEMM library.
+ *   axn_gemm_workspace_bytes(op, M, N, K): bytes the call below would use for
+ *   dense operands, 0 if it would not split.  op, M, N, K as in the call.
+ *   axn_gemm_*_ws: arguments as axn_gemm_fwd (epilogue NONE) / _dgrad / _wgrad,
+ *   plus dtype (AXN_BF16 or AXN_F16) of the 16-bit operands and results, and
+ *   the workspace.  workspace == NULL, or a shape that does not profit: the
+ *   call is the plain GEMM. */
+typedef enum axn_gemm_op { AXN_GEMM_FWD = 0, AXN_GEMM_DGRAD = 1, AXN_GEMM_WGRAD = 2 } axn_gemm_op;
+AXN_API size_t axn_gemm_workspace_bytes(int op, int64_t M, int64_t N, int64_t K);
+AXN_API int axn_gemm_fwd_ws(const void* X, const void* W, void* Y, int dtype, int64_t M,
+                    int64_t N, int64_t K, int64_t ldx, int64_t ldw, int64_t ldy,
+                    void* workspace, size_t workspace_bytes, void* stream);
+AXN_API int axn_gemm_dgrad_ws(const void* dY, const void* W, void* dX, int dtype, int64_t M,
+                      int64_t N, int64_t K, int64_t lddy, int64_t ldw, int64_t lddx,
+                      void* workspace, size_t workspace_bytes, void* stream);
+AXN_API int axn_gemm_wgrad_ws(const void* dY, const void* X, void* dW, int dtype, int64_t M,
+                      int64_t N, int64_t K, int64_t lddy, int64_t ldx, int64_t lddw,
+                      int beta, int dw_dtype, void* workspace, size_t workspace_bytes,
+                      void* stream);
 
 /* SwiGLU activation of the Llama MLP, one pass over [M,N]:
  *   out = silu(gate) * up,  silu(x) = x / (1 + exp(-x)).

@@ -42,6 +42,15 @@ def test_workspace_queries():
     assert lib.axn_mt_scan_workspace_bytes(-1, 5) == 0
     assert lib.axn_dgelu_dbias_workspace_bytes(8192, 5120) == 64 * 5120 * 4
     assert lib.axn_dgelu_dbias_workspace_bytes(0, 8) == 0
+    # split contraction: fp32 partial products, only for problems with few 128 x 128 tiles
+    assert lib.axn_gemm_workspace_bytes(1, 512, 8192, 3584) == 4 * 512 * 3584 * 4   # dgrad, 112 tiles
+    assert lib.axn_gemm_workspace_bytes(0, 512, 8192, 3584) == 0                    # fwd, 256 tiles: no gain
+    assert lib.axn_gemm_workspace_bytes(2, 512, 8192, 3584) == 0                    # wgrad, 1792 tiles
+    assert lib.axn_gemm_workspace_bytes(0, 4096, 4096, 4096) == 0
+    assert lib.axn_gemm_workspace_bytes(0, 100, 128, 1024) == 0                     # ragged: no split
+    assert lib.axn_gemm_workspace_bytes(0, 128, 128, 512) == 0                      # contraction too short
+    assert lib.axn_gemm_workspace_bytes(0, 128, 128, 4096) == 8 * 128 * 128 * 4
+    assert lib.axn_gemm_workspace_bytes(3, 128, 128, 4096) == 0 and lib.axn_gemm_workspace_bytes(0, 0, 8, 8) == 0
     # embedding: four int32 arrays over the tokens, one over the rows, the sort's own storage
     T, V = 16384, 128256
     need = lib.axn_embedding_workspace_bytes(T, V)
@@ -81,6 +90,16 @@ def test_gemm_argument_errors():
     assert lib.axn_gemm_dgrad_f16(A, None, A, 8, 8, 8, 8, 8, 8, None) == nv.AXN_EINVAL
     assert lib.axn_gemm_wgrad_f16(A, A, A, 8, 8, 8, 8, 8, 8, 0, nv.BF16, None) == nv.AXN_EINVAL
     assert "fp16 or fp32" in _err()
+    # split-contraction variants
+    ws = lib.axn_gemm_dgrad_ws
+    assert ws(A, A, A, nv.F32, 512, 8192, 3584, 8192, 3584, 3584, A, 1 << 30, None) == nv.AXN_EINVAL
+    assert ws(A, A, A, nv.BF16, 512, 8192, 3584, 8192, 3584, 3584, A, 1024, None) == nv.AXN_EINVAL
+    assert "workspace too small" in _err()
+    assert ws(A, A, A, nv.BF16, 512, 8192, 3584, 8192, 3584, 3584, ctypes.c_void_p(0x1008), 1 << 30,
+              None) == nv.AXN_EALIGN
+    assert ws(A, None, A, nv.BF16, 512, 8192, 3584, 8192, 3584, 3584, A, 1 << 30, None) == nv.AXN_EINVAL
+    assert lib.axn_gemm_wgrad_ws(A, A, A, nv.BF16, 8, 8, 8, 8, 8, 8, 0, nv.F16, A, 64, None) == nv.AXN_EINVAL
+    assert lib.axn_gemm_fwd_ws(A, A, A, nv.F16, 8, 12, 8, 8, 8, 16, None, 0, None) == nv.AXN_ESHAPE
     assert lib.axn_gemm_fwd_f32(A, None, None, A, None, 4, 4, 4, 0, None) == nv.AXN_EINVAL
     assert lib.axn_gemm_wgrad_f32(A, A, A, 4, 4, 4, 3, None) == nv.AXN_EINVAL
     assert lib.axn_gemm_dgrad_f32(ctypes.c_void_p(0x1002), A, A, 4, 4, 4, None) == nv.AXN_EALIGN

@@ -375,3 +375,61 @@ def test_operand_of_two_gibibytes_takes_the_64_bit_path():
     assert rel(np64(dw[:, cols]), np64(refw)) < 1e-4
     del X
     torch.cuda.empty_cache()
+
+
+@pytest.mark.parametrize("M,N,K", [(128, 128, 4096), (512, 8192, 3584), (256, 1024, 2048), (384, 512, 1024)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_split_contraction_matches_oracle_and_is_deterministic(M, N, K, dtype):
+    """Problems with few output tiles run with the contraction cut into 2, 4 or 8 parts
+    whose fp32 partial products are added in a fixed order: the same bar as the plain
+    kernels (what is left is the final rounding), and bit-identical results on repeats."""
+    from axonn_amd import _native as nv
+    from axonn_amd import ops
+
+    lib = nv.load()
+    g = torch.Generator().manual_seed(M + N + K)
+    X = torch.randn(M, K, generator=g).to(dtype)
+    W = (torch.randn(N, K, generator=g) * 0.02).to(dtype)
+    dY = (torch.randn(M, N, generator=g) * 1e-2).to(dtype)
+    split = [lib.axn_gemm_workspace_bytes(op, M, N, K) > 0 for op in (0, 1, 2)]
+    assert any(split), "shape chosen to exercise the split path"
+    yo, _ = ol.linear_forward(np64(X), np64(W).reshape(-1), (N, K))
+    bw = ol.linear_backward(np64(X), np64(W).reshape(-1), (N, K), np64(dY))
+    tol = BF16_TOL if dtype == torch.bfloat16 else 1e-3
+    Xd, Wd, dYd = X.cuda(), W.cuda(), dY.cuda()
+    y, _ = ops.gemm_fwd(Xd, Wd)
+    dx = ops.gemm_dgrad(dYd, Wd)
+    dw = ops.gemm_wgrad(dYd, Xd)
+    dw32 = ops.gemm_wgrad(dYd, Xd, out_dtype=torch.float32)
+    assert rel(np64(y), yo) < tol and rel(np64(dx), bw["dx"]) < tol
+    assert rel(np64(dw), bw["dw"].reshape(N, K)) < tol
+    assert rel(np64(dw32), bw["dw"].reshape(N, K)) < F32_TOL
+    # accumulation into an existing fp32 gradient through the reducing pass
+    acc = dw32.clone()
+    ops.gemm_wgrad(dYd, Xd, out=acc, accumulate=True)
+    assert rel(np64(acc), 2 * bw["dw"].reshape(N, K)) < F32_TOL
+    for _ in range(2):
+        assert torch.equal(ops.gemm_fwd(Xd, Wd)[0], y) and torch.equal(ops.gemm_dgrad(dYd, Wd), dx)
+    # the split result equals the unsplit kernel's up to the order of the fp32 sums
+    y_plain = torch.empty_like(y)
+    name = "axn_gemm_fwd" if dtype == torch.bfloat16 else "axn_gemm_fwd_f16"
+    nv.call(name, nv.ptr(Xd), nv.ptr(Wd), None, nv.ptr(y_plain), None, M, N, K, K, K, N, 0, nv.current_stream())
+    assert rel(np64(y), np64(y_plain)) < (4e-3 if dtype == torch.bfloat16 else 5e-4)
+
+
+def test_split_contraction_output_rows_may_be_strided():
+    from axonn_amd import _native as nv
+
+    M, N, K = 128, 256, 2048
+    g = torch.Generator(device="cuda").manual_seed(3)
+    X = torch.randn(M, K, device="cuda", generator=g).bfloat16()
+    W = (torch.randn(N, K, device="cuda", generator=g) * 0.02).bfloat16()
+    big = torch.zeros(M, N + 64, device="cuda", dtype=torch.bfloat16)
+    nbytes = nv.load().axn_gemm_workspace_bytes(0, M, N, K)
+    assert nbytes > 0
+    ws = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
+    nv.call("axn_gemm_fwd_ws", nv.ptr(X), nv.ptr(W), nv.ptr(big), nv.BF16, M, N, K, K, K, N + 64,
+            nv.ptr(ws), nbytes, nv.current_stream())
+    want = (X.float() @ W.float().t())
+    assert rel(np64(big[:, :N]), np64(want)) < BF16_TOL
+    assert not big[:, N:].any()
