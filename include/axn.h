@@ -193,7 +193,10 @@ AXN_API int axn_embedding_fwd(const int64_t* ids, const void* W, void* out, int 
                       int64_t T, int64_t V, int64_t H, int64_t ldw, int64_t ldo,
                       int32_t* status, void* stream);
 
-/* Workspace of the two entry points below (token positions sorted by id). */
+/* Workspace of the two entry points below (token positions sorted by id).
+ * Both call a library sort (rocPRIM), which may clear its own storage with
+ * memset operations: keep them out of captured HIP graphs.  Every other entry
+ * point of this library launches kernels only and can be captured. */
 AXN_API size_t axn_embedding_workspace_bytes(int64_t T, int64_t V);
 
 /* Backward.  Replaces the autograd of the same F.embedding call

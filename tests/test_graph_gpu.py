@@ -1,0 +1,88 @@
+"""The entry points under HIP graph capture: a captured training step (forward with
+the fused epilogue, dgrad, accumulating wgrad, gradient scan, Adam) is replayed several
+times, with eager work and synchronisations between the replays, and every replay must
+equal the eager step on the same inputs bit for bit.  The library issues no memset, copy,
+allocation or synchronisation of its own, so a capture holds kernel nodes only.
+"""
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+def _state(seed):
+    g = torch.Generator(device="cuda").manual_seed(seed)
+    n1, n2 = 70001, 4099
+    s = {
+        "X": torch.randn(384, 256, device="cuda", generator=g).bfloat16(),
+        "W": (torch.randn(512, 256, device="cuda", generator=g) * 0.05).bfloat16(),
+        "b": torch.randn(512, device="cuda", generator=g) * 0.1,
+        "dY": (torch.randn(384, 512, device="cuda", generator=g) * 0.01).bfloat16(),
+        "dW": torch.zeros(512, 256, device="cuda"),
+        "P": torch.randn(n1 + n2, device="cuda", generator=g) * 0.02,
+        "M": torch.zeros(n1 + n2, device="cuda"),
+        "V": torch.zeros(n1 + n2, device="cuda"),
+        "G": (torch.randn(n1 + n2, device="cuda", generator=g) * 64.0).bfloat16(),
+        "PL": torch.zeros(n1 + n2, device="cuda", dtype=torch.bfloat16),
+    }
+    s["sizes"] = (n1, n2)
+    return s
+
+
+def _views(t, sizes):
+    out, off = [], 0
+    for n in sizes:
+        out.append(t[off:off + n])
+        off += n
+    return out
+
+
+def _step(s):
+    from axonn_amd import ops
+
+    y, z = ops.gemm_fwd(s["X"], s["W"], bias=s["b"], activation="gelu", save_z=True)
+    dz, db = ops.dgelu_dbias(s["dY"], z, want_dbias=True)
+    dx = ops.gemm_dgrad(dz, s["W"])
+    ops.gemm_wgrad(dz, s["X"], out=s["dW"], accumulate=True)
+    v = lambda k: _views(s[k], s["sizes"])  # noqa: E731
+    scan = ops.mt_scan(v("G"), inv_scale=1.0 / 64.0, max_norm=1.0)
+    ops.mt_adam(v("G"), v("P"), v("M"), v("V"), v("PL"), ops.adam_hparams(3, 1e-3, 0.9, 0.999, 1e-8, 0.01),
+                inv_scale=1.0 / 64.0, scan=scan)
+    return y, dx, db
+
+
+MUTATED = ("dW", "P", "M", "V", "PL")
+
+
+def test_captured_step_replays_like_the_eager_step():
+    live = _state(1)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):  # first launches outside the capture
+        warm = {k: (v.clone() if torch.is_tensor(v) else v) for k, v in live.items()}
+        _step(warm)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+
+    graph = torch.cuda.CUDAGraph()
+    before_capture = {k: live[k].clone() for k in MUTATED}
+    with torch.cuda.graph(graph):
+        outs = _step(live)
+    for k in MUTATED:  # capturing runs nothing
+        assert torch.equal(live[k], before_capture[k]), k
+
+    for replay in range(4):
+        fresh = _state(10 + replay)
+        for k in ("X", "W", "b", "dY", "G"):  # new inputs at the captured addresses
+            live[k].copy_(fresh[k])
+        twin = {k: (v.clone() if torch.is_tensor(v) else v) for k, v in live.items()}
+        want = _step(twin)          # eager, on copies of the state the replay starts from
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for got, exp, name in zip(outs, want, ("y", "dx", "db")):
+            assert torch.equal(got, exp), (replay, name)
+        for k in MUTATED:
+            assert torch.equal(live[k], twin[k]), (replay, k)
+    assert live["dW"].abs().sum() > 0 and not torch.equal(live["P"], before_capture["P"])
