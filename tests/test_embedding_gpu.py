@@ -246,3 +246,26 @@ def test_bad_arguments_raise_before_any_launch():
         ops.embedding_renorm_(W, ids, -1.0)
     with pytest.raises(RuntimeError, match="GPU only"):
         ops.embedding_fwd(ids.cpu(), W.cpu())
+
+
+def test_table_of_more_than_two_to_the_31_elements():
+    """Row offsets are 64-bit: a 2^18 x 8192 bf16 table (4 GiB) with ids in its last rows."""
+    from axonn_amd import ops
+
+    V, H, T = 1 << 18, 8192, 96
+    g = torch.Generator(device="cuda").manual_seed(7)
+    W = torch.empty(V, H, device="cuda", dtype=torch.bfloat16)
+    W[-4096:].normal_(generator=g)
+    ids = torch.randint(V - 4096, V, (T,), device="cuda", generator=g)
+    ids[:8] = V - 1
+    out = ops.embedding_fwd(ids, W)
+    assert torch.equal(out, W[ids])
+    dy = torch.randn(T, H, device="cuda", generator=g).bfloat16()
+    dW = ops.embedding_bwd(ids, dy, V, out_dtype=torch.float32)
+    rows = torch.unique(ids)
+    base = V - 4096
+    want = oe.embedding_backward((ids - base).cpu().numpy(), host(dy), 4096)
+    assert np.array_equal(host(dW[base:]), want)
+    assert not dW[:base:4099].any() and len(rows) > 50
+    del W, dW
+    torch.cuda.empty_cache()
