@@ -60,6 +60,7 @@ def parse():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-adam", action="store_true")
+    ap.add_argument("--no-library-baseline", action="store_true")
     ap.add_argument("--no-extra-shapes", action="store_true")
     ap.add_argument("--adam-elements", type=float, default=1.3e9)
     ap.add_argument("--no-launch-events", action="store_true",
@@ -193,6 +194,30 @@ def main():
                                "frac": round(v["tflops"] / PEAK_BF16_TFLOPS, 4)}
                            for k, v in kinds.items()},
         }
+    # The same 15 products through the vendor GEMM library (torch.matmul = hipBLASLt), same
+    # operands, same order, timed the same way: a yardstick on this box, not a code path
+    # of the library under test.
+    library = None
+    if not args.no_library_baseline:
+        def library_step():
+            for L in layers:
+                torch.matmul(L.X, L.W.t(), out=L.Y)
+            for L in reversed(layers):
+                torch.matmul(L.dY, L.W, out=L.dX)
+                torch.matmul(L.dY.t(), L.X, out=L.dW)
+
+        for _ in range(max(args.warmup, 2)):
+            library_step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            library_step()
+        torch.cuda.synchronize()
+        lib_elapsed = (time.perf_counter() - t0) / args.steps
+        library = {"kind": "torch.matmul (hipBLASLt) on the same operands, fwd + dgrad + wgrad of the 5 layers",
+                   "value": round(total_flops / lib_elapsed / 1e12, 2), "unit": "TFLOP/s",
+                   "ms_per_step": round(lib_elapsed * 1e3, 4),
+                   "ours_over_library": round(value / (total_flops / lib_elapsed / 1e12), 4)}
     del layers
     torch.cuda.empty_cache()
 
@@ -347,6 +372,7 @@ def main():
         },
         "roofline": roofline,
         "cpu_baseline": cpu,
+        "library_baseline": library,
         "adam": adam,
         "shapes": shapes,
     }
