@@ -10,7 +10,7 @@ The package keeps the reference's Python surface for the one path it covers
     axonn_amd.optim.CPUAdam                        (axonn/optim.py)
     axonn_amd.inter_layer.LossScaler / GradScalerEngine   (axonn/inter_layer.py:18-28, :274-302, :426-460)
     axonn_amd.checkpoint.save / load               (axonn/checkpoint.py)
-    axonn_amd.models.transformers.parallelize      (axonn/models/transformers, Llama only)
+    axonn_amd.models.transformers.parallelize      (axonn/models/transformers)
 
 and runs all of its arithmetic in hand-written gfx950 kernels behind the C ABI
 of libaxn_gfx950.so (include/axn.h).  There is no CPU or library fallback.

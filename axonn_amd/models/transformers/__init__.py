@@ -1,6 +1,7 @@
 """Swaps the projections of Hugging Face models for `axonn_amd.intra_layer.Linear`,
 as `axonn.models.transformers` does (axonn/models/transformers/__init__.py:22-60).
-Only the Llama family is covered here."""
+Llama, Mistral, OPT and Mixtral (attention only: current transformers releases keep the
+experts in fused 3-D parameters) are covered; a model family is imported when asked for."""
 
 from contextlib import contextmanager
 
@@ -9,8 +10,31 @@ from .modify_llama import (  # noqa: F401
     reverse_monkey_patch_llama_with_axonn,
 )
 
+
+def _lazy(module, family):
+    """(patch, unpatch) that import the family's module on first use, so that importing
+    this package does not import every model family of transformers."""
+    def patch():
+        import importlib
+
+        mod = importlib.import_module(__name__ + "." + module)
+        return getattr(mod, "monkey_patch_%s_with_axonn" % family)()
+
+    def unpatch(original_attention_init, original_mlp_init):
+        import importlib
+
+        mod = importlib.import_module(__name__ + "." + module)
+        return getattr(mod, "reverse_monkey_patch_%s_with_axonn" % family)(
+            original_attention_init, original_mlp_init)
+
+    return patch, unpatch
+
+
 modify_dict = {
     "LlamaForCausalLM": (monkey_patch_llama_with_axonn, reverse_monkey_patch_llama_with_axonn),
+    "MistralForCausalLM": _lazy("modify_mistral", "mistral"),
+    "OPTForCausalLM": _lazy("modify_opt", "opt"),
+    "MixtralForCausalLM": _lazy("modify_mixtral", "mixtral"),
 }
 
 

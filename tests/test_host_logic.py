@@ -263,3 +263,38 @@ def test_bench_refuses_more_than_one_gpu():
                           capture_output=True, text=True, timeout=120)
     assert proc.returncode != 0
     assert "ONE GPU" in proc.stderr and proc.stdout.strip() == ""
+
+
+@pytest.mark.parametrize("family,n_linear", [("mistral", 14), ("opt", 12), ("mixtral", 8)])
+def test_parallelize_patches_every_family_the_reference_patches(family, n_linear):
+    """axonn/models/transformers/__init__.py:22-39 lists OPT, Llama, Mixtral and Mistral;
+    models built inside the context get the Linear projections, models built after it
+    do not (construction only: no kernel runs on the CPU)."""
+    from transformers import MistralConfig, MixtralConfig, OPTConfig
+    from transformers.models.mistral.modeling_mistral import MistralForCausalLM
+    from transformers.models.mixtral.modeling_mixtral import MixtralForCausalLM
+    from transformers.models.opt.modeling_opt import OPTForCausalLM
+
+    from axonn_amd.models.transformers import modify_dict, parallelize
+
+    assert set(modify_dict) == {"OPTForCausalLM", "LlamaForCausalLM", "MixtralForCausalLM", "MistralForCausalLM"}
+    ax.init(1, 1, 1, 1)
+    common = dict(hidden_size=64, num_attention_heads=4, num_hidden_layers=2, vocab_size=64,
+                  max_position_embeddings=32)
+    cls, cfg = {
+        "mistral": (MistralForCausalLM, MistralConfig(intermediate_size=128, num_key_value_heads=2,
+                                                      architectures=["MistralForCausalLM"], **common)),
+        "opt": (OPTForCausalLM, OPTConfig(ffn_dim=128, word_embed_proj_dim=64,
+                                          architectures=["OPTForCausalLM"], **common)),
+        "mixtral": (MixtralForCausalLM, MixtralConfig(intermediate_size=128, num_key_value_heads=2,
+                                                      num_local_experts=4,
+                                                      architectures=["MixtralForCausalLM"], **common)),
+    }[family]
+    with parallelize(cfg):
+        model = cls(cfg)
+    assert sum(isinstance(m, Linear) for m in model.modules()) == n_linear
+    assert not any(isinstance(m, Linear) for m in cls(cfg).modules())
+    with pytest.raises(AssertionError, match="has not been parallelized"):
+        cfg.architectures = ["GPT2LMHeadModel"]
+        with parallelize(cfg):
+            pass

@@ -197,3 +197,59 @@ def test_auto_parallelize_builds_hugging_face_mlp_on_the_kernels():
     wg, wu, wd = (np64(p).reshape(-1) for p in (mlp.gate_proj.weight, mlp.up_proj.weight, mlp.down_proj.weight))
     fwd = om.llama_mlp_forward(np64(x), wg, wu, wd, 128, 256, store="bf16")
     assert rel(np64(y), fwd["out"]) < 1e-2
+
+
+def _twin_models(family):
+    from transformers import MistralConfig, MixtralConfig, OPTConfig
+    from transformers.models.mistral.modeling_mistral import MistralForCausalLM
+    from transformers.models.mixtral.modeling_mixtral import MixtralForCausalLM
+    from transformers.models.opt.modeling_opt import OPTForCausalLM
+
+    common = dict(hidden_size=256, num_attention_heads=4, num_hidden_layers=2, vocab_size=128,
+                  max_position_embeddings=64)
+    if family == "mistral":
+        return MistralForCausalLM, MistralConfig(intermediate_size=512, num_key_value_heads=2,
+                                                 architectures=["MistralForCausalLM"], **common), 2 * 7
+    if family == "opt":
+        # OPT has dropout by default: off, so that the two models see the same function
+        return OPTForCausalLM, OPTConfig(ffn_dim=512, word_embed_proj_dim=256, dropout=0.0,
+                                         attention_dropout=0.0, layerdrop=0.0,
+                                         architectures=["OPTForCausalLM"], **common), 2 * 6
+    return MixtralForCausalLM, MixtralConfig(intermediate_size=512, num_key_value_heads=2, num_local_experts=4,
+                                             architectures=["MixtralForCausalLM"], **common), 2 * 4
+
+
+@pytest.mark.parametrize("family", ["mistral", "opt", "mixtral"])
+def test_other_model_families_under_parallelize_match_their_torch_twins(family):
+    """The reference patches OPT, Mistral and Mixtral as it patches Llama
+    (axonn/models/transformers/__init__.py:22-39): a 2-layer model of each family built
+    inside `parallelize` against the same model from torch.nn.Linear with the same
+    weights; bf16, logits normwise 2e-2, gradients 5e-2, as for Llama above."""
+    import axonn_amd.axonn as ax
+    from axonn_amd.intra_layer import Linear
+    from axonn_amd.models.transformers import parallelize
+
+    ax.init(1, 1, 1, 1)
+    cls, cfg, n_expected = _twin_models(family)
+    cfg._attn_implementation = "eager"
+    torch.manual_seed(0)
+    ref = cls(cfg)
+    with parallelize(cfg):
+        ours = cls(cfg)
+    assert sum(isinstance(m, Linear) for m in ours.modules()) == n_expected
+    assert not any(isinstance(m, Linear) for m in cls(cfg).modules())   # the patch is undone
+    missing = ours.load_state_dict(ref.state_dict(), strict=True)
+    assert not missing.missing_keys and not missing.unexpected_keys
+    ref, ours = ref.cuda().bfloat16(), ours.cuda().bfloat16()
+    ids = torch.randint(0, 128, (4, 32), generator=torch.Generator().manual_seed(1)).cuda()
+    out_r = ref(input_ids=ids, labels=ids)
+    out_o = ours(input_ids=ids, labels=ids)
+    assert rel(np64(out_o.logits), np64(out_r.logits)) < 2e-2
+    assert abs(out_o.loss.item() - out_r.loss.item()) < 2e-2 * abs(out_r.loss.item())
+    out_r.loss.backward()
+    out_o.loss.backward()
+    for (name, p_r), (_, p_o) in zip(ref.named_parameters(), ours.named_parameters()):
+        if p_r.grad is None:
+            assert p_o.grad is None, name
+            continue
+        assert rel(np64(p_o.grad).reshape(-1), np64(p_r.grad).reshape(-1)) < 5e-2, name
