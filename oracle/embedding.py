@@ -49,8 +49,9 @@ def embedding_backward(ids, dY, num_embeddings, padding_idx=None, scale_grad_by_
     rounded to fp32.  `accumulate_into` (fp32 [V,H]) is added to the rows that
     received terms, after their sum.  Ids outside the table are skipped."""
     ids = np.asarray(ids, dtype=np.int64).reshape(-1)
-    dY = np.asarray(dY, dtype=np.float32).reshape(ids.size, -1)
-    H = dY.shape[1]
+    dY = np.asarray(dY, dtype=np.float32)
+    H = dY.shape[-1]
+    dY = dY.reshape(ids.size, H)
     keep = (ids >= 0) & (ids < num_embeddings)
     if padding_idx is not None:
         keep &= ids != padding_idx
@@ -81,7 +82,8 @@ def embedding_backward(ids, dY, num_embeddings, padding_idx=None, scale_grad_by_
 def embedding_backward_f64(ids, dY, num_embeddings, padding_idx=None, scale_grad_by_freq=False):
     """The same sums in float64, order-free: what every summation order approximates."""
     ids = np.asarray(ids, dtype=np.int64).reshape(-1)
-    dY = np.asarray(dY, dtype=np.float64).reshape(ids.size, -1)
+    dY = np.asarray(dY, dtype=np.float64)
+    dY = dY.reshape(ids.size, dY.shape[-1])
     keep = (ids >= 0) & (ids < num_embeddings)
     counts = np.bincount(ids[keep], minlength=num_embeddings).astype(np.float64)
     if padding_idx is not None:
