@@ -27,19 +27,29 @@ constexpr int EW_TY = 4;           // row phases per workgroup
 constexpr int EW_COLS = EW_TX * 8; // 512 columns per workgroup
 constexpr int EW_BAND = 128;       // rows per workgroup
 
-// 8 consecutive columns as floats, for bf16 (16 bytes) and fp32 (32 bytes) rows.
+// 8 consecutive columns as floats, for bf16 / fp16 (16 bytes) and fp32 (32 bytes) rows.
+// NT: non-temporal loads, for operands read once.  They are worth 15 % on the SwiGLU
+// forward and 23 % on its backward and cost 12 % on dGELU (measured), so each kernel
+// names its own.
+template <bool NT, typename V>
+__device__ __forceinline__ V load_vec(const void* p) {
+  return NT ? __builtin_nontemporal_load((const V*)p) : *(const V*)p;
+}
+template <bool NT = false>
 __device__ __forceinline__ void load8(const uint16_t* p, float (&x)[8]) {
-  const bf16x8 v = *(const bf16x8*)p;
+  const bf16x8 v = load_vec<NT, bf16x8>(p);
 #pragma unroll
   for (int e = 0; e < 8; ++e) x[e] = (float)v[e];
 }
+template <bool NT = false>
 __device__ __forceinline__ void load8(const _Float16* p, float (&x)[8]) {
-  const f16x8 v = *(const f16x8*)p;
+  const f16x8 v = load_vec<NT, f16x8>(p);
 #pragma unroll
   for (int e = 0; e < 8; ++e) x[e] = (float)v[e];
 }
+template <bool NT = false>
 __device__ __forceinline__ void load8(const float* p, float (&x)[8]) {
-  const f32x4 a = *(const f32x4*)p, b = *(const f32x4*)(p + 4);
+  const f32x4 a = load_vec<NT, f32x4>(p), b = load_vec<NT, f32x4>(p + 4);
 #pragma unroll
   for (int e = 0; e < 4; ++e) {
     x[e] = a[e];
@@ -148,8 +158,8 @@ __global__ void __launch_bounds__(EW_TX* EW_TY)
   for (int64_t r = r0 + ty; r < r1; r += EW_TY) {
     const int64_t o = r * ld + col;
     float g[8], u[8];
-    load8(gate + o, g);
-    load8(up + o, u);
+    load8<true>(gate + o, g);
+    load8<true>(up + o, u);
 #pragma unroll
     for (int e = 0; e < 8; ++e) g[e] = g[e] * sigmoid_f(g[e]) * u[e];
     store8(out + o, g);
@@ -170,9 +180,9 @@ __global__ void __launch_bounds__(EW_TX* EW_TY)
   for (int64_t r = r0 + ty; r < r1; r += EW_TY) {
     const int64_t o = r * ld + col;
     float d[8], g[8], u[8], dg[8], du[8];
-    load8(dout + o, d);
-    load8(gate + o, g);
-    load8(up + o, u);
+    load8<true>(dout + o, d);
+    load8<true>(gate + o, g);
+    load8<true>(up + o, u);
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
       const float sg = sigmoid_f(g[e]);
