@@ -377,7 +377,8 @@ def test_operand_of_two_gibibytes_takes_the_64_bit_path():
     torch.cuda.empty_cache()
 
 
-@pytest.mark.parametrize("M,N,K", [(128, 128, 4096), (512, 8192, 3584), (256, 1024, 2048), (384, 512, 1024)])
+@pytest.mark.parametrize("M,N,K", [(128, 128, 4096), (512, 8192, 3584), (256, 1024, 2048), (384, 512, 1024),
+                                   (4096, 256, 512)])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_split_contraction_matches_oracle_and_is_deterministic(M, N, K, dtype):
     """Problems with few output tiles run with the contraction cut into 2, 4 or 8 parts
@@ -408,6 +409,9 @@ def test_split_contraction_matches_oracle_and_is_deterministic(M, N, K, dtype):
     acc = dw32.clone()
     ops.gemm_wgrad(dYd, Xd, out=acc, accumulate=True)
     assert rel(np64(acc), 2 * bw["dw"].reshape(N, K)) < F32_TOL
+    acc16 = dw.clone()   # and into a 16-bit gradient: old value + sum, rounded once
+    ops.gemm_wgrad(dYd, Xd, out=acc16, accumulate=True)
+    assert rel(np64(acc16), np64(dw) + bw["dw"].reshape(N, K)) < tol
     for _ in range(2):
         assert torch.equal(ops.gemm_fwd(Xd, Wd)[0], y) and torch.equal(ops.gemm_dgrad(dYd, Wd), dx)
     # the split result equals the unsplit kernel's up to the order of the fp32 sums
