@@ -389,3 +389,39 @@ def test_full_size_adam_properties():
                 1.0 / 65536.0, scan)
     assert int(scan.found_inf.item()) == 1
     assert torch.equal(P, P1) and torch.equal(M, M1) and torch.equal(V, V1)
+
+
+def test_cpuadam_parameter_groups_follow_torch_adam():
+    """Two parameter groups with their own lr / betas / weight decay
+    (axonn/optim.py:17-26 takes torch's param-group form, :100-150 walks the groups):
+    three steps against torch.optim.Adam on fp32 copies fed the same gradients."""
+    from axonn_amd.inter_layer import LossScaler
+    from axonn_amd.optim import CPUAdam
+
+    torch.manual_seed(21)
+    a = torch.nn.Parameter((torch.randn(3001) * 0.05).bfloat16().cuda())
+    b = torch.nn.Parameter((torch.randn(517, 8) * 0.05).bfloat16().cuda())
+    groups = [{"params": [a], "lr": 1e-3, "weight_decay": 0.0},
+              {"params": [b], "lr": 3e-2, "betas": (0.8, 0.95), "weight_decay": 0.05}]
+    opt = CPUAdam(groups, loss_scaler=LossScaler(loss_scale=256.0), dynamic_loss_scale=False)
+    ra = torch.nn.Parameter(a.detach().float().clone())
+    rb = torch.nn.Parameter(b.detach().float().clone())
+    ref = torch.optim.Adam([{"params": [ra], "lr": 1e-3, "weight_decay": 0.0},
+                            {"params": [rb], "lr": 3e-2, "betas": (0.8, 0.95), "weight_decay": 0.05}],
+                           foreach=False)
+    assert opt.group_offsets == [0, 3001, 3001 + 517 * 8]
+    for _ in range(3):
+        opt.zero_grad()
+        ga = (torch.randn(3001, device="cuda") * 0.01)
+        gb = (torch.randn(517, 8, device="cuda") * 0.01)
+        a.grad.copy_((ga * 256.0).bfloat16())
+        b.grad.copy_((gb * 256.0).bfloat16())
+        ra.grad = a.grad.float() / 256.0     # the same bf16-rounded gradients, unscaled
+        rb.grad = b.grad.float() / 256.0
+        opt.step()
+        ref.step()
+        got = opt.model_params_fp32
+        want = torch.cat([ra.detach().reshape(-1), rb.detach().reshape(-1)])
+        assert float((got - want).abs().max() / want.abs().max()) <= P_TOL
+    assert torch.equal(a.detach(), opt.model_params_fp32[:3001].bfloat16())
+    assert torch.equal(b.detach().reshape(-1), opt.model_params_fp32[3001:].bfloat16())
