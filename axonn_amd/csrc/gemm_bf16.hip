@@ -518,6 +518,12 @@ __device__ __forceinline__ void solo_gemm(const GemmArgs& g) {
   if (KP > 1) {
     static_for<NC>(copy_a); a_done();
     static_for<NC>(copy_b); b_done();
+  }
+  // The accumulators are cleared here, while the first tiles are on their way: left
+  // to itself the compiler clears them where they are first used, behind the wait.
+#pragma unroll
+  for (int i = 0; i < FR; ++i) settle_accumulators(acc[i]);
+  if (KP > 1) {
     wait_vmcnt<2 * NC>();
   } else {
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
