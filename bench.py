@@ -41,8 +41,8 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 # file, scaled by what the same counters read for the 1 GiB copy below
 # (profiles/gemm_adam_llama_set_pmc.txt has the runs and the arithmetic).  The
 # counters sit between L2 and the fabric, so hits in the memory-side cache are included.
-TRAFFIC_BYTES_PER_LAUNCH = {"fwd": 634551521, "dgrad": 594959413, "wgrad": 707605136}
-ADAM_TRAFFIC_BYTES_PER_STEP = 39285015143   # scan + update, 1.3e9 elements
+TRAFFIC_BYTES_PER_LAUNCH = {"fwd": 620626199, "dgrad": 593562126, "wgrad": 666643150}
+ADAM_TRAFFIC_BYTES_PER_STEP = 39286702598   # scan + update, 1.3e9 elements
 
 LLAMA_SET = [  # (name, M, N, K), gate and up are two layers of one shape
     ("qkv", 4096, 6144, 4096),
@@ -179,7 +179,9 @@ def main():
                 "tflops": tot_fl / (tot_ms * 1e-3) / 1e12, "total_ms": tot_ms,
             }
         dom = max(kinds, key=lambda k: kinds[k]["total_ms"])
-        # template arguments: <tile, A contraction-contiguous, B contraction-contiguous, epilogue, fp32 out>
+        # template arguments: <tile, A contraction-contiguous, B contraction-contiguous, epilogue, fp32 out>.
+        # A call whose output is k x 256 + r large tiles with 0 < r <= 128 is two launches, k rounds
+        # of this instance and the rest on its <128, ...> twin; the events bracket the call.
         kernel_names = {"fwd": "gemm_bf16_solo_kernel<256, true, true, 0, false> (Y = X W^T)",
                         "dgrad": "gemm_bf16_solo_kernel<256, true, false, 0, false> (dX = dY W)",
                         "wgrad": "gemm_bf16_solo_kernel<256, false, false, 0, false> (dW = dY^T X)"}
