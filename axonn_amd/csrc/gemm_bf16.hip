@@ -405,6 +405,11 @@ __device__ __forceinline__ void wait_all_fragments(bf16x8 (&fa)[8], bf16x8 (&fb)
                  "+v"(fa[6]), "+v"(fa[7]), "+v"(fb[0]), "+v"(fb[1]), "+v"(fb[2]), "+v"(fb[3]),
                  "+v"(fb[4]), "+v"(fb[5]), "+v"(fb[6]), "+v"(fb[7]));
 }
+__device__ __forceinline__ void wait_all_fragments(bf16x8 (&fa)[8], bf16x8 (&fb)[4]) {
+  asm volatile("s_waitcnt lgkmcnt(0)"
+               : "+v"(fa[0]), "+v"(fa[1]), "+v"(fa[2]), "+v"(fa[3]), "+v"(fa[4]), "+v"(fa[5]),
+                 "+v"(fa[6]), "+v"(fa[7]), "+v"(fb[0]), "+v"(fb[1]), "+v"(fb[2]), "+v"(fb[3]));
+}
 __device__ __forceinline__ void wait_all_fragments(bf16x8 (&fa)[4], bf16x8 (&fb)[4]) {
   asm volatile("s_waitcnt lgkmcnt(0)"
                : "+v"(fa[0]), "+v"(fa[1]), "+v"(fa[2]), "+v"(fa[3]), "+v"(fb[0]), "+v"(fb[1]),
@@ -442,18 +447,27 @@ __device__ __forceinline__ void wait_vmcnt() {
 // TILE = 128 is the same schedule on a 128 x 128 tile for problems that do not
 // fill the chip with 256 x 256 tiles: 64 x 64 per wave (4 x 4 blocks, 16 MFMAs per
 // step, 4 copies per tile and wave), an 80 KiB ring, two workgroups per CU.
-template <int TILE, bool A_KMAJOR, bool B_KMAJOR, int EPI, bool OUT_F32, bool HALF>
+//
+// BM x BN = 256 x 128 is the tile of the launches that finish a problem after its full
+// rounds of 256 x 256 tiles: a rest of r <= 128 large tiles makes 2 r <= 256 of these,
+// one per CU, and needs 3/4 of the global -> LDS bytes per MFMA of the 128 x 128 tile.
+// Its ring has five slots of the larger (A) tile's size.
+template <int BM, int BN, bool A_KMAJOR, bool B_KMAJOR, int EPI, bool OUT_F32, bool HALF>
 __device__ __forceinline__ void solo_gemm(const GemmArgs& g) {
-  constexpr int BM = TILE, BN = TILE, WTM = TILE / 2, WTN = TILE / 2, FR = TILE / 32;
+  constexpr int WTM = BM / 2, WTN = BN / 2, FRM = BM / 32, FRN = BN / 32;
   constexpr int PK = 64, NSLOT = 5;
-  constexpr int NM = FR * FR;           // MFMAs per step
-  using OA = DeepOperand<A_KMAJOR, false, TILE>;
-  using OB = DeepOperand<B_KMAJOR, true, TILE>;
-  constexpr uint32_t SLOT = OA::BYTES;  // 32 or 16 KiB
-  constexpr int NC = OA::DMA_N;         // copies per tile and wave
-  constexpr int READ_EVERY = NM / (4 * FR);  // a fragment read every .. MFMAs, first half of a step
-  constexpr int COPY_EVERY = NM / (2 * NC);  // a copy every .. MFMAs, second half
-  static_assert(TILE == 256 || TILE == 128, "tile sizes with a schedule below");
+  constexpr int NM = FRM * FRN;         // MFMAs per step
+  using OA = DeepOperand<A_KMAJOR, false, BM>;
+  using OB = DeepOperand<B_KMAJOR, true, BN>;
+  constexpr uint32_t SLOT = OA::BYTES > OB::BYTES ? OA::BYTES : OB::BYTES;  // 32 or 16 KiB
+  constexpr int NCA = OA::DMA_N, NCB = OB::DMA_N;  // copies per tile and wave
+  constexpr int NFRAG = FRM + FRN;                 // fragment reads per step
+  constexpr int READ_EVERY = (NM / 2) / NFRAG;     // a fragment read every .. MFMAs, first half of a step
+  constexpr int COPY_EVERY_A = (NM / 2) / NCA;     // a copy every .. MFMAs, second half
+  constexpr int COPY_EVERY_B = (NM / 2) / NCB;
+  static_assert((BM == 256 || BM == 128) && (BN == 256 || BN == 128) && BM >= BN,
+                "tile sizes with a schedule below");
+  static_assert(READ_EVERY >= 1 && COPY_EVERY_A >= 1 && COPY_EVERY_B >= 1, "schedule fits a step");
 
   extern __shared__ __attribute__((aligned(16))) char lds[];
 
@@ -471,11 +485,11 @@ __device__ __forceinline__ void solo_gemm(const GemmArgs& g) {
   tile_of_workgroup(pid, g.tiles_m, g.tiles_n, tm, tn);
   const int m0 = tm * BM, n0 = tn * BN;
 
-  f32x4 acc[FR][FR];
+  f32x4 acc[FRM][FRN];
 #pragma unroll
-  for (int i = 0; i < FR; ++i)
+  for (int i = 0; i < FRM; ++i)
 #pragma unroll
-    for (int j = 0; j < FR; ++j) acc[i][j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    for (int j = 0; j < FRN; ++j) acc[i][j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
 
   const int KP = (g.splits > 1 ? g.k_split : g.Kc) / PK;  // stages of this workgroup
   const uint32_t a_bytes = (uint32_t)((int64_t)(A_KMAJOR ? g.M : g.Kc) * g.lda * 2);
@@ -513,31 +527,31 @@ __device__ __forceinline__ void solo_gemm(const GemmArgs& g) {
   auto b_done = [&]() { kb += b_step; wslot = next_slot(wslot); };
 
   // A0 B0 (A1 B1) up front.
-  static_for<NC>(copy_a); a_done();
-  static_for<NC>(copy_b); b_done();
+  static_for<NCA>(copy_a); a_done();
+  static_for<NCB>(copy_b); b_done();
   if (KP > 1) {
-    static_for<NC>(copy_a); a_done();
-    static_for<NC>(copy_b); b_done();
+    static_for<NCA>(copy_a); a_done();
+    static_for<NCB>(copy_b); b_done();
   }
   // The accumulators are cleared here, while the first tiles are on their way: left
   // to itself the compiler clears them where they are first used, behind the wait.
 #pragma unroll
-  for (int i = 0; i < FR; ++i) settle_accumulators(acc[i]);
+  for (int i = 0; i < FRM; ++i) settle_accumulators(acc[i]);
   if (KP > 1) {
-    wait_vmcnt<2 * NC>();
+    wait_vmcnt<NCA + NCB>();
   } else {
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   }
   __builtin_amdgcn_s_barrier();
 
-  bf16x8 fa0[FR], fb0[FR], fa1[FR], fb1[FR];  // register sets of steps 0 / 1
-  // fragment f of 2 FR (A fragments, then B fragments) of step ST of the stage
+  bf16x8 fa0[FRM], fb0[FRN], fa1[FRM], fb1[FRN];  // register sets of steps 0 / 1
+  // fragment f of FRM + FRN (A fragments, then B fragments) of step ST of the stage
   // whose tiles sit at sa / sb, into register set ST
   auto read = [&](auto st_, auto f_, uint32_t sa, uint32_t sb) {
     constexpr int ST = decltype(st_)::value, f = decltype(f_)::value;
-    bf16x8(&fa)[FR] = ST ? fa1 : fa0;
-    bf16x8(&fb)[FR] = ST ? fb1 : fb0;
-    if constexpr (f < FR) {
+    bf16x8(&fa)[FRM] = ST ? fa1 : fa0;
+    bf16x8(&fb)[FRN] = ST ? fb1 : fb0;
+    if constexpr (f < FRM) {
       uint32_t ra[OA::NADDR];
 #pragma unroll
       for (int i = 0; i < OA::NADDR; ++i) ra[i] = ra0[i] + sa;
@@ -546,11 +560,11 @@ __device__ __forceinline__ void solo_gemm(const GemmArgs& g) {
       uint32_t rb[OB::NADDR];
 #pragma unroll
       for (int i = 0; i < OB::NADDR; ++i) rb[i] = rb0[i] + sb;
-      OB::template read_frag<ST, f - FR>(fb[f - FR], rb);
+      OB::template read_frag<ST, f - FRM>(fb[f - FRM], rb);
     }
   };
   uint32_t sa = 0, sb = SLOT;  // slots of the current stage's tiles
-  static_for<2 * FR>([&](auto f_) { read(std::integral_constant<int, 0>{}, f_, sa, sb); });
+  static_for<NFRAG>([&](auto f_) { read(std::integral_constant<int, 0>{}, f_, sa, sb); });
 
   // HAS2: stage p + 2 exists (its tiles are copied during this stage);
   // LAST: no stage follows.
@@ -560,18 +574,18 @@ __device__ __forceinline__ void solo_gemm(const GemmArgs& g) {
     const uint32_t na = next_slot(sb), nb = next_slot(na);  // slots of stage p + 1
     static_for<2>([&](auto st_) {
       constexpr int ST = decltype(st_)::value;
-      bf16x8(&fa)[FR] = ST ? fa1 : fa0;
-      bf16x8(&fb)[FR] = ST ? fb1 : fb0;
+      bf16x8(&fa)[FRM] = ST ? fa1 : fa0;
+      bf16x8(&fb)[FRN] = ST ? fb1 : fb0;
       wait_all_fragments(fa, fb);  // every read of this set was issued during the previous step
       if constexpr (ST == 1 && !LAST) {
-        if (HAS2) wait_vmcnt<NC>();  // A(p+2) may be in flight
+        if (HAS2) wait_vmcnt<NCA>();  // A(p+2) may be in flight
         else wait_vmcnt<0>();
         __builtin_amdgcn_s_barrier();
       }
       __builtin_amdgcn_sched_barrier(0);
       static_for<NM>([&](auto m_) {
         constexpr int m = decltype(m_)::value;
-        constexpr int i = m / FR, j = m % FR;
+        constexpr int i = m / FRN, j = m % FRN;
         // Inline assembly pins the register classes (accumulators in AGPRs, fragments
         // in VGPRs): with the builtin the allocator moves two-instruction
         // (transposed) fragments through AGPRs and spills.  No MFMA hazard can arise:
@@ -586,14 +600,17 @@ __device__ __forceinline__ void solo_gemm(const GemmArgs& g) {
           asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0"
                        : "+a"(acc[i][j])
                        : "v"(fb[j]), "v"(fa[i]));
-        if constexpr (m < NM / 2 && m % READ_EVERY == 0) {
+        constexpr int CE = ST == 0 ? COPY_EVERY_A : COPY_EVERY_B;  // step 0 copies A, step 1 B
+        constexpr int NCX = ST == 0 ? NCA : NCB;
+        if constexpr (m < NM / 2 && m % READ_EVERY == 0 && m / READ_EVERY < NFRAG) {
           if constexpr (ST == 0) read(std::integral_constant<int, 1>{},
                                       std::integral_constant<int, m / READ_EVERY>{}, sa, sb);
           else if constexpr (!LAST) read(std::integral_constant<int, 0>{},
                                          std::integral_constant<int, m / READ_EVERY>{}, na, nb);
-        } else if constexpr (HAS2 && m >= NM / 2 && (m - NM / 2) % COPY_EVERY == COPY_EVERY - 1) {
-          if constexpr (ST == 0) copy_a(std::integral_constant<int, (m - NM / 2) / COPY_EVERY>{});
-          else copy_b(std::integral_constant<int, (m - NM / 2) / COPY_EVERY>{});
+        } else if constexpr (HAS2 && m >= NM / 2 && (m - NM / 2) % CE == CE - 1 &&
+                             (m - NM / 2) / CE < NCX) {
+          if constexpr (ST == 0) copy_a(std::integral_constant<int, (m - NM / 2) / CE>{});
+          else copy_b(std::integral_constant<int, (m - NM / 2) / CE>{});
         }
         __builtin_amdgcn_sched_barrier(0);
       });
@@ -615,7 +632,7 @@ __device__ __forceinline__ void solo_gemm(const GemmArgs& g) {
   // latency; the epilogue can only read the values these statements return.
   asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
 #pragma unroll
-  for (int i = 0; i < FR; ++i) settle_accumulators(acc[i]);
+  for (int i = 0; i < FRM; ++i) settle_accumulators(acc[i]);
   // With the permuted column fragments a lane owns, per block row i and block
   // pair t, the 8 consecutive columns 32 t + 8 (l / 16) .. + 7 of row 16 i + l % 16:
   // they go out straight from the registers, 64 contiguous bytes per row and
@@ -625,9 +642,9 @@ __device__ __forceinline__ void solo_gemm(const GemmArgs& g) {
   GemmArgs go = g;  // a split writes its own fp32 partial product
   if (OUT_F32 && g.splits > 1) go.C = (float*)g.C + (int64_t)split * g.M * g.ldc;
 #pragma unroll
-  for (int i = 0; i < FR; ++i)
+  for (int i = 0; i < FRM; ++i)
 #pragma unroll
-    for (int t = 0; t < FR / 2; ++t) {
+    for (int t = 0; t < FRN / 2; ++t) {
       const f32x4 lo = acc[i][2 * t], hi = acc[i][2 * t + 1];
       float v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
       store_row8<EPI, OUT_F32, HALF>(v, go, orow + 16 * i, ocol + 32 * t);
@@ -636,11 +653,20 @@ __device__ __forceinline__ void solo_gemm(const GemmArgs& g) {
 
 template <int TILE, bool A_KMAJOR, bool B_KMAJOR, int EPI, bool OUT_F32>
 __global__ void __launch_bounds__(256) gemm_bf16_solo_kernel(const GemmArgs g) {
-  solo_gemm<TILE, A_KMAJOR, B_KMAJOR, EPI, OUT_F32, false>(g);
+  solo_gemm<TILE, TILE, A_KMAJOR, B_KMAJOR, EPI, OUT_F32, false>(g);
 }
 template <int TILE, bool A_KMAJOR, bool B_KMAJOR, int EPI, bool OUT_F32>
 __global__ void __launch_bounds__(256) gemm_f16_solo_kernel(const GemmArgs g) {
-  solo_gemm<TILE, A_KMAJOR, B_KMAJOR, EPI, OUT_F32, true>(g);
+  solo_gemm<TILE, TILE, A_KMAJOR, B_KMAJOR, EPI, OUT_F32, true>(g);
+}
+// The 256 x 128 tile of the launches that finish a problem.
+template <bool A_KMAJOR, bool B_KMAJOR, int EPI, bool OUT_F32>
+__global__ void __launch_bounds__(256) gemm_bf16_rest_kernel(const GemmArgs g) {
+  solo_gemm<256, 128, A_KMAJOR, B_KMAJOR, EPI, OUT_F32, false>(g);
+}
+template <bool A_KMAJOR, bool B_KMAJOR, int EPI, bool OUT_F32>
+__global__ void __launch_bounds__(256) gemm_f16_rest_kernel(const GemmArgs g) {
+  solo_gemm<256, 128, A_KMAJOR, B_KMAJOR, EPI, OUT_F32, true>(g);
 }
 
 // ---------------------------------------------------------------------------
@@ -793,6 +819,21 @@ int launch_solo(const GemmArgs& in, hipStream_t stream) {
   return AXN_OK;
 }
 
+template <bool AK, bool BKM, int EPI, bool OUT_F32, bool HALF>
+int launch_rest(const GemmArgs& in, hipStream_t stream) {
+  GemmArgs g = in;
+  g.tiles_m = g.M / 256;
+  g.tiles_n = g.N / 128;
+  constexpr size_t lds = 5 * 256 * 64 * 2;  // five slots of the A tile's size
+  void (*kern)(const GemmArgs) = gemm_bf16_rest_kernel<AK, BKM, EPI, OUT_F32>;
+  if constexpr (HALF) kern = gemm_f16_rest_kernel<AK, BKM, EPI, OUT_F32>;
+  AXN_HIP_TRY(hipFuncSetAttribute((const void*)kern,
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+  hipLaunchKernelGGL(kern, dim3((unsigned)(g.tiles_m * g.tiles_n)), dim3(256), lds, stream, g);
+  AXN_HIP_TRY(hipGetLastError());
+  return AXN_OK;
+}
+
 // Kernel selection.  Problems made of whole 256 x 256 tiles, more than 128 of
 // them (half of the CUs) and not just above one round of 256, take the
 // one-wave-per-SIMD kernel at that tile size;
@@ -826,7 +867,8 @@ int launch_whole(const GemmArgs& g, hipStream_t stream) {
 // Full rounds and the rest.  A problem of k * 256 + r large tiles with 0 < r <= 128 ends
 // in a round that leaves at least half of the CUs idle.  It is cut along one output
 // dimension into a part of exactly k rounds of large tiles and the remaining r tiles,
-// which launch_whole gives to the small tile (4 r workgroups, two per CU: one round).
+// which go to 256 x 128 tiles (2 r workgroups, one per CU) or, for r <= 64, to the small
+// tile (4 r workgroups).
 // Measured on 4096-row problems, K = 4096: +8..12 % at 272..384 tiles, +11..13 % at
 // 544..576, +4 % at 640, +10 % at 800, +1 % at 896; with r > 128 the cut loses 2..3 %.
 // The two parts run one after the other on the caller's stream.
@@ -860,6 +902,14 @@ int launch_shape(const GemmArgs& g, hipStream_t stream) {
       if (cut) {
         const int rc = launch_whole<AK, BKM, EPI, OUT_F32, HALF>(g1, stream);
         if (rc != AXN_OK) return rc;
+        // More than 64 tiles left: 256 x 128 tiles, one per CU on more than half of the CUs
+        // (qkv forward +5 %, down dgrad +3 % against the small tile); fewer: the small tile,
+        // whose 4 r workgroups still give every CU at most one (MLP shard dgrad, r = 64: -7 %
+        // with the 256 x 128 tile).
+        const int64_t a_span = (int64_t)(AK ? g2.M : g2.Kc) * g2.lda * 2;
+        const int64_t b_span = (int64_t)(BKM ? g2.N : g2.Kc) * g2.ldb * 2;
+        if (rest > 64 && a_span < (1LL << 31) && b_span < (1LL << 31))
+          return launch_rest<AK, BKM, EPI, OUT_F32, HALF>(g2, stream);
         return launch_whole<AK, BKM, EPI, OUT_F32, HALF>(g2, stream);
       }
     }

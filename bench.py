@@ -181,7 +181,8 @@ def main():
         dom = max(kinds, key=lambda k: kinds[k]["total_ms"])
         # template arguments: <tile, A contraction-contiguous, B contraction-contiguous, epilogue, fp32 out>.
         # A call whose output is k x 256 + r large tiles with 0 < r <= 128 is two launches, k rounds
-        # of this instance and the rest on its <128, ...> twin; the events bracket the call.
+        # of this instance and the rest on 256 x 128 tiles (gemm_bf16_rest_kernel) or, for r <= 64,
+        # on its <128, ...> twin; the events bracket the call.
         kernel_names = {"fwd": "gemm_bf16_solo_kernel<256, true, true, 0, false> (Y = X W^T)",
                         "dgrad": "gemm_bf16_solo_kernel<256, true, false, 0, false> (dX = dY W)",
                         "wgrad": "gemm_bf16_solo_kernel<256, false, false, 0, false> (dW = dY^T X)"}
