@@ -836,7 +836,7 @@ int launch_rest(const GemmArgs& in, hipStream_t stream) {
 
 // Kernel selection.  Problems made of whole 256 x 256 tiles, more than 128 of
 // them (half of the CUs) and not just above one round of 256, take the
-// one-wave-per-SIMD kernel at that tile size;
+// one-wave-per-SIMD kernel at that tile size, 65..128 of them take it at 256 x 128;
 // other problems made of whole 128 x 128 tiles take it at 128 x 128; ragged
 // shapes, and operands too large for 32-bit byte offsets, take the
 // register-staged kernel.
@@ -858,6 +858,10 @@ int launch_whole(const GemmArgs& g, hipStream_t stream) {
   const bool large_tile = tiles256 > 128 && !(tiles256 > 256 && tiles256 <= 320);
   if (small_spans && whole256 && large_tile)
     return launch_solo<256, AK, BKM, EPI, OUT_F32, HALF>(g, stream);
+  // 65..128 large tiles: 256 x 128 tiles, one workgroup per CU on more than half of the CUs
+  // (+4..11 % against the small tile, measured at 80, 96, 112 and 128 tiles).
+  if (small_spans && whole256 && tiles256 > 64 && tiles256 <= 128)
+    return launch_rest<AK, BKM, EPI, OUT_F32, HALF>(g, stream);
   if (small_spans && whole128 && tiles128 < (1LL << 31))
     return launch_solo<128, AK, BKM, EPI, OUT_F32, HALF>(g, stream);
   if (whole128) return launch_cfg<128, 128, 2, 2, AK, BKM, EPI, OUT_F32, false, HALF>(g, stream);

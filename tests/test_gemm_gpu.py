@@ -223,7 +223,8 @@ def test_fp32_gemms_match_oracle(M, N, K):
 
 @pytest.mark.parametrize("M,N,K", [(128, 128, 64), (256, 384, 192), (512, 256, 320), (4096, 3072, 128),
                                    (4096, 3072, 320), (4608, 4096, 64),
-                                   (4096, 6144, 4096), (4096, 256, 6144), (6144, 4096, 128)])
+                                   (4096, 6144, 4096), (4096, 256, 6144), (6144, 4096, 128),
+                                   (2304, 2048, 192), (2048, 4096, 64)])
 def test_tile_kernels_every_output_block_with_epilogues(M, N, K):
     """Whole-tile shapes on the one-wave-per-SIMD kernel (128 x 128 tiles up to 128
     tiles of 256 x 256 and from 257 to 320 of them, else 256 x 256), checked element by
@@ -232,7 +233,8 @@ def test_tile_kernels_every_output_block_with_epilogues(M, N, K):
     other shapes).  The last three shapes have 384 large tiles in one of their products:
     one full round of large tiles and a rest of 128 for the small tile, cut along the
     output columns (forward of the first, dgrad of the second) or rows (wgrad of the
-    first, forward of the third), with the bias and the saved pre-activation cut too."""
+    first, forward of the third), with the bias and the saved pre-activation cut too.  The
+    last two have 72 and 128 large tiles in their forward: 256 x 128 tiles throughout."""
     from axonn_amd import ops
 
     g = torch.Generator(device="cuda").manual_seed(M + N + K)
