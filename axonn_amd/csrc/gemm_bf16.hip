@@ -437,12 +437,13 @@ __device__ __forceinline__ void wait_vmcnt() {
 //
 // LDS holds a ring of 5 operand tiles (160 KiB); the tiles A0 B0 A1 B1 A2 ... of
 // the contraction stages take the slots 0 1 2 3 4 0 1 ...  Stage p (64 deep):
-//   step 0 : MFMAs | reads of (p, 1) | this wave's 8 copies of A(p+2)
+//   step 0 : MFMAs | this wave's 8 copies of A(p+2) | reads of (p, 1)
 //   step 1 : wait for own copies of A(p+1), B(p+1); barrier;
-//            MFMAs | reads of (p+1, 0) | this wave's 8 copies of B(p+2)
+//            MFMAs | this wave's 8 copies of B(p+2) | reads of (p+1, 0)
 // At the barrier every wave holds the last fragments of stage p in registers, so
 // both of its slots are free: B(p+2) takes A(p)'s, A(p+3) (next step 0) B(p)'s.
-// A tile has at least two steps (128 MFMAs per wave) to land.
+// The copies come first in a step, the reads second: a tile has at least a whole
+// stage (128 MFMAs per wave) to land.
 //
 // TILE = 128 is the same schedule on a 128 x 128 tile for problems that do not
 // fill the chip with 256 x 256 tiles: 64 x 64 per wave (4 x 4 blocks, 16 MFMAs per
@@ -602,15 +603,21 @@ __device__ __forceinline__ void solo_gemm(const GemmArgs& g) {
                        : "v"(fb[j]), "v"(fa[i]));
         constexpr int CE = ST == 0 ? COPY_EVERY_A : COPY_EVERY_B;  // step 0 copies A, step 1 B
         constexpr int NCX = ST == 0 ? NCA : NCB;
-        if constexpr (m < NM / 2 && m % READ_EVERY == 0 && m / READ_EVERY < NFRAG) {
+        // Copies in the first half of a step, fragment reads in the second: a copy is issued
+        // as soon as the barrier (step 1) or the previous step (step 0) has freed its slot,
+        // which gives the tile a quarter of a stage more to arrive than the other order
+        // (measured: +2.6 % on the step, +7 % on the MLP shard); the reads still have half
+        // a step to return.
+        constexpr int mc = m;            // position in the copying half
+        constexpr int mr = m - NM / 2;   // position in the reading half
+        if constexpr (mr >= 0 && mr < NM / 2 && mr % READ_EVERY == 0 && mr / READ_EVERY < NFRAG) {
           if constexpr (ST == 0) read(std::integral_constant<int, 1>{},
-                                      std::integral_constant<int, m / READ_EVERY>{}, sa, sb);
+                                      std::integral_constant<int, mr / READ_EVERY>{}, sa, sb);
           else if constexpr (!LAST) read(std::integral_constant<int, 0>{},
-                                         std::integral_constant<int, m / READ_EVERY>{}, na, nb);
-        } else if constexpr (HAS2 && m >= NM / 2 && (m - NM / 2) % CE == CE - 1 &&
-                             (m - NM / 2) / CE < NCX) {
-          if constexpr (ST == 0) copy_a(std::integral_constant<int, (m - NM / 2) / CE>{});
-          else copy_b(std::integral_constant<int, (m - NM / 2) / CE>{});
+                                         std::integral_constant<int, mr / READ_EVERY>{}, na, nb);
+        } else if constexpr (HAS2 && mc >= 0 && mc < NM / 2 && mc % CE == CE - 1 && mc / CE < NCX) {
+          if constexpr (ST == 0) copy_a(std::integral_constant<int, mc / CE>{});
+          else copy_b(std::integral_constant<int, mc / CE>{});
         }
         __builtin_amdgcn_sched_barrier(0);
       });
