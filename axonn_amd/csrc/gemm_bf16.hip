@@ -615,7 +615,10 @@ __device__ __forceinline__ void solo_gemm(const GemmArgs& g) {
                                       std::integral_constant<int, mr / READ_EVERY>{}, sa, sb);
           else if constexpr (!LAST) read(std::integral_constant<int, 0>{},
                                          std::integral_constant<int, mr / READ_EVERY>{}, na, nb);
-        } else if constexpr (HAS2 && mc >= 0 && mc < NM / 2 && mc % CE == CE - 1 && mc / CE < NCX) {
+        }
+        // (an independent statement: a read and a copy may fall behind the same MFMA)
+        static_assert((NM / 2) / CE >= NCX, "every copy of the tile has a place in the half step");
+        if constexpr (HAS2 && mc >= 0 && mc < NM / 2 && mc % CE == CE - 1 && mc / CE < NCX) {
           if constexpr (ST == 0) copy_a(std::integral_constant<int, mc / CE>{});
           else copy_b(std::integral_constant<int, mc / CE>{});
         }
