@@ -41,8 +41,8 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 # file, scaled by what the same counters read for the 1 GiB copy below
 # (profiles/gemm_adam_llama_set_pmc.txt has the runs and the arithmetic).  The
 # counters sit between L2 and the fabric, so hits in the memory-side cache are included.
-TRAFFIC_BYTES_PER_LAUNCH = {"fwd": 634719198, "dgrad": 593501297, "wgrad": 670422671}
-ADAM_TRAFFIC_BYTES_PER_STEP = 39290548955   # scan + update, 1.3e9 elements
+TRAFFIC_BYTES_PER_LAUNCH = {"fwd": 634630868, "dgrad": 587543761, "wgrad": 664843464}
+ADAM_TRAFFIC_BYTES_PER_STEP = 39291755669   # scan + update, 1.3e9 elements
 
 LLAMA_SET = [  # (name, M, N, K), gate and up are two layers of one shape
     ("qkv", 4096, 6144, 4096),
