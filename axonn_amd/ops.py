@@ -81,6 +81,11 @@ def gemm_fwd(x, w, bias=None, activation=None, save_z=False):
         if bias.numel() != N:
             raise ValueError("bias has %d elements, expected %d" % (bias.numel(), N))
     want_z = activation is not None and save_z
+    if x.dtype not in _GEMM16 and x.dtype != torch.float32:
+        raise TypeError("the Linear kernels take bf16, fp16 or fp32 operands, got %s" % x.dtype)
+    if M == 0:  # an empty batch: nothing to launch (the library takes M >= 1)
+        y = torch.empty((0, N), dtype=x.dtype, device=x.device)
+        return y, (torch.empty_like(y) if want_z else None)
     if x.dtype in _GEMM16:
         x, ldx = _prep_bf16(x)
         w, ldw = _prep_bf16(w)
@@ -112,6 +117,10 @@ def gemm_dgrad(dy, w):
         raise TypeError("grad_output is %s but weight is %s" % (dy.dtype, w.dtype))
     M, N = dy.shape
     K = w.shape[1]
+    if dy.dtype not in _GEMM16 and dy.dtype != torch.float32:
+        raise TypeError("the Linear kernels take bf16, fp16 or fp32 operands, got %s" % dy.dtype)
+    if M == 0:
+        return torch.empty((0, K), dtype=dy.dtype, device=dy.device)
     if dy.dtype in _GEMM16:
         dy, lddy = _prep_bf16(dy)
         w, ldw = _prep_bf16(w)
@@ -150,6 +159,11 @@ def gemm_wgrad(dy, x, out=None, accumulate=False, out_dtype=None):
         raise ValueError("accumulate=True needs `out`")
     if out_dtype is None:
         out_dtype = dy.dtype
+    if M == 0 and (dy.dtype in _GEMM16 or dy.dtype == torch.float32):
+        # an empty batch contributes a zero gradient
+        if out is None:
+            return torch.zeros((N, K), dtype=out_dtype, device=dy.device)
+        return out if accumulate else out.zero_()
     if dy.dtype in _GEMM16:
         if out_dtype not in (dy.dtype, torch.float32):
             raise TypeError("dW must be %s or fp32, got %s" % (dy.dtype, out_dtype))
@@ -190,6 +204,15 @@ def dgelu_dbias(dy, z=None, want_dbias=True, dbias_out=None, accumulate=False):
         ld = dy.shape[1]
     M, N = dy.shape
     dz = None
+    if M == 0:
+        if z is not None and (z.dtype != dy.dtype or z.shape != dy.shape):
+            raise ValueError("z must match dy in dtype and shape")
+        dbias = None
+        if want_dbias:
+            dbias = dbias_out if dbias_out is not None else torch.zeros(N, dtype=torch.float32, device=dy.device)
+            if dbias_out is not None and not accumulate:
+                dbias.zero_()
+        return (torch.empty_like(dy) if z is not None else dy), dbias
     if z is not None:
         if z.dtype != dy.dtype or z.shape != dy.shape:
             raise ValueError("z must match dy in dtype and shape")
@@ -242,6 +265,8 @@ def swiglu_fwd(gate, up):
     gate, up = _swiglu_operands("swiglu_fwd", [gate, up])
     M, N = gate.shape
     out = torch.empty_like(gate)
+    if M == 0:
+        return out
     nv.call("axn_swiglu_fwd", nv.ptr(gate), nv.ptr(up), nv.ptr(out), nv.dtype_code(gate.dtype),
             M, N, N, nv.current_stream())
     return out
@@ -253,6 +278,8 @@ def swiglu_bwd(dout, gate, up):
     dout, gate, up = _swiglu_operands("swiglu_bwd", [dout, gate, up])
     M, N = gate.shape
     dgate, dup = torch.empty_like(gate), torch.empty_like(up)
+    if M == 0:
+        return dgate, dup
     nv.call("axn_swiglu_bwd", nv.ptr(dout), nv.ptr(gate), nv.ptr(up), nv.ptr(dgate), nv.ptr(dup),
             nv.dtype_code(gate.dtype), M, N, N, nv.current_stream())
     return dgate, dup

@@ -105,6 +105,28 @@ def test_bf16_layer_matches_oracle(B, Hin, Hout, bias, act):
         assert r(layer.bias.grad, bw["db"]) < 1e-2
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("act", [None, "gelu"])
+def test_empty_batch_behaves_like_torch(dtype, act):
+    """No rows: the output is empty and every gradient is zero, as with torch.nn.Linear."""
+    kw = {"fused_activation": act} if act else {}
+    layer, seq = make_pair(64, 128, True, dtype, **kw)
+    X = torch.empty(0, 64, dtype=dtype, device="cuda", requires_grad=True)
+    Xs = X.detach().clone().requires_grad_(True)
+    Y = layer(X)
+    Ys = seq(Xs)
+    if act:
+        Ys = torch.nn.functional.gelu(Ys)
+    assert Y.shape == Ys.shape == (0, 128) and Y.dtype == Ys.dtype
+    Y.sum().backward()
+    Ys.sum().backward()
+    assert X.grad.shape == Xs.grad.shape == (0, 64)
+    assert layer.weight.grad.shape == layer.weight.shape
+    assert torch.equal(layer.weight.grad.view_as(seq.weight.grad), seq.weight.grad)   # zeros
+    assert torch.equal(layer.bias.grad, seq.bias.grad)
+    assert not layer.weight.grad.any() and not layer.bias.grad.any()
+
+
 def test_skip_bias_add_returns_tuple():
     layer, seq = make_pair(64, 64, True, torch.bfloat16, skip_bias_add=True)
     X = torch.randn(8, 64).bfloat16().cuda()
@@ -181,7 +203,7 @@ def test_two_layer_mlp_step_matches_cpu_path():
     y = model(x.cuda())
     loss = torch.nn.functional.mse_loss(y, tgt.cuda())
     loss.backward()
-    assert abs(float(loss) - float(want["loss"])) < 1e-5 * float(want["loss"])
+    assert abs(float(loss.detach()) - float(want["loss"])) < 1e-5 * float(want["loss"])
     grads = [p.grad.detach().clone() for p in model.parameters()]
     for g, w in zip(grads, want["grads"]):
         assert rel(g.reshape(-1), w.reshape(-1)) < 1e-4
