@@ -34,6 +34,7 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 PEAK_BF16_TFLOPS = 2516.6   # MI355X dense bf16 MFMA
+EVENT_EVERY = 4              # timed steps between two steps whose launches are bracketed by events
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 
 # HBM bytes per launch (read + written), averaged over the launches of each kernel in
@@ -41,8 +42,8 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 # file, scaled by what the same counters read for the 1 GiB copy below
 # (profiles/gemm_adam_llama_set_pmc.txt has the runs and the arithmetic).  The
 # counters sit between L2 and the fabric, so hits in the memory-side cache are included.
-TRAFFIC_BYTES_PER_LAUNCH = {"fwd": 634630868, "dgrad": 587543761, "wgrad": 664843464}
-ADAM_TRAFFIC_BYTES_PER_STEP = 39291755669   # scan + update, 1.3e9 elements
+TRAFFIC_BYTES_PER_LAUNCH = {"fwd": 634638544, "dgrad": 587542396, "wgrad": 664855104}
+ADAM_TRAFFIC_BYTES_PER_STEP = 39286797387   # scan + update, 1.3e9 elements
 
 LLAMA_SET = [  # (name, M, N, K), gate and up are two layers of one shape
     ("qkv", 4096, 6144, 4096),
@@ -161,8 +162,10 @@ def main():
         step(False)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step(True)
+    # Events bracket the launches of every fourth timed step: recorded on every step they cost
+    # 0.7-1.5 % of the step, and the per-kernel averages need no more samples than that.
+    for i in range(args.steps):
+        step(i % EVENT_EVERY == 0)
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
     ms_per_step = elapsed / args.steps * 1e3
@@ -191,6 +194,7 @@ def main():
             "achieved": round(kinds[dom]["tflops"], 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
             "frac": round(kinds[dom]["tflops"] / PEAK_BF16_TFLOPS, 4),
             "avg_launch_us": round(kinds[dom]["avg_us"], 1),
+            "launches_timed": kinds[dom]["launches"],  # those of every EVENT_EVERY-th timed step
             "flops_per_launch": kinds[dom]["tflops"] * 1e12 * kinds[dom]["avg_us"] * 1e-6,
             "traffic": TRAFFIC_BYTES_PER_LAUNCH.get(dom),
             "per_kernel": {k: {"avg_us": round(v["avg_us"], 1), "tflops": round(v["tflops"], 1),
