@@ -363,6 +363,11 @@ def main():
         del table, ids, dye, oute, dtab, wse
         torch.cuda.empty_cache()
 
+        # The reference's CPU-runnable configuration: batch 64, 1024 -> 4096 GELU -> 1024 in
+        # fp32, MSE loss, one Adam step, through the package's modules (launch-bound: a
+        # sanity figure, not a roofline target).
+        shapes["mlp_64x1024x4096x1024_fp32_train_step"] = small_mlp_step(torch, time_loop)
+
     adam = None
     if not args.no_adam:
         adam = bench_adam(args, torch, nv, lib, stream, time_loop)
@@ -372,6 +377,9 @@ def main():
         cpu = cpu_baseline(torch)
         if adam is not None:
             adam["cpu_baseline"] = cpu_adam_baseline(torch)
+        key = "mlp_64x1024x4096x1024_fp32_train_step"
+        if key in shapes:
+            shapes[key]["cpu_baseline"] = cpu_small_mlp_baseline(torch)
 
     out = {
         "metric": "Linear fwd+bwd TFLOP/s on the Llama-3-8B-shaped set (Adam step GB/s under 'adam')",
@@ -391,6 +399,54 @@ def main():
         "shapes": shapes,
     }
     print(json.dumps(out))
+
+
+def small_mlp_tensors(torch):
+    import math
+
+    torch.manual_seed(0)
+    w1 = torch.nn.init.kaiming_uniform_(torch.empty(4096, 1024), a=math.sqrt(5))
+    w2 = torch.nn.init.kaiming_uniform_(torch.empty(1024, 4096), a=math.sqrt(5))
+    return w1, torch.zeros(4096), w2, torch.zeros(1024), torch.randn(64, 1024), torch.randn(64, 1024)
+
+
+def small_mlp_step(torch, time_loop):
+    from axonn_amd.intra_layer import Linear
+    from axonn_amd.optim import CPUAdam
+
+    w1, b1, w2, b2, x, tgt = small_mlp_tensors(torch)
+    l1 = Linear(1024, 4096, fused_activation="gelu")
+    l2 = Linear(4096, 1024)
+    l1.load_state_dict({"weight": w1, "bias": b1})
+    l2.load_state_dict({"weight": w2, "bias": b2})
+    model = torch.nn.Sequential(l1, l2).cuda()
+    opt = CPUAdam(model.parameters(), lr=1e-3, betas=(0.9, 0.999), eps=1e-8)
+    x, tgt = x.cuda(), tgt.cuda()
+
+    def train_step():
+        opt.zero_grad()
+        torch.nn.functional.mse_loss(model(x), tgt).backward()
+        opt.step()
+
+    t = time_loop(train_step, 20)
+    flops = 2 * 3 * 2.0 * 64 * 1024 * 4096
+    return {"us_per_step": round(t * 1e6, 1), "gflops": round(flops / t / 1e9, 1)}
+
+
+def cpu_small_mlp_baseline(torch):
+    from oracle import torch_cpu as ot
+
+    w1, b1, w2, b2, x, tgt = small_mlp_tensors(torch)
+    ot.mlp_step(x, tgt, w1, b1, w2, b2)
+    reps = 10
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        ot.mlp_step(x, tgt, w1, b1, w2, b2)
+    secs = (time.perf_counter() - t0) / reps
+    flops = 2 * 3 * 2.0 * 64 * 1024 * 4096
+    return {"us_per_step": round(secs * 1e6, 1), "gflops": round(flops / secs / 1e9, 1),
+            "cores": torch.get_num_threads(), "kind": "port",
+            "sample": "the same step in torch CPU ops, %d timed steps" % reps}
 
 
 def adam_sizes(total, n=64, seed=0):
