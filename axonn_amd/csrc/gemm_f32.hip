@@ -92,12 +92,15 @@ __device__ __forceinline__ void load_block(float (&x)[F][4], const float* __rest
   }
 }
 
-template <bool AK, bool BKM, int EPI, int FM, int FN, int U, bool VEC>
-__global__ void __launch_bounds__(64)
+// WAVES > 1: the waves of a workgroup share one tile and take the 16 U-deep chunks of
+// the contraction in turn; their partial sums meet in LDS and are added in wave order.
+template <bool AK, bool BKM, int EPI, int FM, int FN, int U, bool VEC, int WAVES>
+__global__ void __launch_bounds__(64 * WAVES)
     gemm_f32_kernel(const float* __restrict__ A, const float* __restrict__ B,
                     float* __restrict__ C, const float* __restrict__ bias,
                     float* __restrict__ Z, int M, int N, int Kc, int tiles_n, int beta) {
-  const int lane = threadIdx.x;
+  const int lane = threadIdx.x & 63;
+  const int wave = WAVES > 1 ? threadIdx.x >> 6 : 0;
   const int r = lane & 15, q = lane >> 4;
   const int tm = blockIdx.x / tiles_n, tn = blockIdx.x - tm * tiles_n;
   const int m0 = tm * 16 * FM, n0 = tn * 16 * FN;
@@ -132,11 +135,29 @@ __global__ void __launch_bounds__(64)
             acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[u][i][s], b[u][j][s], acc[i][j], 0, 0, 0);
   };
 
-  int k0 = 0;
-  for (; k0 + 16 * U <= Kc; k0 += 16 * U)
+  const int whole = Kc / (16 * U) * (16 * U);  // the part made of whole chunks
+  for (int k0 = wave * 16 * U; k0 < whole; k0 += WAVES * 16 * U)
     blocks(std::false_type{}, k0, std::integral_constant<int, U>{});
-  for (; k0 < Kc; k0 += 16)
+  for (int k0 = whole + wave * 16; k0 < Kc; k0 += WAVES * 16)
     blocks(std::true_type{}, k0, std::integral_constant<int, 1>{});
+
+  if constexpr (WAVES > 1) {
+    __shared__ f32x4 part[WAVES - 1][FM * FN][64];
+    if (wave > 0) {
+#pragma unroll
+      for (int i = 0; i < FM; ++i)
+#pragma unroll
+        for (int j = 0; j < FN; ++j) part[wave - 1][i * FN + j][lane] = acc[i][j];
+    }
+    __syncthreads();
+    if (wave > 0) return;
+#pragma unroll
+    for (int w = 0; w < WAVES - 1; ++w)
+#pragma unroll
+      for (int i = 0; i < FM; ++i)
+#pragma unroll
+        for (int j = 0; j < FN; ++j) acc[i][j] += part[w][i * FN + j][lane];
+  }
 
   // Register v of acc[i][j] in lane (r, q) is output row FM (4 q + v) + i, column FN r + j.
   using vec = typename VecOf<FN>::type;
@@ -198,7 +219,7 @@ __global__ void __launch_bounds__(64)
     }
 }
 
-template <bool AK, bool BKM, int EPI, int FM, int FN, int U>
+template <bool AK, bool BKM, int EPI, int FM, int FN, int U, int WAVES>
 int launch_tile(const float* A, const float* B, float* C, const float* bias, float* Z, int M,
                 int N, int Kc, int beta, hipStream_t stream) {
   const long long tiles_m = (M + 16 * FM - 1) / (16 * FM), tiles_n = (N + 16 * FN - 1) / (16 * FN);
@@ -212,28 +233,32 @@ int launch_tile(const float* A, const float* B, float* C, const float* bias, flo
   const uintptr_t ptrs = (uintptr_t)A | (uintptr_t)B | (uintptr_t)C | (uintptr_t)bias | (uintptr_t)Z;
   const bool vec = Kc % 4 == 0 && (AK || M % FM == 0) && N % FN == 0 && (ptrs & 15u) == 0;
   if (vec)
-    hipLaunchKernelGGL((gemm_f32_kernel<AK, BKM, EPI, FM, FN, U, true>), dim3((unsigned)nwg), dim3(64),
-                       0, stream, A, B, C, bias, Z, M, N, Kc, (int)tiles_n, beta);
+    hipLaunchKernelGGL((gemm_f32_kernel<AK, BKM, EPI, FM, FN, U, true, WAVES>), dim3((unsigned)nwg),
+                       dim3(64 * WAVES), 0, stream, A, B, C, bias, Z, M, N, Kc, (int)tiles_n, beta);
   else
-    hipLaunchKernelGGL((gemm_f32_kernel<AK, BKM, EPI, FM, FN, U, false>), dim3((unsigned)nwg),
-                       dim3(64), 0, stream, A, B, C, bias, Z, M, N, Kc, (int)tiles_n, beta);
+    hipLaunchKernelGGL((gemm_f32_kernel<AK, BKM, EPI, FM, FN, U, false, WAVES>), dim3((unsigned)nwg),
+                       dim3(64 * WAVES), 0, stream, A, B, C, bias, Z, M, N, Kc, (int)tiles_n, beta);
   AXN_HIP_TRY(hipGetLastError());
   return AXN_OK;
 }
 
 // The largest of the 64 x 64, 32 x 32 and 16 x 16 tiles (a loaded element is used 4,
 // 2, 1 times) that still gives the chip's 1024 SIMDs a wave each; smaller tiles keep
-// more loads in flight per wave.
+// more loads in flight per wave.  A small output with a long contraction (fewer than
+// 1024 of the smallest tiles, more than one chunk per wave) puts four waves on a tile.
 template <bool AK, bool BKM, int EPI>
 int launch_epi(const float* A, const float* B, float* C, const float* bias, float* Z, int M, int N,
                int Kc, int beta, hipStream_t stream) {
   const long long tiles64 = (long long)((M + 63) / 64) * ((N + 63) / 64);
   const long long tiles32 = (long long)((M + 31) / 32) * ((N + 31) / 32);
+  const long long tiles16 = (long long)((M + 15) / 16) * ((N + 15) / 16);
   if (tiles64 >= 1024)
-    return launch_tile<AK, BKM, EPI, 4, 4, 2>(A, B, C, bias, Z, M, N, Kc, beta, stream);
+    return launch_tile<AK, BKM, EPI, 4, 4, 2, 1>(A, B, C, bias, Z, M, N, Kc, beta, stream);
   if (tiles32 >= 1024)
-    return launch_tile<AK, BKM, EPI, 2, 2, 4>(A, B, C, bias, Z, M, N, Kc, beta, stream);
-  return launch_tile<AK, BKM, EPI, 1, 1, 8>(A, B, C, bias, Z, M, N, Kc, beta, stream);
+    return launch_tile<AK, BKM, EPI, 2, 2, 4, 1>(A, B, C, bias, Z, M, N, Kc, beta, stream);
+  if (tiles16 < 1024 && Kc >= 4 * 16 * 4)
+    return launch_tile<AK, BKM, EPI, 1, 1, 4, 4>(A, B, C, bias, Z, M, N, Kc, beta, stream);
+  return launch_tile<AK, BKM, EPI, 1, 1, 8, 1>(A, B, C, bias, Z, M, N, Kc, beta, stream);
 }
 
 }  // namespace
