@@ -244,8 +244,17 @@ int launch_tile(const float* A, const float* B, float* C, const float* bias, flo
 
 // The largest of the 64 x 64, 32 x 32 and 16 x 16 tiles (a loaded element is used 4,
 // 2, 1 times) that still gives the chip's 1024 SIMDs a wave each; smaller tiles keep
-// more loads in flight per wave.  A small output with a long contraction (fewer than
-// 1024 of the smallest tiles, more than one chunk per wave) puts four waves on a tile.
+// more loads in flight per wave.  With fewer than 4096 tiles and a contraction of KMIN
+// or more (256 for the smallest tile, 2048 for the middle one; measured: the split
+// loses on the largest tile and on shorter contractions), four waves share a tile.
+template <bool AK, bool BKM, int EPI, int FM, int FN, int U, int KMIN>
+int launch_waves(long long tiles, const float* A, const float* B, float* C, const float* bias,
+                 float* Z, int M, int N, int Kc, int beta, hipStream_t stream) {
+  if (tiles < 4096 && Kc >= KMIN)
+    return launch_tile<AK, BKM, EPI, FM, FN, (U > 4 ? 4 : U), 4>(A, B, C, bias, Z, M, N, Kc, beta, stream);
+  return launch_tile<AK, BKM, EPI, FM, FN, U, 1>(A, B, C, bias, Z, M, N, Kc, beta, stream);
+}
+
 template <bool AK, bool BKM, int EPI>
 int launch_epi(const float* A, const float* B, float* C, const float* bias, float* Z, int M, int N,
                int Kc, int beta, hipStream_t stream) {
@@ -255,10 +264,8 @@ int launch_epi(const float* A, const float* B, float* C, const float* bias, floa
   if (tiles64 >= 1024)
     return launch_tile<AK, BKM, EPI, 4, 4, 2, 1>(A, B, C, bias, Z, M, N, Kc, beta, stream);
   if (tiles32 >= 1024)
-    return launch_tile<AK, BKM, EPI, 2, 2, 4, 1>(A, B, C, bias, Z, M, N, Kc, beta, stream);
-  if (tiles16 < 1024 && Kc >= 4 * 16 * 4)
-    return launch_tile<AK, BKM, EPI, 1, 1, 4, 4>(A, B, C, bias, Z, M, N, Kc, beta, stream);
-  return launch_tile<AK, BKM, EPI, 1, 1, 8, 1>(A, B, C, bias, Z, M, N, Kc, beta, stream);
+    return launch_waves<AK, BKM, EPI, 2, 2, 4, 2048>(tiles32, A, B, C, bias, Z, M, N, Kc, beta, stream);
+  return launch_waves<AK, BKM, EPI, 1, 1, 8, 256>(tiles16, A, B, C, bias, Z, M, N, Kc, beta, stream);
 }
 
 }  // namespace

@@ -205,13 +205,13 @@ def test_unsupported_shapes_raise():
 @pytest.mark.parametrize("M,N,K", [(1, 1, 1), (5, 7, 3), (64, 48, 40), (130, 70, 257), (66, 130, 8),
                                    (33, 17, 1000), (64, 1024, 4096),
                                    (1030, 1034, 70), (1032, 1040, 72), (2050, 2052, 36), (2048, 2064, 40),
-                                   (2049, 2051, 33)])
+                                   (2049, 2051, 33), (2048, 1030, 1034)])
 def test_fp32_gemms_match_oracle(M, N, K):
     """Ragged and whole shapes on each of the fp32 kernel's tiles (16, 32 and 64 rows and
     columns per wave: the last five shapes), with and without the divisibility its vector
     loads and stores need; small outputs with a contraction of 256 or more have four waves
-    share a tile (each of the three products of (64, 1024, 4096) and (33, 17, 1000) has
-    one such case or more)."""
+    share a tile (products of (64, 1024, 4096) and (33, 17, 1000)), and so do 1024 to 4095
+    of the 32 x 32 tiles with a contraction of 2048 or more (wgrad of the last shape)."""
     from axonn_amd import ops
 
     g = torch.Generator().manual_seed(M + N + K)
