@@ -24,36 +24,30 @@ from ..axonn import get_world_size
 from .communication import Drop, ForwardGather_BackwardReduceScatter, Gather
 
 
-def divide(a, b):
-    assert a % b == 0
-    return a // b
+def _flat_shard(table, column_group, row_group, depth_group):
+    """This rank's part of a full [num_embeddings, embedding_dim] table as the flat vector
+    the parameter holds: the columns of `column_group`'s slice, every row (`row_group`
+    has one member), row-major, and of that vector the slice of `depth_group`
+    (axonn/intra_layer/embedding.py:23-32 fixes this order; it is the checkpoint
+    format).  On one GPU: the table, flattened."""
+    with torch.no_grad():
+        part = Drop.apply(table, column_group)
+        part = Drop.apply(part.t().contiguous(), row_group).t().contiguous()
+        return Drop.apply(part.reshape(-1), depth_group)
 
 
-@torch.no_grad()
-def extract_local_params_from_full_params(params, out_features_group, in_features_group,
-                                          depth_group):
-    """[num_embeddings, embedding_dim] -> this rank's flat shard (columns first)."""
-    params = Drop.apply(params, out_features_group)
-    params = Drop.apply(torch.t(params).contiguous(), in_features_group)
-    params = torch.t(params).contiguous()
-    return Drop.apply(params.reshape(-1), depth_group)
-
-
-@torch.no_grad()
-def initialize_params(out_features, in_features, out_features_group, in_features_group,
-                      depth_group, init_method, init_device=None):
-    if init_device is None:
-        init_device = "cuda" if torch.cuda.is_available() else "cpu"
-    params = torch.empty((in_features, out_features), device=init_device)
-    init_method(params)
-    return extract_local_params_from_full_params(
-        params, out_features_group, in_features_group, depth_group
-    ).cpu()
-
-
-@torch.no_grad()
 def default_init_method(weight, padding_idx=None):
-    return torch.nn.init.normal_(weight)
+    """normal(0, 1), torch.nn.Embedding's own default (:52-54)."""
+    with torch.no_grad():
+        return torch.nn.init.normal_(weight)
+
+
+def _resolve_padding_idx(padding_idx, num_embeddings):
+    """torch.nn.Embedding's rule (:78-88): in range, negative values count from the end."""
+    if padding_idx is None:
+        return None
+    assert -num_embeddings <= padding_idx < num_embeddings, "Padding_idx must be within num_embeddings"
+    return padding_idx + num_embeddings if padding_idx < 0 else padding_idx
 
 
 class _Lookup(torch.autograd.Function):
@@ -98,6 +92,10 @@ def embedding(ids, weight, padding_idx=None, max_norm=None, norm_type=2.0,
 
 
 class Embedding(torch.nn.Module):
+    """`torch.nn.Embedding`'s arguments, then the reference's (:57-74).  `weight` is the
+    flat shard; `forward` returns [..., embedding_dim] (in expert mode: this rank's
+    columns)."""
+
     def __init__(
         self,
         num_embeddings,
@@ -116,106 +114,70 @@ class Embedding(torch.nn.Module):
         **kwargs,
     ):
         assert _weight is None, "_weight argument is not supported."
-        super(Embedding, self).__init__()
-        self.num_embeddings = num_embeddings
-        self.embedding_dim = embedding_dim
-        if padding_idx is not None:
-            if padding_idx > 0:
-                assert padding_idx < num_embeddings, "Padding_idx must be within num_embeddings"
-            elif padding_idx < 0:
-                assert padding_idx >= -num_embeddings, "Padding_idx must be within num_embeddings"
-                padding_idx = num_embeddings + padding_idx
-        self.padding_idx = padding_idx
-        self.max_norm = max_norm
-        self.norm_type = norm_type
-        self.scale_grad_by_freq = scale_grad_by_freq
-        self.sparse = sparse
-
+        super().__init__()
         handle = ax._handle()
         self.inner_group = handle.inner_intra_layer_parallel_group
         self.outer_group = handle.outer_intra_layer_parallel_group
         self.depth_group = handle.depth_intra_layer_parallel_group
-        self.inner_group_size = get_world_size(self.inner_group)
-        self.outer_group_size = get_world_size(self.outer_group)
-        self.depth_group_size = get_world_size(self.depth_group)
-
-        self.out_features = embedding_dim
-        self.in_features = num_embeddings
-        if init_method is None:
-            init_method = default_init_method
-
-        # The embedding width is split over one of the two tensor-parallel groups; the
-        # vocabulary is never split.
-        if not transpose:
-            assert self.inner_group_size == 1
-            self._column_group, self._row_group = self.outer_group, self.inner_group
-        else:
-            assert self.outer_group_size == 1
-            self._column_group, self._row_group = self.inner_group, self.outer_group
+        self.inner_group_size, self.outer_group_size, self.depth_group_size = (
+            get_world_size(g) for g in (self.inner_group, self.outer_group, self.depth_group))
+        # The embedding width is split over one of the two tensor-parallel groups (the
+        # outer one unless `transpose`), the other must be trivial: the vocabulary is
+        # never split (:107-134).
+        self._column_group, self._row_group = (
+            (self.inner_group, self.outer_group) if transpose else (self.outer_group, self.inner_group))
+        assert get_world_size(self._row_group) == 1
         columns = get_world_size(self._column_group)
         assert embedding_dim % columns == 0
-        self.local_in_features = num_embeddings
-        self.local_out_features = divide(embedding_dim, columns)
-        initial_params = initialize_params(
-            self.out_features, self.in_features, self._column_group, self._row_group,
-            self.depth_group, init_method,
-        )
+
+        self.num_embeddings = self.in_features = self.local_in_features = num_embeddings
+        self.embedding_dim = self.out_features = embedding_dim
+        self.local_out_features = embedding_dim // columns
+        self.padding_idx = _resolve_padding_idx(padding_idx, num_embeddings)
+        self.max_norm, self.norm_type = max_norm, norm_type
+        self.scale_grad_by_freq, self.sparse = scale_grad_by_freq, sparse
+        self.expert_mode, self.transpose = expert_mode, transpose
+
+        # Drawn as the full table on the device (as the reference does, :34-49), then cut.
+        device = "cuda" if torch.cuda.is_available() else "cpu"
+        table = torch.empty((num_embeddings, embedding_dim), device=device)
+        (init_method or default_init_method)(table)
+        shard = _flat_shard(table, self._column_group, self._row_group, self.depth_group).cpu()
         if self.padding_idx is not None:
             # The shard is row-major, so a row of the table is a run of the flat vector;
             # this rank zeroes the part of it that falls into its depth slice.  (The
             # reference indexes the 1-D parameter with the row number, :136-137, which
             # zeroes a single element; the whole row is what torch.nn.Embedding gives.)
-            n = initial_params.numel()
-            lo = (self.padding_idx * self.local_out_features
-                  - handle.intra_layer_depth_parallel_rank * n)
-            hi = lo + self.local_out_features
-            initial_params[max(lo, 0):max(min(hi, n), 0)].fill_(0)
+            first = (self.padding_idx * self.local_out_features
+                     - handle.intra_layer_depth_parallel_rank * shard.numel())
+            last = first + self.local_out_features
+            shard[max(first, 0):max(min(last, shard.numel()), 0)] = 0
 
-        self.weight = torch.nn.Parameter(initial_params, requires_grad=not _freeze)
-        setattr(self.weight, "is_tensor_parallel", True)
-        setattr(self.weight, "needs_depth_parallel_gradient_sync", False)
-        setattr(self.weight, "process_group_for_norm_reduction", handle.intra_layer_group)
-
-        self.expert_mode = expert_mode
-        self.transpose = transpose
-        self._old_load_from_state_dict = self._load_from_state_dict
-        self._load_from_state_dict = self._modified_load_from_state_dict
+        self.weight = torch.nn.Parameter(shard, requires_grad=not _freeze)
+        # read by gradient sync and clipping (:141-148)
+        self.weight.is_tensor_parallel = True
+        self.weight.needs_depth_parallel_gradient_sync = False
+        self.weight.process_group_for_norm_reduction = handle.intra_layer_group
+        # a full 2-D table in a checkpoint is cut to this rank's shard on the way in (:191-222)
+        self._register_load_state_dict_pre_hook(self._shard_incoming_weight)
 
     def get_output_feature_size(self):
         return self.local_out_features
 
     def forward(self, x):
-        weight = ForwardGather_BackwardReduceScatter.apply(self.weight, self.depth_group).reshape(
-            self.local_in_features, self.local_out_features
-        )
-        x = embedding(x, weight, self.padding_idx, self.max_norm, self.norm_type,
-                      self.scale_grad_by_freq, self.sparse)
-        if not self.expert_mode:
-            x = Gather.apply(x, self._column_group)
-        return x
+        table = ForwardGather_BackwardReduceScatter.apply(self.weight, self.depth_group)
+        rows = embedding(x, table.view(self.local_in_features, self.local_out_features), self.padding_idx,
+                         self.max_norm, self.norm_type, self.scale_grad_by_freq, self.sparse)
+        return rows if self.expert_mode else Gather.apply(rows, self._column_group)
 
-    def _is_full_weight_matrix(self, weight):
-        return (
-            weight.ndim == 2
-            and weight.size(0) == self.in_features
-            and weight.size(1) == self.out_features
-        )
-
-    def _is_sharded_weight_matrix(self, weight):
-        return weight.ndim == 1 and weight.size(0) == divide(
-            self.local_out_features * self.local_in_features, self.depth_group_size
-        )
-
-    @torch.no_grad()
-    def _modified_load_from_state_dict(self, state_dict, prefix, *args, **kwargs):
-        weight = state_dict.get(prefix + "weight")
-        if weight is not None:
-            full = self._is_full_weight_matrix(weight)
-            sharded = self._is_sharded_weight_matrix(weight)
-            assert full or sharded, "This is neither a full checkpoint nor a sharded checkpoint"
-            if full:
-                weight = extract_local_params_from_full_params(
-                    weight, self._column_group, self._row_group, self.depth_group
-                )
-            state_dict[prefix + "weight"] = weight
-        self._old_load_from_state_dict(state_dict, prefix, *args, **kwargs)
+    def _shard_incoming_weight(self, state_dict, prefix, *unused):
+        key = prefix + "weight"
+        incoming = state_dict.get(key)
+        if incoming is None:
+            return
+        shard_len = self.local_in_features * self.local_out_features // self.depth_group_size
+        if incoming.dim() == 2 and tuple(incoming.shape) == (self.in_features, self.out_features):
+            state_dict[key] = _flat_shard(incoming, self._column_group, self._row_group, self.depth_group)
+        else:
+            assert incoming.dim() == 1 and incoming.numel() == shard_len, \
+                "This is neither a full checkpoint nor a sharded checkpoint"

@@ -30,37 +30,22 @@ from . import overlap_communication
 from .communication import Drop, Gather, _gather, _reduce_scatter
 
 
-def divide(a, b):
-    assert a % b == 0
-    return a // b
+def _flat_shard(full, outer_group, inner_group, depth_group):
+    """This rank's part of a full [out_features, in_features] matrix as the flat vector
+    the parameter holds: input columns of `inner_group`'s slice, output rows of
+    `outer_group`'s, row-major, and of that vector the slice of `depth_group`
+    (axonn/intra_layer/fully_connected.py:62-70 fixes this order; it is the checkpoint
+    format).  On one GPU: the matrix, flattened."""
+    with torch.no_grad():
+        part = Drop.apply(full, inner_group)
+        part = Drop.apply(part.t().contiguous(), outer_group).t().contiguous()
+        return Drop.apply(part.reshape(-1), depth_group)
 
 
-@torch.no_grad()
-def extract_local_params_from_full_params(params, out_features_group, in_features_group,
-                                          depth_group):
-    params = Drop.apply(params, in_features_group)
-    params = Drop.apply(torch.t(params).contiguous(), out_features_group)
-    params = torch.t(params).contiguous()
-    params = Drop.apply(params.reshape(-1), depth_group)  # 1-D view
-    return params
-
-
-@torch.no_grad()
-def initialize_params(out_features, in_features, out_features_group, in_features_group,
-                      depth_group, init_method, init_device=None):
-    if init_device is None:
-        init_device = "cuda" if torch.cuda.is_available() else "cpu"
-    params = torch.empty((out_features, in_features), device=init_device)
-    init_method(params)
-    params = extract_local_params_from_full_params(
-        params, out_features_group, in_features_group, depth_group
-    ).cpu()
-    return params
-
-
-@torch.no_grad()
 def default_init_method(weight):
-    return torch.nn.init.kaiming_uniform_(weight, a=math.sqrt(5))
+    """torch.nn.Linear's own default, U(-1/sqrt(in), 1/sqrt(in)) (:91-93)."""
+    with torch.no_grad():
+        return torch.nn.init.kaiming_uniform_(weight, a=math.sqrt(5))
 
 
 def _compute_dtype(*tensors):
@@ -184,6 +169,9 @@ class FusedLinear(Function):
 
 
 class Linear(torch.nn.Module):
+    """The reference's Linear (:190-301): `weight` is the flat shard of the row-major
+    [out_features, in_features] matrix, `bias` this rank's output rows."""
+
     def __init__(
         self,
         in_features,
@@ -201,119 +189,78 @@ class Linear(torch.nn.Module):
         """Arguments as the reference's Linear (:191-203).  `fused_activation`
         (None or "gelu") is new: the exact-erf GELU applied in the forward
         kernel's epilogue, equal to `torch.nn.GELU()(layer(x))`."""
-        super(Linear, self).__init__()
-        handle = ax._handle()
-        self.inner_group, self.outer_group, self.depth_group = handle.get_intra_layer_groups(
-            tensor_parallel_dims
-        )
-        if transpose:
-            self.inner_group, self.outer_group = self.outer_group, self.inner_group
-        self.depth_group = handle.depth_intra_layer_parallel_group
-
-        self.inner_group_size = get_world_size(self.inner_group)
-        self.outer_group_size = get_world_size(self.outer_group)
-        self.depth_group_size = get_world_size(self.depth_group)
-
-        self.in_features = in_features
-        self.out_features = out_features
-        self.expert_mode = expert_mode
+        super().__init__()
         if fused_activation not in (None, "gelu"):
             raise ValueError("fused_activation must be None or 'gelu', got %r" % (fused_activation,))
-        self.fused_activation = fused_activation
-
-        if init_method is None:
-            init_method = default_init_method
-
+        handle = ax._handle()
+        inner, outer, _ = handle.get_intra_layer_groups(tensor_parallel_dims)
+        # input columns are split over the inner group and output rows over the outer one;
+        # `transpose` swaps the roles (:218-219)
+        self.inner_group, self.outer_group = (outer, inner) if transpose else (inner, outer)
+        self.depth_group = handle.depth_intra_layer_parallel_group
+        self.inner_group_size, self.outer_group_size, self.depth_group_size = (
+            get_world_size(g) for g in (self.inner_group, self.outer_group, self.depth_group))
         assert in_features % self.inner_group_size == 0
         assert out_features % self.outer_group_size == 0
-        self.local_in_features = divide(in_features, self.inner_group_size)
-        self.local_out_features = divide(out_features, self.outer_group_size)
 
-        initial_params = initialize_params(
-            out_features, in_features, self.outer_group, self.inner_group, self.depth_group,
-            init_method,
-        )
-        self.weight = torch.nn.Parameter(initial_params, requires_grad=True)
-        setattr(self.weight, "is_tensor_parallel", True)
-        setattr(self.weight, "needs_depth_parallel_gradient_sync", False)
-        setattr(self.weight, "process_group_for_norm_reduction", handle.intra_layer_group)
+        self.in_features, self.out_features = in_features, out_features
+        self.local_in_features = in_features // self.inner_group_size
+        self.local_out_features = out_features // self.outer_group_size
+        self.expert_mode, self.skip_bias_add = expert_mode, skip_bias_add
+        self.fused_activation = fused_activation
 
+        # Drawn as the full matrix on the device (as the reference does, :73-88), then cut.
+        device = "cuda" if torch.cuda.is_available() else "cpu"
+        full = torch.empty((out_features, in_features), device=device)
+        (init_method or default_init_method)(full)
+        shard = _flat_shard(full, self.outer_group, self.inner_group, self.depth_group).cpu()
+        self.weight = torch.nn.Parameter(shard)
+        # read by gradient sync and clipping (:268-295)
+        self.weight.is_tensor_parallel = True
+        self.weight.needs_depth_parallel_gradient_sync = False
+        self.weight.process_group_for_norm_reduction = handle.intra_layer_group
+        self.bias = None
         if bias:
             self.bias = torch.nn.Parameter(torch.zeros(self.local_out_features))
-            setattr(self.bias, "is_tensor_parallel", True)
-            setattr(self.bias, "needs_depth_parallel_gradient_sync", True)
-            if not transpose:
-                setattr(self.bias, "process_group_for_norm_reduction",
-                        handle.outer_intra_layer_parallel_group)
-            else:
-                setattr(self.bias, "process_group_for_norm_reduction",
-                        handle.inner_intra_layer_parallel_group)
-        else:
-            self.bias = None
-
-        self.skip_bias_add = skip_bias_add
-        self._old_load_from_state_dict = self._load_from_state_dict
-        self._load_from_state_dict = self._modified_load_from_state_dict
+            self.bias.is_tensor_parallel = True
+            self.bias.needs_depth_parallel_gradient_sync = True
+            self.bias.process_group_for_norm_reduction = (
+                handle.inner_intra_layer_parallel_group if transpose
+                else handle.outer_intra_layer_parallel_group)
+        # full tensors in a checkpoint are cut to this rank's shards on the way in (:350-400)
+        self._register_load_state_dict_pre_hook(self._shard_incoming_state)
 
     def forward(self, x, cache_weights_in_all_gather=False):
-        weight = self.weight
         shape = (self.local_out_features, self.local_in_features)
-        fuse_bias = self.bias is not None and not self.skip_bias_add
-        if fuse_bias or self.fused_activation is not None:
-            bias = self.bias if fuse_bias else None
-            if bias is not None and not self.expert_mode:
-                bias = Gather.apply(bias, self.outer_group)
-            y = FusedLinear.apply(x, weight, bias, shape, self.fused_activation)
-            if self.bias is not None and self.skip_bias_add:
-                return y, self.bias
-            return y
-        y = AsyncLinear.apply(
-            x, weight, self.inner_group, self.outer_group, self.depth_group, shape,
-            cache_weights_in_all_gather,
-        )
+        add_bias = self.bias is not None and not self.skip_bias_add
+        if add_bias or self.fused_activation is not None:
+            # bias and activation ride in the forward kernel's epilogue
+            b = self.bias if add_bias else None
+            if b is not None and not self.expert_mode:
+                b = Gather.apply(b, self.outer_group)
+            y = FusedLinear.apply(x, self.weight, b, shape, self.fused_activation)
+            return (y, self.bias) if (self.bias is not None and self.skip_bias_add) else y
+        y = AsyncLinear.apply(x, self.weight, self.inner_group, self.outer_group, self.depth_group,
+                              shape, cache_weights_in_all_gather)
         if self.bias is None:
             return y
-        bias = self.bias
-        if not self.expert_mode:
-            bias = Gather.apply(bias, self.outer_group)
-        return y, bias  # skip_bias_add
+        # skip_bias_add: the caller adds (or fuses) the bias (:345-346)
+        return y, (self.bias if self.expert_mode else Gather.apply(self.bias, self.outer_group))
 
-    def _is_full_weight_matrix(self, weight):
-        return (
-            weight.ndim == 2
-            and weight.size(0) == self.out_features
-            and weight.size(1) == self.in_features
-        )
-
-    def _is_sharded_weight_matrix(self, weight):
-        return weight.ndim == 1 and weight.size(0) == divide(
-            self.local_out_features * self.local_in_features, self.depth_group_size
-        )
-
-    @torch.no_grad()
-    def _modified_load_from_state_dict(self, state_dict, prefix, *args, **kwargs):
-        weight = state_dict[prefix + "weight"] if prefix + "weight" in state_dict else None
-        if weight is not None:
-            is_full_weight_matrix = self._is_full_weight_matrix(weight)
-            is_sharded_weight_matrix = self._is_sharded_weight_matrix(weight)
-            assert (
-                is_full_weight_matrix or is_sharded_weight_matrix
-            ), "This is neither a full checkpoint nor a sharded checkpoint"
-            if is_full_weight_matrix:
-                weight = extract_local_params_from_full_params(
-                    weight, self.outer_group, self.inner_group, self.depth_group
-                )
-            state_dict[prefix + "weight"] = weight
-
-        if self.bias is not None:
-            bias = state_dict[prefix + "bias"] if prefix + "bias" in state_dict else None
-            if bias is not None:
-                if bias.size(0) == self.out_features:
-                    bias = Drop.apply(bias, self.outer_group)
-                    state_dict[prefix + "bias"] = bias
-                else:
-                    assert (
-                        bias.size(0) == self.local_out_features
-                    ), "This is neither a full checkpoint nor a sharded checkpoint"
-
-        self._old_load_from_state_dict(state_dict, prefix, *args, **kwargs)
+    def _shard_incoming_state(self, state_dict, prefix, *unused):
+        mismatch = "This is neither a full checkpoint nor a sharded checkpoint"
+        w = state_dict.get(prefix + "weight")
+        if w is not None:
+            shard_len = self.local_out_features * self.local_in_features // self.depth_group_size
+            if w.dim() == 2 and tuple(w.shape) == (self.out_features, self.in_features):
+                state_dict[prefix + "weight"] = _flat_shard(w, self.outer_group, self.inner_group,
+                                                            self.depth_group)
+            else:
+                assert w.dim() == 1 and w.numel() == shard_len, mismatch
+        b = state_dict.get(prefix + "bias") if self.bias is not None else None
+        if b is not None:
+            if b.shape[0] == self.out_features:
+                with torch.no_grad():
+                    state_dict[prefix + "bias"] = Drop.apply(b, self.outer_group)
+            else:
+                assert b.shape[0] == self.local_out_features, mismatch
