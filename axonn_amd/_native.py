@@ -145,18 +145,27 @@ def call(name, *args):
     check(getattr(load(), name)(*args))
 
 
-def dtype_code(torch_dtype):
-    import torch
+_DTYPE_CODES = {}
 
-    table = {torch.bfloat16: BF16, torch.float16: F16, torch.float32: F32}
-    if torch_dtype not in table:
+
+def dtype_code(torch_dtype):
+    if not _DTYPE_CODES:
+        import torch
+
+        _DTYPE_CODES.update({torch.bfloat16: BF16, torch.float16: F16, torch.float32: F32})
+    code = _DTYPE_CODES.get(torch_dtype)
+    if code is None:
         raise TypeError("unsupported dtype %s (bf16, fp16 or fp32 expected)" % torch_dtype)
-    return table[torch_dtype]
+    return code
 
 
 def current_stream():
+    """torch's current stream on the current device as a `hipStream_t`."""
     import torch
 
+    raw = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+    if raw is not None:  # the handle itself, without building a Stream object (5-10 us less per call)
+        return ctypes.c_void_p(raw(torch.cuda.current_device()))
     return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
 
 
