@@ -86,3 +86,40 @@ def test_captured_step_replays_like_the_eager_step():
         for k in MUTATED:
             assert torch.equal(live[k], twin[k]), (replay, k)
     assert live["dW"].abs().sum() > 0 and not torch.equal(live["P"], before_capture["P"])
+
+
+@pytest.mark.parametrize("M,N,K", [(512, 512, 512), (4096, 2304, 256), (256, 1024, 4096)])
+def test_captured_tile_kernels_replay_like_eager(M, N, K):
+    """The one-wave-per-SIMD kernels (128 x 128 tiles; 256 x 256 tiles; a forward whose
+    contraction is split over workgroups through a workspace) under capture: they ask
+    for their LDS size with a function attribute at launch time, which must not disturb
+    a capture, and every replay equals the eager launch bit for bit."""
+    from axonn_amd import ops
+
+    g = torch.Generator(device="cuda").manual_seed(M + N + K)
+    X = torch.randn(M, K, device="cuda", generator=g).bfloat16()
+    W = (torch.randn(N, K, device="cuda", generator=g) * 0.05).bfloat16()
+    dY = (torch.randn(M, N, device="cuda", generator=g) * 0.01).bfloat16()
+
+    def work():
+        y, _ = ops.gemm_fwd(X, W)
+        return y, ops.gemm_dgrad(dY, W), ops.gemm_wgrad(dY, X, out_dtype=torch.float32)
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        work()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        outs = work()
+    for replay in range(3):
+        X.copy_(torch.randn(M, K, device="cuda", generator=g).bfloat16())
+        dY.copy_((torch.randn(M, N, device="cuda", generator=g) * 0.01).bfloat16())
+        want = work()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for got, exp, name in zip(outs, want, ("y", "dx", "dw")):
+            assert torch.equal(got, exp), (replay, name)
