@@ -225,9 +225,6 @@ def main():
                    "value": round(total_flops / lib_elapsed / 1e12, 2), "unit": "TFLOP/s",
                    "ms_per_step": round(lib_elapsed * 1e3, 4),
                    "ours_over_library": round(value / (total_flops / lib_elapsed / 1e12), 4)}
-    del layers
-    torch.cuda.empty_cache()
-
     def time_loop(fn, n, w=3):
         for _ in range(w):
             fn()
@@ -241,6 +238,30 @@ def main():
         return s.elapsed_time(e) / n * 1e-3
 
     shapes = {}
+    if not args.no_extra_shapes:
+        # The same step on fp16 operands (the reference's default autocast type): the same
+        # kernels with v_mfma_f32_16x16x32_f16.
+        half = [(L.X.half(), L.W.half(), L.dY.half(), torch.empty_like(L.Y, dtype=torch.float16),
+                 torch.empty_like(L.dX, dtype=torch.float16), torch.empty_like(L.dW, dtype=torch.float16))
+                for L in layers]
+
+        def fp16_step():
+            for L, (X, W, dY, Y, dX, dW) in zip(layers, half):
+                nv.check(lib.axn_gemm_fwd_f16(X.data_ptr(), W.data_ptr(), None, Y.data_ptr(), None,
+                                              L.M, L.N, L.K, L.K, L.K, L.N, nv.EPI_NONE, stream))
+            for L, (X, W, dY, Y, dX, dW) in zip(reversed(layers), reversed(half)):
+                nv.check(lib.axn_gemm_dgrad_f16(dY.data_ptr(), W.data_ptr(), dX.data_ptr(), L.M, L.N,
+                                                L.K, L.N, L.K, L.K, stream))
+                nv.check(lib.axn_gemm_wgrad_f16(dY.data_ptr(), X.data_ptr(), dW.data_ptr(), L.M, L.N,
+                                                L.K, L.N, L.K, L.K, 0, nv.F16, stream))
+
+        t = time_loop(fp16_step, max(args.steps // 2, 3))
+        shapes["llama_set_fp16"] = {"ms_per_step": round(t * 1e3, 4),
+                                    "tflops": round(total_flops / t / 1e12, 1),
+                                    "frac_mfma": round(total_flops / t / 1e12 / PEAK_BF16_TFLOPS, 4)}
+        del half
+    del layers
+    torch.cuda.empty_cache()
     if not args.no_extra_shapes:
         # 12B-style MLP shard: bias + GELU fused, dW accumulated over 4 micro-batches
         L = Layer("mlp_shard", 8192, 5120, 2560, 10, torch, bias=True)
