@@ -494,3 +494,28 @@ def test_back_to_back_launches_are_bitwise_reproducible(M, N, K):
                 assert float((t.float() - want).norm() / want.norm()) < 3e-3
         for a, b in zip(got, first):
             assert torch.equal(a, b)
+
+
+@pytest.mark.parametrize("M,N,K", [(512, 512, 512), (4096, 2304, 256), (4096, 6144, 256), (2304, 2048, 192)])
+def test_tile_kernels_take_row_strided_operands(M, N, K):
+    """Operands that are column slices of wider buffers (leading dimension twice the row
+    length) on the 128 x 128-, 256 x 256- and 256 x 128-tile kernels and on a cut problem
+    (384 large tiles): the result equals the one from contiguous copies bit for bit."""
+    from axonn_amd import ops
+
+    g = torch.Generator(device="cuda").manual_seed(M + N + K)
+    Xb = torch.randn(M, 2 * K, device="cuda", generator=g).bfloat16()
+    Wb = (torch.randn(N, 2 * K, device="cuda", generator=g) * 0.05).bfloat16()
+    dYb = (torch.randn(M, 2 * N, device="cuda", generator=g) * 0.1).bfloat16()
+    X, W, dY = Xb[:, K:], Wb[:, :K], dYb[:, N:]
+    assert not X.is_contiguous() and X.stride(0) == 2 * K
+    Xc, Wc, dYc = X.contiguous(), W.contiguous(), dY.contiguous()
+    b = torch.randn(N, device="cuda", generator=g)
+    y, z = ops.gemm_fwd(X, W, bias=b, activation="gelu", save_z=True)
+    yc, zc = ops.gemm_fwd(Xc, Wc, bias=b, activation="gelu", save_z=True)
+    assert torch.equal(y, yc) and torch.equal(z, zc)
+    assert torch.equal(ops.gemm_dgrad(dY, W), ops.gemm_dgrad(dYc, Wc))
+    assert torch.equal(ops.gemm_wgrad(dY, X, out_dtype=torch.float32),
+                       ops.gemm_wgrad(dYc, Xc, out_dtype=torch.float32))
+    ref = torch.nn.functional.gelu(Xc.float() @ Wc.float().t() + b)
+    assert rel(np64(y), np64(ref)) < BF16_TOL
