@@ -519,3 +519,34 @@ def test_tile_kernels_take_row_strided_operands(M, N, K):
                        ops.gemm_wgrad(dYc, Xc, out_dtype=torch.float32))
     ref = torch.nn.functional.gelu(Xc.float() @ Wc.float().t() + b)
     assert rel(np64(y), np64(ref)) < BF16_TOL
+
+
+@pytest.mark.parametrize("tm,tn", [(8, 16), (8, 17), (16, 16), (16, 17), (17, 17), (16, 20), (16, 21),
+                                   (12, 24), (20, 20), (16, 33), (5, 13)])
+def test_every_launch_rule_boundary(tm, tn):
+    """Output sizes of tm x tn large tiles around every threshold of the kernel selection:
+    128 tiles (small tile) and 136 (large); 256 (one round); 272 and 320 (a round and a
+    rest of 16 / 64 for the small tile); 289 and 288 (no whole tile rows or columns to
+    cut: small tile throughout); 336 (rest of 80 on 256 x 128 tiles); 400 (rest of 144:
+    not cut); 528 (two rounds and 16); 65 (256 x 128 tiles throughout).  Forward, dgrad
+    and wgrad of each, every element against an fp32 product of the same operands."""
+    from axonn_amd import ops
+
+    M, N, K = 256 * tm, 256 * tn, 64
+    g = torch.Generator(device="cuda").manual_seed(100 * tm + tn)
+    X = torch.randn(M, K, device="cuda", generator=g).bfloat16()
+    W = (torch.randn(N, K, device="cuda", generator=g) * 0.1).bfloat16()
+    y, _ = ops.gemm_fwd(X, W)
+    ref = X.float() @ W.float().t()
+    assert float((y.float() - ref).abs().max()) <= 2e-2 * float(ref.abs().max())
+    # the same tile grids as outputs of dgrad (M x K') and wgrad (N' x K'), contraction 64
+    dY = (torch.randn(M, 64, device="cuda", generator=g) * 0.1).bfloat16()     # [M, N''=64]
+    W2 = (torch.randn(64, N, device="cuda", generator=g) * 0.1).bfloat16()      # [N''=64, K'=N]
+    dx = ops.gemm_dgrad(dY, W2)
+    ref = dY.float() @ W2.float()
+    assert float((dx.float() - ref).abs().max()) <= 2e-2 * float(ref.abs().max())
+    G = (torch.randn(64, M, device="cuda", generator=g) * 0.1).bfloat16()       # [tokens=64, N'=M]
+    A = torch.randn(64, N, device="cuda", generator=g).bfloat16()               # [tokens=64, K'=N]
+    dw = ops.gemm_wgrad(G, A, out_dtype=torch.float32)
+    ref = G.float().t() @ A.float()
+    assert float((dw - ref).abs().max()) <= 1e-4 * float(ref.abs().max())
