@@ -197,6 +197,11 @@ def main():
             "launches_timed": kinds[dom]["launches"],  # those of every EVENT_EVERY-th timed step
             "flops_per_launch": kinds[dom]["tflops"] * 1e12 * kinds[dom]["avg_us"] * 1e-6,
             "traffic": TRAFFIC_BYTES_PER_LAUNCH.get(dom),
+            "traffic_counts": "bytes between the 8 XCD-private L2s and the fabric (FETCH_SIZE + WRITE_SIZE), "
+                              "reads served by the 256 MB memory-side cache included: each L2 pulls its own "
+                              "copy of a shared operand panel, so this bounds HBM bytes from above",
+            "algorithmic_bytes_per_launch": round(sum(2.0 * (L[1] * L[3] + L[2] * L[3] + L[1] * L[2])
+                                                      for L in LLAMA_SET) / len(LLAMA_SET)),
             "per_kernel": {k: {"avg_us": round(v["avg_us"], 1), "tflops": round(v["tflops"], 1),
                                "frac": round(v["tflops"] / PEAK_BF16_TFLOPS, 4)}
                            for k, v in kinds.items()},
