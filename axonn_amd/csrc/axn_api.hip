@@ -311,6 +311,32 @@ int axn_gemm_wgrad_ws(const void* dY, const void* X, void* dW, int dtype, int64_
                  beta, dw_dtype, workspace, workspace_bytes, stream);
 }
 
+int axn_gemm_swiglu_fwd(const void* X, const void* Wg, const void* Wu, void* H, void* gate_save,
+                        void* up_save, int dtype, int64_t M, int64_t N, int64_t K, int64_t ldx,
+                        int64_t ldw, int64_t ldh, void* stream) {
+  const char* name = "axn_gemm_swiglu_fwd";
+  REQUIRE(dtype == AXN_BF16 || dtype == AXN_F16, AXN_EINVAL, "%s: dtype must be bf16 or fp16", name);
+  int rc = check_gemm(name, X, Wg, H, M, N, K, ldx, ldw, ldh, K, K, N);
+  if (rc) return rc;
+  REQUIRE(Wu != nullptr, AXN_EINVAL, "%s: null operand pointer", name);
+  REQUIRE(aligned16(Wu) && aligned16(gate_save) && aligned16(up_save), AXN_EALIGN,
+          "%s: operand pointers must be 16-byte aligned", name);
+  GemmArgs g = {};
+  g.A = (const uint16_t*)X;
+  g.B = (const uint16_t*)Wg;
+  g.B2 = (const uint16_t*)Wu;
+  g.C = H;
+  g.G = (uint16_t*)gate_save;
+  g.U = (uint16_t*)up_save;
+  g.M = (int)M;
+  g.N = (int)N;
+  g.Kc = (int)K;
+  g.lda = ldx;
+  g.ldb = ldw;
+  g.ldc = ldh;
+  return launch_gemm_swiglu(g, dtype == AXN_F16, (hipStream_t)stream);
+}
+
 size_t axn_dgelu_dbias_workspace_bytes(int64_t M, int64_t N) {
   return dgelu_dbias_workspace_bytes(M, N);
 }

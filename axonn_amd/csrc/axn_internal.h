@@ -71,6 +71,12 @@ __device__ __forceinline__ float dgelu_exact(float x) {
   return fmaf(x * 0.39894228040143267794f, g.expo, g.cdf);
 }
 
+// sigmoid(x) = 1 / (1 + exp(-x)); exp overflows to +inf for x < -88 and the
+// reciprocal then gives the correct limit 0.
+__device__ __forceinline__ float sigmoid_f(float x) {
+  return __builtin_amdgcn_rcpf(1.0f + __expf(-x));
+}
+
 // ---- bf16 GEMM ------------------------------------------------------------
 // C[M x N] (+)= A * B over a contraction of length Kc, bf16 operands, fp32
 // accumulate.  Each operand is either "K-major" (stored [rows][Kc], the
@@ -89,6 +95,12 @@ struct GemmArgs {
   // split, which covers k_split contraction elements and writes its fp32 partial
   // product to C + split * M * ldc.  0 or 1: no split.
   int splits, k_split;
+  // Gate/up forward with the SwiGLU in the epilogue (launch_gemm_swiglu): B holds the gate
+  // weights, B2 the up weights (same shape and ldb); C receives silu(gate) * up, G and U
+  // (optional, ld = ldc) the two pre-activations; N counts the columns of C.
+  const uint16_t* B2;
+  uint16_t* G;
+  uint16_t* U;
 };
 
 enum GemmLayout { GEMM_NT = 0, GEMM_NN = 1, GEMM_TN = 2 };
@@ -109,6 +121,10 @@ int launch_gemm_f16(GemmLayout layout, const GemmArgs& args, int epilogue, bool 
 int gemm_splits(GemmLayout layout, const GemmArgs& args);
 int launch_gemm_splitk(GemmLayout layout, const GemmArgs& args, bool half, int out_dtype,
                        int splits, float* ws, hipStream_t stream);
+
+// C = silu(A B^T) * (A B2^T) in one launch (both weight matrices [N][Kc], K-major), for
+// M % 256 == 0, N % 128 == 0, Kc % 64 == 0 and operands below 2 GiB; AXN_ESHAPE otherwise.
+int launch_gemm_swiglu(const GemmArgs& args, bool half, hipStream_t stream);
 
 // ---- fp32 GEMM (full-precision layers) --------------------------------------
 int launch_gemm_f32(GemmLayout layout, const float* A, const float* B, float* C,

@@ -141,12 +141,6 @@ __global__ void __launch_bounds__(256)
   }
 }
 
-// sigmoid(x) = 1 / (1 + exp(-x)); exp overflows to +inf for x < -88 and the
-// reciprocal then gives the correct limit 0.
-__device__ __forceinline__ float sigmoid_f(float x) {
-  return __builtin_amdgcn_rcpf(1.0f + __expf(-x));
-}
-
 template <typename T>
 __global__ void __launch_bounds__(EW_TX* EW_TY)
     swiglu_fwd_kernel(const T* gate, const T* up, T* out, int64_t M, int64_t N, int64_t ld) {

@@ -49,6 +49,9 @@ typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
 constexpr int BK = 64;          // contraction elements per step
 constexpr int NUM_XCD = 8;      // MI355X: 8 accelerator dies, round-robin dispatch
 constexpr int EPI_LD = 68;      // floats per row of the epilogue staging buffer
+// Internal epilogue of the gate/up forward: the tile's B rows are 64 gate rows and 64 up
+// rows per wave, and the output is silu(gate) * up (not part of the public axn_epilogue).
+constexpr int EPI_SWIGLU = 100;
 
 #define LDS_PTR(T, p) ((__attribute__((address_space(3))) T*)(p))
 
@@ -220,6 +223,29 @@ __device__ __forceinline__ void store_row8(float (&v)[8], const GemmArgs& g, int
   }
 }
 
+// Epilogue of the gate/up forward for 8 consecutive columns of one row: both
+// pre-activations are rounded to the 16-bit type (and stored, if asked for: the backward
+// pass reads them), and the output is computed from the rounded values, so that it equals
+// the separate activation kernel applied to the stored pre-activations bit for bit.
+template <bool HALF>
+__device__ __forceinline__ void store_swiglu8(const float (&vg)[8], const float (&vu)[8],
+                                              const GemmArgs& g, int row, int col) {
+  using lp = std::conditional_t<HALF, _Float16, __bf16>;
+  using lpx8 = std::conditional_t<HALF, f16x8, bf16x8>;
+  const int64_t o = (int64_t)row * g.ldc + col;
+  lpx8 gate, up, out;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    gate[e] = (lp)vg[e];
+    up[e] = (lp)vu[e];
+    const float x = (float)gate[e];
+    out[e] = (lp)(x * sigmoid_f(x) * (float)up[e]);
+  }
+  if (g.G != nullptr) *(lpx8*)(g.G + o) = gate;
+  if (g.U != nullptr) *(lpx8*)(g.U + o) = up;
+  *(lpx8*)((uint16_t*)g.C + o) = out;
+}
+
 // Writes a wave's accumulators to C with the fused epilogue.  With the operands
 // swapped, lane l register r of acc[i][j] is the output element
 //   row = l % 32,  col = 8 * (r / 4) + 4 * (l / 32) + r % 4
@@ -346,13 +372,15 @@ struct DeepOperand {
     }
   }
 
-  template <int I>
+  // Copy I of the tile (LDS kilobytes 4 I .. 4 I + 3); it reads the operand IO copy strides
+  // behind copy 0 (IO = I unless the tile's rows are gathered from two places).
+  template <int I, int IO = I>
   __device__ __forceinline__ static void dma_one(__amdgpu_buffer_rsrc_t rsrc, uint32_t voff,
                                                  uint32_t tile_ofs, uint32_t istride,
                                                  char* lds_tile, int wave) {
-    static_assert(I >= 0 && I < DMA_N, "copy index");
+    static_assert(I >= 0 && I < DMA_N && IO >= 0 && IO < DMA_N, "copy index");
     __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, LDS_PTR(void, lds_tile + (NW * I + wave) * 1024),
-                                             16, (int)voff, (int)(tile_ofs + I * istride), 0, 0);
+                                             16, (int)voff, (int)(tile_ofs + IO * istride), 0, 0);
   }
 
   // Per-lane LDS byte offsets (relative to the tile) the fragment reads start from.
@@ -469,6 +497,13 @@ __device__ __forceinline__ void solo_gemm(const GemmArgs& g) {
   static_assert((BM == 256 || BM == 128) && (BN == 256 || BN == 128) && BM >= BN,
                 "tile sizes with a schedule below");
   static_assert(READ_EVERY >= 1 && COPY_EVERY_A >= 1 && COPY_EVERY_B >= 1, "schedule fits a step");
+  // Gate/up forward: the B tile's 256 rows are, per 128-row half (one wave column), 64
+  // rows of the gate weights and the 64 rows of the up weights with the same indices, so
+  // that a lane ends with a gate value in accumulator block j and the up value of the
+  // same output element in block j + 4.  The tile covers 128 output columns.
+  constexpr bool SWIGLU = EPI == EPI_SWIGLU;
+  static_assert(!SWIGLU || (BM == 256 && BN == 256 && A_KMAJOR && B_KMAJOR && !OUT_F32),
+                "the gate/up forward runs on the 256 x 256 tile with contraction-contiguous operands");
 
   extern __shared__ __attribute__((aligned(16))) char lds[];
 
@@ -484,7 +519,7 @@ __device__ __forceinline__ void solo_gemm(const GemmArgs& g) {
   }
   int tm, tn;
   tile_of_workgroup(pid, g.tiles_m, g.tiles_n, tm, tn);
-  const int m0 = tm * BM, n0 = tn * BN;
+  const int m0 = tm * BM, n0 = tn * (SWIGLU ? BN / 2 : BN);
 
   f32x4 acc[FRM][FRN];
 #pragma unroll
@@ -499,6 +534,8 @@ __device__ __forceinline__ void solo_gemm(const GemmArgs& g) {
       __builtin_amdgcn_make_buffer_rsrc((void*)g.A, 0, (int)a_bytes, 0x00020000);
   const __amdgpu_buffer_rsrc_t rb_rsrc =
       __builtin_amdgcn_make_buffer_rsrc((void*)g.B, 0, (int)b_bytes, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rb2_rsrc =
+      __builtin_amdgcn_make_buffer_rsrc((void*)(SWIGLU ? g.B2 : g.B), 0, (int)b_bytes, 0x00020000);
   uint32_t a_is, b_is;
   const uint32_t va = OA::dma_offset(g.lda, m0, wave, lane, a_is);
   const uint32_t vb = OB::dma_offset(g.ldb, n0, wave, lane, b_is);
@@ -522,7 +559,15 @@ __device__ __forceinline__ void solo_gemm(const GemmArgs& g) {
     OA::template dma_one<decltype(c_)::value>(ra_rsrc, va, ka, a_is, lds + wslot, wave);
   };
   auto copy_b = [&](auto c_) {
-    OB::template dma_one<decltype(c_)::value>(rb_rsrc, vb, kb, b_is, lds + wslot, wave);
+    constexpr int I = decltype(c_)::value;
+    if constexpr (SWIGLU) {
+      // copies 4 h + {0, 1} of a half h bring 64 gate rows, 4 h + {2, 3} the 64 up rows
+      // with the same indices: both are rows 64 h + 32 (I % 2) .. of their matrix
+      constexpr int IO = 2 * (I / 4) + I % 2;
+      OB::template dma_one<I, IO>(I % 4 < 2 ? rb_rsrc : rb2_rsrc, vb, kb, b_is, lds + wslot, wave);
+    } else {
+      OB::template dma_one<I>(rb_rsrc, vb, kb, b_is, lds + wslot, wave);
+    }
   };
   auto a_done = [&]() { ka += a_step; wslot = next_slot(wslot); };
   auto b_done = [&]() { kb += b_step; wslot = next_slot(wslot); };
@@ -649,16 +694,32 @@ __device__ __forceinline__ void solo_gemm(const GemmArgs& g) {
   // instruction.
   const int orow = m0 + wm * WTM + (lane & 15);
   const int ocol = n0 + wn * WTN + 8 * (lane >> 4);
-  GemmArgs go = g;  // a split writes its own fp32 partial product
-  if (OUT_F32 && g.splits > 1) go.C = (float*)g.C + (int64_t)split * g.M * g.ldc;
+  if constexpr (SWIGLU) {
+    // blocks 0..3 of a lane's row hold 64 gate columns, blocks 4..7 the up values of the
+    // same columns
+    const int hcol = n0 + wn * (WTN / 2) + 8 * (lane >> 4);
 #pragma unroll
-  for (int i = 0; i < FRM; ++i)
+    for (int i = 0; i < FRM; ++i)
 #pragma unroll
-    for (int t = 0; t < FRN / 2; ++t) {
-      const f32x4 lo = acc[i][2 * t], hi = acc[i][2 * t + 1];
-      float v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-      store_row8<EPI, OUT_F32, HALF>(v, go, orow + 16 * i, ocol + 32 * t);
-    }
+      for (int t = 0; t < FRN / 4; ++t) {
+        const f32x4 gl = acc[i][2 * t], gh = acc[i][2 * t + 1];
+        const f32x4 ul = acc[i][2 * t + FRN / 2], uh = acc[i][2 * t + 1 + FRN / 2];
+        const float vg[8] = {gl[0], gl[1], gl[2], gl[3], gh[0], gh[1], gh[2], gh[3]};
+        const float vu[8] = {ul[0], ul[1], ul[2], ul[3], uh[0], uh[1], uh[2], uh[3]};
+        store_swiglu8<HALF>(vg, vu, g, orow + 16 * i, hcol + 32 * t);
+      }
+  } else {
+    GemmArgs go = g;  // a split writes its own fp32 partial product
+    if (OUT_F32 && g.splits > 1) go.C = (float*)g.C + (int64_t)split * g.M * g.ldc;
+#pragma unroll
+    for (int i = 0; i < FRM; ++i)
+#pragma unroll
+      for (int t = 0; t < FRN / 2; ++t) {
+        const f32x4 lo = acc[i][2 * t], hi = acc[i][2 * t + 1];
+        float v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        store_row8<EPI, OUT_F32, HALF>(v, go, orow + 16 * i, ocol + 32 * t);
+      }
+  }
 }
 
 template <int TILE, bool A_KMAJOR, bool B_KMAJOR, int EPI, bool OUT_F32>
@@ -677,6 +738,15 @@ __global__ void __launch_bounds__(256) gemm_bf16_rest_kernel(const GemmArgs g) {
 template <bool A_KMAJOR, bool B_KMAJOR, int EPI, bool OUT_F32>
 __global__ void __launch_bounds__(256) gemm_f16_rest_kernel(const GemmArgs g) {
   solo_gemm<256, 128, A_KMAJOR, B_KMAJOR, EPI, OUT_F32, true>(g);
+}
+
+// The gate/up forward of a gated MLP: silu(A B^T) * (A B2^T), 256 rows x 128 columns of
+// the output per workgroup (the MFMA work of a 256 x 256 tile).
+__global__ void __launch_bounds__(256) gemm_bf16_swiglu_kernel(const GemmArgs g) {
+  solo_gemm<256, 256, true, true, EPI_SWIGLU, false, false>(g);
+}
+__global__ void __launch_bounds__(256) gemm_f16_swiglu_kernel(const GemmArgs g) {
+  solo_gemm<256, 256, true, true, EPI_SWIGLU, false, true>(g);
 }
 
 // ---------------------------------------------------------------------------
@@ -1010,6 +1080,28 @@ int launch_layout(GemmLayout layout, const GemmArgs& g, int epilogue, bool out_f
   return AXN_EINVAL;
 }
 }  // namespace
+
+int launch_gemm_swiglu(const GemmArgs& in, bool half, hipStream_t stream) {
+  GemmArgs g = in;
+  const int64_t a_span = (int64_t)g.M * g.lda * 2, b_span = (int64_t)g.N * g.ldb * 2;
+  if (g.M % 256 != 0 || g.N % 128 != 0 || g.Kc % 64 != 0 || a_span >= (1LL << 31) ||
+      b_span >= (1LL << 31)) {
+    set_error("gemm_swiglu: needs M %% 256 == 0, N %% 128 == 0, K %% 64 == 0 and operands below "
+              "2 GiB (got M=%d, N=%d, K=%d)", g.M, g.N, g.Kc);
+    return AXN_ESHAPE;
+  }
+  g.tiles_m = g.M / 256;
+  g.tiles_n = g.N / 128;
+  g.splits = 0;
+  constexpr size_t lds = 5 * 256 * 64 * 2;
+  void (*kern)(const GemmArgs) = half ? gemm_f16_swiglu_kernel : gemm_bf16_swiglu_kernel;
+  AXN_HIP_TRY(hipFuncSetAttribute((const void*)kern,
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+  hipLaunchKernelGGL(kern, dim3((unsigned)((long long)g.tiles_m * g.tiles_n)), dim3(256), lds,
+                     stream, g);
+  AXN_HIP_TRY(hipGetLastError());
+  return AXN_OK;
+}
 
 int launch_gemm_bf16(GemmLayout layout, const GemmArgs& g, int epilogue,
                      bool out_f32, hipStream_t stream) {

@@ -8,7 +8,9 @@ forward passes to Hugging Face.  Here
 * the MLP is rebuilt the same way (`modified_mlp_init`, :76-95), and its forward
   `down_proj(act_fn(gate_proj(x)) * up_proj(x))` additionally runs the activation
   and the product as one kernel (`SwiGLU`, axn_swiglu_fwd / axn_swiglu_bwd) when
-  the activation is SiLU;
+  the activation is SiLU - or, for 16-bit layers without bias and whole-tile shapes,
+  both projections and the activation as one launch (`GateUpSwiGLU`,
+  axn_gemm_swiglu_fwd), with the same results bit for bit;
 * the attention projections are swapped after the original constructor has run,
   instead of restating that constructor (:12-73): the constructor's other fields
   changed across transformers releases, the four projections did not.  At a
@@ -20,6 +22,7 @@ from transformers.models.llama.modeling_llama import LlamaAttention, LlamaMLP, A
 
 from axonn_amd import ops
 from axonn_amd.intra_layer import Linear
+from axonn_amd.intra_layer.fully_connected import _compute_dtype, _weight_grad
 
 _original_mlp_forward = None
 
@@ -49,6 +52,57 @@ def swiglu(gate, up):
     return SwiGLU.apply(gate, up)
 
 
+class GateUpSwiGLU(torch.autograd.Function):
+    """silu(x Wg^T) * (x Wu^T): the two projections and the activation in one launch
+    forward; backward is the one-pass SwiGLU backward, two dgrads whose results are
+    added as autograd would add them, and the two wgrads."""
+
+    @staticmethod
+    @torch.amp.custom_fwd(device_type="cuda")
+    def forward(ctx, x, w_gate, w_up, shape):
+        dt = _compute_dtype(x, w_gate.reshape(shape))
+        x2 = x.reshape(-1, x.shape[-1]).to(dt)
+        needs_grad = any(ctx.needs_input_grad[:3])
+        h, gate, up = ops.gemm_swiglu_fwd(x2, w_gate.reshape(shape).to(dt), w_up.reshape(shape).to(dt),
+                                          save=needs_grad)
+        ctx.save_for_backward(x2, w_gate, w_up, gate, up)
+        ctx.shape, ctx.input_shape, ctx.compute_dtype = shape, x.shape, dt
+        return h.reshape(*x.shape[:-1], shape[0])
+
+    @staticmethod
+    @torch.amp.custom_bwd(device_type="cuda")
+    def backward(ctx, grad_out):
+        x2, w_gate, w_up, gate, up = ctx.saved_tensors
+        dt = ctx.compute_dtype
+        d2 = grad_out.reshape(-1, ctx.shape[0]).to(dt)
+        dgate, dup = ops.swiglu_bwd(d2, gate, up)
+        grad_x = grad_wg = grad_wu = None
+        if ctx.needs_input_grad[0]:
+            grad_x = ops.gemm_dgrad(dgate, w_gate.reshape(ctx.shape).to(dt))
+            grad_x += ops.gemm_dgrad(dup, w_up.reshape(ctx.shape).to(dt))
+            grad_x = grad_x.reshape(ctx.input_shape)
+        if ctx.needs_input_grad[1]:
+            grad_wg = _weight_grad(dgate, x2, w_gate)
+        if ctx.needs_input_grad[2]:
+            grad_wu = _weight_grad(dup, x2, w_up)
+        return grad_x, grad_wg, grad_wu, None
+
+
+def _one_launch_gate_up(mlp, x):
+    """The MLP's gate/up pair qualifies for the one-launch forward: SiLU, no biases,
+    plain layers on one rank, 16-bit compute type and whole-tile shapes."""
+    g, u = mlp.gate_proj, mlp.up_proj
+    if not (getattr(mlp, "_axonn_fused_swiglu", False) and x.is_cuda):
+        return False
+    if g.bias is not None or u.bias is not None or g.fused_activation or u.fused_activation:
+        return False
+    dt = torch.get_autocast_dtype("cuda") if torch.is_autocast_enabled("cuda") else g.weight.dtype
+    if not torch.is_autocast_enabled("cuda") and not (x.dtype == g.weight.dtype == u.weight.dtype):
+        return False
+    tokens = x.numel() // max(x.shape[-1], 1)
+    return ops.gemm_swiglu_supported(tokens, g.local_out_features, g.local_in_features, dt)
+
+
 def modified_mlp_init(self, config):
     super(LlamaMLP, self).__init__()
     self.config = config
@@ -64,6 +118,9 @@ def modified_mlp_init(self, config):
 
 
 def modified_mlp_forward(self, x):
+    if _one_launch_gate_up(self, x):
+        shape = (self.gate_proj.local_out_features, self.gate_proj.local_in_features)
+        return self.down_proj(GateUpSwiGLU.apply(x, self.gate_proj.weight, self.up_proj.weight, shape))
     gate, up = self.gate_proj(x), self.up_proj(x)
     if getattr(self, "_axonn_fused_swiglu", False) and gate.is_cuda and gate.dtype == up.dtype \
             and gate.dtype in (torch.bfloat16, torch.float16, torch.float32):

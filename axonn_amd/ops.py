@@ -272,6 +272,40 @@ def swiglu_fwd(gate, up):
     return out
 
 
+def gemm_swiglu_supported(M, N, K, dtype):
+    """Shapes the one-launch gate/up forward takes (see axn_gemm_swiglu_fwd)."""
+    return (dtype in _GEMM16 and M > 0 and M % 256 == 0 and N % 128 == 0 and K % 64 == 0
+            and M * K * 2 < 2 ** 31 and N * K * 2 < 2 ** 31)
+
+
+def gemm_swiglu_fwd(x, w_gate, w_up, save=True):
+    """silu(X Wg^T) * (X Wu^T) in one launch.  x [M,K], w_gate / w_up [N,K], bf16 or
+    fp16.  Returns (h, gate, up); gate and up (the pre-activations, for the backward
+    pass) are None unless `save`.  Callers check `gemm_swiglu_supported` first."""
+    _require_gpu(x, w_gate, w_up)
+    if not (x.dtype == w_gate.dtype == w_up.dtype):
+        raise TypeError("operand dtypes differ: %s, %s, %s" % (x.dtype, w_gate.dtype, w_up.dtype))
+    if x.dtype not in _GEMM16:
+        raise TypeError("gemm_swiglu_fwd takes bf16 or fp16 operands, got %s" % x.dtype)
+    M, K = x.shape
+    N = w_gate.shape[0]
+    if tuple(w_gate.shape) != (N, K) or tuple(w_up.shape) != (N, K):
+        raise ValueError("weights are %s and %s, input has %d features"
+                         % (tuple(w_gate.shape), tuple(w_up.shape), K))
+    x, ldx = _prep_bf16(x)
+    w_gate, ldg = _prep_bf16(w_gate)
+    w_up, ldu = _prep_bf16(w_up)
+    if ldg != ldu:  # one leading dimension for both weights
+        w_gate, w_up = w_gate.contiguous(), w_up.contiguous()
+        ldg = K
+    h = torch.empty((M, N), dtype=x.dtype, device=x.device)
+    gate = torch.empty_like(h) if save else None
+    up = torch.empty_like(h) if save else None
+    nv.call("axn_gemm_swiglu_fwd", nv.ptr(x), nv.ptr(w_gate), nv.ptr(w_up), nv.ptr(h), nv.ptr(gate),
+            nv.ptr(up), nv.dtype_code(x.dtype), M, N, K, ldx, ldg, N, nv.current_stream())
+    return h, gate, up
+
+
 def swiglu_bwd(dout, gate, up):
     """(dgate, dup) for out = silu(gate) * up."""
     _require_gpu(dout, gate, up)

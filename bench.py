@@ -334,11 +334,19 @@ def main():
         dwg, dwu, dwd = torch.empty(I, H, **bf), torch.empty(I, H, **bf), torch.empty(H, I, **bf)
         P = lambda t: t.data_ptr()  # noqa: E731
 
-        def mlp_block_step():
+        def gate_up_three_calls():
             chk = nv.check
             chk(lib.axn_gemm_fwd(P(x), P(wg), None, P(gt), None, Mt, I, H, H, H, I, nv.EPI_NONE, stream))
             chk(lib.axn_gemm_fwd(P(x), P(wu), None, P(up), None, Mt, I, H, H, H, I, nv.EPI_NONE, stream))
             chk(lib.axn_swiglu_fwd(P(gt), P(up), P(act), nv.BF16, Mt, I, I, stream))
+
+        def gate_up_one_launch():
+            nv.check(lib.axn_gemm_swiglu_fwd(P(x), P(wg), P(wu), P(act), P(gt), P(up), nv.BF16, Mt, I, H,
+                                             H, H, I, stream))
+
+        def mlp_block_step():
+            chk = nv.check
+            gate_up_one_launch()
             chk(lib.axn_gemm_fwd(P(act), P(wd), None, P(y), None, Mt, H, I, I, I, H, nv.EPI_NONE, stream))
             chk(lib.axn_gemm_dgrad(P(dy), P(wd), P(dact), Mt, H, I, H, I, I, stream))
             chk(lib.axn_gemm_wgrad(P(dy), P(act), P(dwd), Mt, H, I, H, I, I, 0, nv.BF16, stream))
@@ -354,9 +362,13 @@ def main():
         t_sw = time_loop(lambda: nv.check(lib.axn_swiglu_fwd(P(gt), P(up), P(act), nv.BF16, Mt, I, I, stream)), 10)
         t_swb = time_loop(lambda: nv.check(lib.axn_swiglu_bwd(P(dact), P(gt), P(up), P(dgt), P(dup), nv.BF16,
                                                              Mt, I, I, stream)), 10)
+        t_gu1 = time_loop(gate_up_one_launch, 10)
+        t_gu3 = time_loop(gate_up_three_calls, 10)
         shapes["llama_mlp_block_4096x4096x14336_swiglu"] = {
             "us": round(t * 1e6, 1), "tflops": round(fl / t / 1e12, 1),
             "frac_mfma": round(fl / t / 1e12 / PEAK_BF16_TFLOPS, 4),
+            "gate_up_swiglu_one_launch_us": round(t_gu1 * 1e6, 1),
+            "gate_up_swiglu_three_calls_us": round(t_gu3 * 1e6, 1),
             "swiglu_fwd_gbs": round(6.0 * Mt * I / t_sw / 1e9, 1),
             "swiglu_bwd_gbs": round(10.0 * Mt * I / t_swb / 1e9, 1)}
         del x, wg, wu, wd, dy, gt, up, act, dact, dgt, dup, y, dx1, dx2, dwg, dwu, dwd

@@ -30,7 +30,7 @@
 extern "C" {
 #endif
 
-#define AXN_ABI_VERSION 5
+#define AXN_ABI_VERSION 6
 
 #if defined(__GNUC__)
 #define AXN_API __attribute__((visibility("default")))
@@ -153,6 +153,23 @@ AXN_API int axn_gemm_wgrad_ws(const void* dY, const void* X, void* dW, int dtype
                       int64_t N, int64_t K, int64_t lddy, int64_t ldx, int64_t lddw,
                       int beta, int dw_dtype, void* workspace, size_t workspace_bytes,
                       void* stream);
+
+/* Gate and up projection of a gated MLP with the activation in the epilogue:
+ *   gate = X Wg^T,  up = X Wu^T,  H = silu(gate) * up     (one launch)
+ * for `down_proj(act_fn(gate_proj(x)) * up_proj(x))` of the model the reference patches
+ * (axonn/models/transformers/modify_llama.py:76-95 builds gate_proj, up_proj and
+ * down_proj from its Linear; each projection is one fully_connected.py:118 product).
+ * X [M,K] (ld ldx), Wg and Wu [N,K] (both ld ldw), H [M,N] (ld ldh) of `dtype`
+ * (AXN_BF16 or AXN_F16); gate_save / up_save (optional, [M,N], ld ldh) receive the two
+ * pre-activations rounded to `dtype`, which is what the backward pass (axn_swiglu_bwd)
+ * reads.  H is computed from the rounded pre-activations: the result equals
+ * axn_gemm_fwd twice followed by axn_swiglu_fwd bit for bit.
+ * Shapes: M % 256 == 0, N % 128 == 0, K % 64 == 0, every operand below 2 GiB
+ * (AXN_ESHAPE otherwise: use the three separate calls); pointers 16-byte aligned,
+ * leading dimensions multiples of 8. */
+AXN_API int axn_gemm_swiglu_fwd(const void* X, const void* Wg, const void* Wu, void* H,
+                                void* gate_save, void* up_save, int dtype, int64_t M, int64_t N,
+                                int64_t K, int64_t ldx, int64_t ldw, int64_t ldh, void* stream);
 
 /* SwiGLU activation of the Llama MLP, one pass over [M,N]:
  *   out = silu(gate) * up,  silu(x) = x / (1 + exp(-x)).

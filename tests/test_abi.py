@@ -118,6 +118,20 @@ def test_swiglu_argument_errors():
     assert "axn_swiglu_bwd" in _err()
 
 
+def test_gate_up_forward_argument_errors():
+    f = nv.load().axn_gemm_swiglu_fwd
+    ok = (nv.BF16, 256, 128, 64, 64, 64, 128, None)
+    assert f(A, A, None, A, A, A, *ok) == nv.AXN_EINVAL                  # no up weights
+    assert f(None, A, A, A, A, A, *ok) == nv.AXN_EINVAL
+    assert f(A, A, A, A, A, A, nv.F32, *ok[1:]) == nv.AXN_EINVAL         # 16-bit types only
+    assert "bf16 or fp16" in _err()
+    assert f(A, A, A, A, ctypes.c_void_p(0x1008), A, *ok) == nv.AXN_EALIGN
+    assert f(A, A, A, A, None, None, nv.BF16, 256, 132, 64, 64, 64, 136, None) == nv.AXN_ESHAPE  # N % 8
+    # a valid GEMM shape that is not made of whole tiles is refused before any launch
+    assert f(A, A, A, A, None, None, nv.BF16, 128, 128, 64, 64, 64, 128, None) == nv.AXN_ESHAPE
+    assert "M % 256 == 0" in _err()
+
+
 def test_embedding_argument_errors():
     lib = nv.load()
     f, b, r = lib.axn_embedding_fwd, lib.axn_embedding_bwd, lib.axn_embedding_renorm

@@ -26,11 +26,12 @@ def gemm_asm(tmp_path_factory):
     subprocess.run(cmd, check=True, capture_output=True, timeout=900)
     text = out.read_text()
     kernels = {}
-    for m in re.finditer(r"^(_ZN3axn\S*gemm_(?:bf16|f16)_(?:solo|rest)_kernel\S*):", text, re.M):
+    for m in re.finditer(r"^(_ZN3axn\S*gemm_(?:bf16|f16)_(?:solo|rest|swiglu)_kernel\S*):", text, re.M):
         end = text.index(".end_amdhsa_kernel", m.end())
         kernels[m.group(1)] = text[m.end():end]
-    # 7 layout/epilogue/output variants x 3 tile shapes (256 x 256, 128 x 128, 256 x 128) x 2 element types
-    assert len(kernels) >= 42, sorted(kernels)
+    # 7 layout/epilogue/output variants x 3 tile shapes (256 x 256, 128 x 128, 256 x 128) x 2 element
+    # types, and the gate/up forward of each type
+    assert len(kernels) >= 44, sorted(kernels)
     return kernels
 
 

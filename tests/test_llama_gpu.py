@@ -253,3 +253,91 @@ def test_other_model_families_under_parallelize_match_their_torch_twins(family):
             assert p_o.grad is None, name
             continue
         assert rel(np64(p_o.grad).reshape(-1), np64(p_r.grad).reshape(-1)) < 5e-2, name
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("M,N,K", [(256, 128, 64), (512, 384, 192), (4096, 1792, 256), (2048, 4096, 128),
+                                   (4096, 8192, 64)])
+def test_gate_up_forward_in_one_launch_equals_the_three_calls(M, N, K, dtype):
+    """axn_gemm_swiglu_fwd against axn_gemm_fwd twice + axn_swiglu_fwd: output and both
+    saved pre-activations bit for bit (1, 6, 224, 256 and 1024 workgroups: less than a
+    round, one round, four rounds), with a row-strided input; and against float64."""
+    from axonn_amd import ops
+
+    g = torch.Generator(device="cuda").manual_seed(M + N + K)
+    xb = torch.randn(M, 2 * K, device="cuda", generator=g).to(dtype)
+    x = xb[:, K:]
+    wg = (torch.randn(N, K, device="cuda", generator=g) * 0.2).to(dtype)
+    wu = (torch.randn(N, K, device="cuda", generator=g) * 0.2).to(dtype)
+    assert ops.gemm_swiglu_supported(M, N, K, dtype)
+    h, gate, up = ops.gemm_swiglu_fwd(x, wg, wu)
+    gate_ref, _ = ops.gemm_fwd(x, wg)
+    up_ref, _ = ops.gemm_fwd(x, wu)
+    assert torch.equal(gate, gate_ref) and torch.equal(up, up_ref)
+    assert torch.equal(h, ops.swiglu_fwd(gate_ref, up_ref))
+    h2, none_g, none_u = ops.gemm_swiglu_fwd(x, wg, wu, save=False)
+    assert none_g is None and none_u is None and torch.equal(h2, h)
+    want = om.swiglu_forward(np64(x) @ np64(wg).T, np64(x) @ np64(wu).T)
+    assert rel(np64(h), want) < 1e-2
+
+
+def test_gate_up_forward_rejects_what_it_cannot_run():
+    from axonn_amd import ops
+
+    assert not ops.gemm_swiglu_supported(255, 128, 64, torch.bfloat16)
+    assert not ops.gemm_swiglu_supported(256, 64, 64, torch.bfloat16)
+    assert not ops.gemm_swiglu_supported(256, 128, 32, torch.bfloat16)
+    assert not ops.gemm_swiglu_supported(256, 128, 64, torch.float32)
+    x = torch.zeros(128, 64, device="cuda", dtype=torch.bfloat16)
+    w = torch.zeros(128, 64, device="cuda", dtype=torch.bfloat16)
+    with pytest.raises(nv.AxnError, match="M % 256 == 0") as e:
+        ops.gemm_swiglu_fwd(x, w, w)
+    assert e.value.code == nv.AXN_ESHAPE
+    with pytest.raises(TypeError, match="bf16 or fp16"):
+        ops.gemm_swiglu_fwd(x.float(), w.float(), w.float())
+
+
+def test_mlp_with_one_launch_gate_up_equals_the_separate_path(monkeypatch):
+    """The patched MLP at a whole-tile shape takes the one-launch gate/up forward; with
+    that path switched off it takes three launches.  Output and every gradient agree bit
+    for bit (the backward of both is the same sequence of kernels)."""
+    from transformers import LlamaConfig
+    from transformers.models.llama.modeling_llama import LlamaMLP
+
+    import axonn_amd.axonn as ax
+    from axonn_amd import ops
+    from axonn_amd.models.transformers import modify_llama, parallelize
+
+    ax.init(1, 1, 1, 1)
+    cfg = LlamaConfig(hidden_size=128, intermediate_size=384, num_attention_heads=4, num_key_value_heads=2,
+                      num_hidden_layers=1, vocab_size=32)
+    with parallelize(cfg):
+        mlp = LlamaMLP(cfg)
+    mlp.forward = modify_llama.modified_mlp_forward.__get__(mlp)
+    mlp = mlp.cuda().bfloat16()
+    g = torch.Generator(device="cuda").manual_seed(5)
+    x0 = torch.randn(2, 128, 128, generator=g, device="cuda").bfloat16()     # 256 tokens
+    dy = (torch.randn(2, 128, 128, generator=g, device="cuda") * 0.1).bfloat16()
+
+    def run():
+        for p in mlp.parameters():
+            p.grad = None
+        x = x0.clone().requires_grad_(True)
+        y = mlp(x)
+        y.backward(dy)
+        return [y.detach(), x.grad] + [p.grad.clone() for p in mlp.parameters()]
+
+    calls = []
+    real = ops.gemm_swiglu_fwd
+    monkeypatch.setattr(ops, "gemm_swiglu_fwd", lambda *a, **k: (calls.append(1), real(*a, **k))[1])
+    fused = run()
+    assert calls, "the one-launch path was not taken"
+    monkeypatch.setattr(ops, "gemm_swiglu_supported", lambda *a: False)
+    n = len(calls)
+    separate = run()
+    assert len(calls) == n
+    for a, b in zip(fused, separate):
+        assert torch.equal(a, b)
+    # a 3-token input does not qualify and still works
+    monkeypatch.undo()
+    assert mlp(x0[0, :3]).shape == (3, 128)
