@@ -7,29 +7,35 @@
 // contraction index is contiguous in memory ([rows][Kc]) and "MN-major" when it
 // is strided ([Kc][rows]).  No transposed copy of an operand is ever made.
 //
-// Common to both kernels in this file
+// Common to both kernel families in this file
 //   * fp32 accumulation in registers; a workgroup owns a BM x BN output tile and
 //     walks the contraction through LDS tiles.
 //   * LDS layouts per storage order such that fragment reads are free of bank
 //     conflicts on the 64-bank LDS; MN-major tiles are read with the transposing
 //     ds_read_b64_tr_b16.
-//   * The MFMA is issued with the operands swapped (D^T = B^T A^T) so a lane
-//     ends up with 4 consecutive output columns; the epilogue transposes
-//     through LDS once more so every lane writes 16 contiguous bytes and a row
-//     segment of 128 bytes is written by 8 lanes.
+//   * The MFMA is issued with the operands swapped (D^T = B^T A^T), so that a lane
+//     holds consecutive output columns of a row and writes 16 contiguous bytes.
 //   * Workgroup ids are remapped so that each of the 8 XCDs (private L2 each)
 //     works on a compact block of neighbouring tiles.
 //
-// gemm_bf16_solo_kernel (whole 256 x 256 tiles, contraction % 64 == 0, more than
-// 128 tiles): 4 waves, one per SIMD, 128 x 128 per wave on v_mfma_f32_16x16x32_bf16;
-// operand tiles go global -> LDS directly (buffer loads to LDS, 16 bytes per
-// lane, no registers) into a ring of five 64-deep tiles; each wave pipelines its
-// LDS fragment reads and its share of the copies between its own MFMAs.
+// One-wave-per-SIMD kernels (solo_gemm: gemm_*_solo_kernel at 256 x 256 and 128 x 128
+// tiles, gemm_*_rest_kernel at 256 x 128, gemm_*_swiglu_kernel; shapes made of whole
+// tiles, contraction % 64 == 0, operands below 2 GiB): 4 waves, one per SIMD, each a
+// quarter of the tile on v_mfma_f32_16x16x32_{bf16,f16}; operand tiles go global -> LDS
+// directly (buffer loads to LDS, 16 bytes per lane, no registers) into a ring of five
+// 64-deep tiles; each wave pipelines its share of the copies and its LDS fragment reads
+// between its own MFMAs; a permuted row order of the column operand's fragments leaves
+// a lane with 8 consecutive output columns, stored straight from the accumulators.
+// launch_shape / launch_whole choose the tile and cut a problem whose last round of
+// large tiles would be at most half full into full rounds and a rest; a workspace
+// variant splits the contraction of problems with few tiles over workgroups; the
+// gate/up forward of a gated MLP gathers its column operand from two weight matrices
+// and applies silu(gate) * up in the epilogue.
 //
-// gemm_bf16_kernel (any shape with N % 8 == 0 and K % 8 == 0): 128 x 128 tiles,
-// v_mfma_f32_32x32x16_bf16, operand tiles staged global -> VGPR -> LDS with
-// bounds checks, one barrier per step; used for ragged shapes and for problems
-// too small to fill the chip with 256 x 256 tiles.
+// Register-staged kernel (gemm_*_kernel: any shape with N % 8 == 0 and K % 8 == 0):
+// 128 x 128 tiles, v_mfma_f32_32x32x16, operand tiles staged global -> VGPR -> LDS with
+// bounds checks, one barrier per step, epilogue transposed through LDS; ragged shapes,
+// contractions that are not multiples of 64, operands of 2 GiB and more.
 #include <utility>
 
 #include "axn_internal.h"
