@@ -341,3 +341,24 @@ def test_mlp_with_one_launch_gate_up_equals_the_separate_path(monkeypatch):
     # a 3-token input does not qualify and still works
     monkeypatch.undo()
     assert mlp(x0[0, :3]).shape == (3, 128)
+
+
+def test_gate_up_forward_in_one_launch_at_the_llama_3_8b_shape():
+    """4096 tokens, 4096 -> 14336 (1792 workgroups, seven rounds): output and both saved
+    pre-activations equal the three separate calls bit for bit, and sampled rows equal the
+    float64 oracle."""
+    from axonn_amd import ops
+
+    M, N, K = 4096, 14336, 4096
+    g = torch.Generator(device="cuda").manual_seed(8)
+    x = torch.randn(M, K, device="cuda", generator=g).bfloat16()
+    wg = (torch.randn(N, K, device="cuda", generator=g) * 0.02).bfloat16()
+    wu = (torch.randn(N, K, device="cuda", generator=g) * 0.02).bfloat16()
+    h, gate, up = ops.gemm_swiglu_fwd(x, wg, wu)
+    gate_ref, _ = ops.gemm_fwd(x, wg)
+    up_ref, _ = ops.gemm_fwd(x, wu)
+    assert torch.equal(gate, gate_ref) and torch.equal(up, up_ref)
+    assert torch.equal(h, ops.swiglu_fwd(gate_ref, up_ref))
+    rows = torch.tensor([0, 255, 256, 1777, 4095], device="cuda")
+    want = om.swiglu_forward(np64(x[rows]) @ np64(wg).T, np64(x[rows]) @ np64(wu).T)
+    assert rel(np64(h[rows]), want) < 1e-2
