@@ -337,6 +337,35 @@ int axn_gemm_swiglu_fwd(const void* X, const void* Wg, const void* Wu, void* H, 
   return launch_gemm_swiglu(g, dtype == AXN_F16, (hipStream_t)stream);
 }
 
+int axn_gemm_dgrad_pair(const void* dY1, const void* W1, const void* dY2, const void* W2, void* dX,
+                        int dtype, int64_t M, int64_t N1, int64_t N2, int64_t K, int64_t lddy,
+                        int64_t ldw, int64_t lddx, void* stream) {
+  const char* name = "axn_gemm_dgrad_pair";
+  REQUIRE(dtype == AXN_BF16 || dtype == AXN_F16, AXN_EINVAL, "%s: dtype must be bf16 or fp16", name);
+  REQUIRE(N1 >= 1 && N2 >= 1 && N1 <= 0x7fffffff - N2, AXN_EINVAL, "%s: N1 and N2 must be >= 1", name);
+  int rc = check_gemm(name, dY1, W1, dX, M, N1, K, lddy, ldw, lddx, N1 > N2 ? N1 : N2, K, K);
+  if (rc) return rc;
+  REQUIRE(N2 % 8 == 0, AXN_ESHAPE, "%s: N and K must be multiples of 8 (got N=%lld)", name,
+          (long long)N2);
+  REQUIRE(dY2 != nullptr && W2 != nullptr, AXN_EINVAL, "%s: null operand pointer", name);
+  REQUIRE(aligned16(dY2) && aligned16(W2), AXN_EALIGN, "%s: operand pointers must be 16-byte aligned",
+          name);
+  GemmArgs g = {};
+  g.A = (const uint16_t*)dY1;
+  g.B = (const uint16_t*)W1;
+  g.A2 = (const uint16_t*)dY2;
+  g.B2 = (const uint16_t*)W2;
+  g.C = dX;
+  g.M = (int)M;
+  g.N = (int)K;
+  g.Kc = (int)(N1 + N2);
+  g.k_first = (int)N1;
+  g.lda = lddy;
+  g.ldb = ldw;
+  g.ldc = lddx;
+  return launch_gemm_pair(g, dtype == AXN_F16, (hipStream_t)stream);
+}
+
 size_t axn_dgelu_dbias_workspace_bytes(int64_t M, int64_t N) {
   return dgelu_dbias_workspace_bytes(M, N);
 }

@@ -101,6 +101,11 @@ struct GemmArgs {
   const uint16_t* B2;
   uint16_t* G;
   uint16_t* U;
+  // Two-term product C = A B + A2 B2 in one pass (launch_gemm_pair): the first k_first
+  // elements of the contraction Kc come from (A, B), the others from (A2, B2), which have
+  // the leading dimensions of A and B.
+  const uint16_t* A2;
+  int k_first;
 };
 
 enum GemmLayout { GEMM_NT = 0, GEMM_NN = 1, GEMM_TN = 2 };
@@ -125,6 +130,12 @@ int launch_gemm_splitk(GemmLayout layout, const GemmArgs& args, bool half, int o
 // C = silu(A B^T) * (A B2^T) in one launch (both weight matrices [N][Kc], K-major), for
 // M % 256 == 0, N % 128 == 0, Kc % 64 == 0 and operands below 2 GiB; AXN_ESHAPE otherwise.
 int launch_gemm_swiglu(const GemmArgs& args, bool half, hipStream_t stream);
+
+// C[M x N] = A B + A2 B2, A / A2 K-major [M][k1], [M][k2], B / B2 MN-major [k1][N], [k2][N]
+// (two input-gradient products added in the accumulators): args.Kc = k1 + k2,
+// args.k_first = k1.  Shapes of whole 128 x 128 tiles, k1 % 64 == 0 and >= 128,
+// k2 % 64 == 0 and >= 64, operands below 2 GiB; AXN_ESHAPE otherwise.
+int launch_gemm_pair(const GemmArgs& args, bool half, hipStream_t stream);
 
 // ---- fp32 GEMM (full-precision layers) --------------------------------------
 int launch_gemm_f32(GemmLayout layout, const float* A, const float* B, float* C,

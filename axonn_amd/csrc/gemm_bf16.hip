@@ -58,6 +58,9 @@ constexpr int EPI_LD = 68;      // floats per row of the epilogue staging buffer
 // Internal epilogue of the gate/up forward: the tile's B rows are 64 gate rows and 64 up
 // rows per wave, and the output is silu(gate) * up (not part of the public axn_epilogue).
 constexpr int EPI_SWIGLU = 100;
+// Internal: no epilogue, but the contraction runs through two operand pairs one after the
+// other (C = A B + A2 B2).
+constexpr int EPI_PAIR = 101;
 
 #define LDS_PTR(T, p) ((__attribute__((address_space(3))) T*)(p))
 
@@ -508,6 +511,10 @@ __device__ __forceinline__ void solo_gemm(const GemmArgs& g) {
   // that a lane ends with a gate value in accumulator block j and the up value of the
   // same output element in block j + 4.  The tile covers 128 output columns.
   constexpr bool SWIGLU = EPI == EPI_SWIGLU;
+  // Two-term product: stages 0 .. k_first / 64 - 1 copy from (A, B), the others from
+  // (A2, B2); everything behind the copies is unchanged.
+  constexpr bool PAIR = EPI == EPI_PAIR;
+  static_assert(!PAIR || (A_KMAJOR && !B_KMAJOR), "the two-term product is the dgrad layout");
   static_assert(!SWIGLU || (BM == 256 && BN == 256 && A_KMAJOR && B_KMAJOR && !OUT_F32),
                 "the gate/up forward runs on the 256 x 256 tile with contraction-contiguous operands");
 
@@ -535,13 +542,16 @@ __device__ __forceinline__ void solo_gemm(const GemmArgs& g) {
 
   const int KP = (g.splits > 1 ? g.k_split : g.Kc) / PK;  // stages of this workgroup
   const uint32_t a_bytes = (uint32_t)((int64_t)(A_KMAJOR ? g.M : g.Kc) * g.lda * 2);
-  const uint32_t b_bytes = (uint32_t)((int64_t)(B_KMAJOR ? g.N : g.Kc) * g.ldb * 2);
+  const uint32_t b_bytes = (uint32_t)((int64_t)(B_KMAJOR ? g.N : (PAIR ? g.k_first : g.Kc)) * g.ldb * 2);
   const __amdgpu_buffer_rsrc_t ra_rsrc =
       __builtin_amdgcn_make_buffer_rsrc((void*)g.A, 0, (int)a_bytes, 0x00020000);
   const __amdgpu_buffer_rsrc_t rb_rsrc =
       __builtin_amdgcn_make_buffer_rsrc((void*)g.B, 0, (int)b_bytes, 0x00020000);
   const __amdgpu_buffer_rsrc_t rb2_rsrc =
       __builtin_amdgcn_make_buffer_rsrc((void*)(SWIGLU ? g.B2 : g.B), 0, (int)b_bytes, 0x00020000);
+  // the pair the copies read from (PAIR only: switched once, two stages before the
+  // first stage of the second pair)
+  __amdgpu_buffer_rsrc_t ra_cur = ra_rsrc, rb_cur = rb_rsrc;
   uint32_t a_is, b_is;
   const uint32_t va = OA::dma_offset(g.lda, m0, wave, lane, a_is);
   const uint32_t vb = OB::dma_offset(g.ldb, n0, wave, lane, b_is);
@@ -562,7 +572,10 @@ __device__ __forceinline__ void solo_gemm(const GemmArgs& g) {
 
   auto next_slot = [&](uint32_t s_) { return s_ + SLOT == NSLOT * SLOT ? 0u : s_ + SLOT; };
   auto copy_a = [&](auto c_) {
-    OA::template dma_one<decltype(c_)::value>(ra_rsrc, va, ka, a_is, lds + wslot, wave);
+    if constexpr (PAIR)
+      OA::template dma_one<decltype(c_)::value>(ra_cur, va, ka, a_is, lds + wslot, wave);
+    else
+      OA::template dma_one<decltype(c_)::value>(ra_rsrc, va, ka, a_is, lds + wslot, wave);
   };
   auto copy_b = [&](auto c_) {
     constexpr int I = decltype(c_)::value;
@@ -571,6 +584,8 @@ __device__ __forceinline__ void solo_gemm(const GemmArgs& g) {
       // with the same indices: both are rows 64 h + 32 (I % 2) .. of their matrix
       constexpr int IO = 2 * (I / 4) + I % 2;
       OB::template dma_one<I, IO>(I % 4 < 2 ? rb_rsrc : rb2_rsrc, vb, kb, b_is, lds + wslot, wave);
+    } else if constexpr (PAIR) {
+      OB::template dma_one<I>(rb_cur, vb, kb, b_is, lds + wslot, wave);
     } else {
       OB::template dma_one<I>(rb_rsrc, vb, kb, b_is, lds + wslot, wave);
     }
@@ -683,7 +698,21 @@ __device__ __forceinline__ void solo_gemm(const GemmArgs& g) {
   };
   using T = std::true_type;
   using F = std::false_type;
-  for (int p = 0; p < KP - 2; ++p) stage(T{}, F{});
+  if constexpr (PAIR) {
+    const int kp1 = g.k_first / PK;  // >= 2: the stages copied up front are of the first pair
+    const uint32_t b2_bytes = (uint32_t)((int64_t)(g.Kc - g.k_first) * g.ldb * 2);
+    for (int p = 0; p < KP - 2; ++p) {
+      if (p == kp1 - 2) {  // this stage copies the tiles of stage kp1, the second pair's first
+        ra_cur = __builtin_amdgcn_make_buffer_rsrc((void*)g.A2, 0, (int)a_bytes, 0x00020000);
+        rb_cur = __builtin_amdgcn_make_buffer_rsrc((void*)g.B2, 0, (int)b2_bytes, 0x00020000);
+        ka = 0;
+        kb = 0;
+      }
+      stage(T{}, F{});
+    }
+  } else {
+    for (int p = 0; p < KP - 2; ++p) stage(T{}, F{});
+  }
   if (KP > 1) stage(F{}, F{});
   stage(F{}, T{});
   // The compiler does not know that the statements above are MFMAs: left alone it
@@ -723,7 +752,7 @@ __device__ __forceinline__ void solo_gemm(const GemmArgs& g) {
       for (int t = 0; t < FRN / 2; ++t) {
         const f32x4 lo = acc[i][2 * t], hi = acc[i][2 * t + 1];
         float v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-        store_row8<EPI, OUT_F32, HALF>(v, go, orow + 16 * i, ocol + 32 * t);
+        store_row8<(PAIR ? (int)AXN_EPI_NONE : EPI), OUT_F32, HALF>(v, go, orow + 16 * i, ocol + 32 * t);
       }
   }
 }
@@ -950,8 +979,14 @@ int launch_whole(const GemmArgs& g, hipStream_t stream) {
     return launch_rest<AK, BKM, EPI, OUT_F32, HALF>(g, stream);
   if (small_spans && whole128 && tiles128 < (1LL << 31))
     return launch_solo<128, AK, BKM, EPI, OUT_F32, HALF>(g, stream);
-  if (whole128) return launch_cfg<128, 128, 2, 2, AK, BKM, EPI, OUT_F32, false, HALF>(g, stream);
-  return launch_cfg<128, 128, 2, 2, AK, BKM, EPI, OUT_F32, true, HALF>(g, stream);
+  if constexpr (EPI == EPI_PAIR) {
+    set_error("gemm_pair: needs whole 128 x 128 tiles, contractions that are multiples of 64 and "
+              "operands below 2 GiB (got M=%d, N=%d, K=%d)", g.M, g.N, g.Kc);
+    return AXN_ESHAPE;
+  } else {
+    if (whole128) return launch_cfg<128, 128, 2, 2, AK, BKM, EPI, OUT_F32, false, HALF>(g, stream);
+    return launch_cfg<128, 128, 2, 2, AK, BKM, EPI, OUT_F32, true, HALF>(g, stream);
+  }
 }
 
 // Full rounds and the rest.  A problem of k * 256 + r large tiles with 0 < r <= 128 ends
@@ -976,6 +1011,7 @@ int launch_shape(const GemmArgs& g, hipStream_t stream) {
         g1.N = (int)n1;
         g2.N = g.N - (int)n1;
         g2.B = BKM ? g.B + n1 * g.ldb : g.B + n1;
+        if (g.B2 != nullptr) g2.B2 = BKM ? g.B2 + n1 * g.ldb : g.B2 + n1;
         g2.C = (char*)g.C + n1 * esz;
         if (g.bias != nullptr) g2.bias = g.bias + n1;
         if (g.Z != nullptr) g2.Z = g.Z + n1;
@@ -985,6 +1021,7 @@ int launch_shape(const GemmArgs& g, hipStream_t stream) {
         g1.M = (int)m1;
         g2.M = g.M - (int)m1;
         g2.A = AK ? g.A + m1 * g.lda : g.A + m1;
+        if (g.A2 != nullptr) g2.A2 = AK ? g.A2 + m1 * g.lda : g.A2 + m1;
         g2.C = (char*)g.C + m1 * g.ldc * esz;
         if (g.Z != nullptr) g2.Z = g.Z + m1 * g.ldc;
         cut = true;
@@ -1086,6 +1123,23 @@ int launch_layout(GemmLayout layout, const GemmArgs& g, int epilogue, bool out_f
   return AXN_EINVAL;
 }
 }  // namespace
+
+int launch_gemm_pair(const GemmArgs& g, bool half, hipStream_t stream) {
+  if (g.k_first % 64 != 0 || g.k_first < 128 || (g.Kc - g.k_first) % 64 != 0 || g.Kc - g.k_first < 64 ||
+      g.splits > 1) {
+    set_error("gemm_pair: both contractions must be multiples of 64, the first at least 128 "
+              "(got %d and %d)", g.k_first, g.Kc - g.k_first);
+    return AXN_ESHAPE;
+  }
+  // the operand spans the kernels address with 32 bits, checked on the longer pair
+  const int k_long = g.k_first > g.Kc - g.k_first ? g.k_first : g.Kc - g.k_first;
+  if ((int64_t)k_long * g.ldb * 2 >= (1LL << 31)) {
+    set_error("gemm_pair: operands must stay below 2 GiB");
+    return AXN_ESHAPE;
+  }
+  return half ? launch_shape<true, false, EPI_PAIR, false, true>(g, stream)
+              : launch_shape<true, false, EPI_PAIR, false, false>(g, stream);
+}
 
 int launch_gemm_swiglu(const GemmArgs& in, bool half, hipStream_t stream) {
   GemmArgs g = in;

@@ -54,8 +54,9 @@ def swiglu(gate, up):
 
 class GateUpSwiGLU(torch.autograd.Function):
     """silu(x Wg^T) * (x Wu^T): the two projections and the activation in one launch
-    forward; backward is the one-pass SwiGLU backward, two dgrads whose results are
-    added as autograd would add them, and the two wgrads."""
+    forward; backward is the one-pass SwiGLU backward, the two input-gradient products
+    in one pass (added in the accumulators, where autograd would add two rounded
+    results), and the two wgrads."""
 
     @staticmethod
     @torch.amp.custom_fwd(device_type="cuda")
@@ -78,8 +79,10 @@ class GateUpSwiGLU(torch.autograd.Function):
         dgate, dup = ops.swiglu_bwd(d2, gate, up)
         grad_x = grad_wg = grad_wu = None
         if ctx.needs_input_grad[0]:
-            grad_x = ops.gemm_dgrad(dgate, w_gate.reshape(ctx.shape).to(dt))
-            grad_x += ops.gemm_dgrad(dup, w_up.reshape(ctx.shape).to(dt))
+            # both products through one set of accumulators, rounded once (two products and
+            # an add where the shape does not fit the one-pass kernel)
+            grad_x = ops.gemm_dgrad_pair(dgate, w_gate.reshape(ctx.shape).to(dt),
+                                         dup, w_up.reshape(ctx.shape).to(dt))
             grad_x = grad_x.reshape(ctx.input_shape)
         if ctx.needs_input_grad[1]:
             grad_wg = _weight_grad(dgate, x2, w_gate)

@@ -306,6 +306,48 @@ def gemm_swiglu_fwd(x, w_gate, w_up, save=True):
     return h, gate, up
 
 
+def gemm_dgrad_pair_supported(M, N1, N2, K, dtype):
+    """Shapes the one-pass two-term input gradient takes (see axn_gemm_dgrad_pair)."""
+    return (dtype in _GEMM16 and M > 0 and M % 128 == 0 and K % 128 == 0 and N1 % 64 == 0
+            and N1 >= 128 and N2 % 64 == 0 and N2 >= 64 and M * max(N1, N2) * 2 < 2 ** 31
+            and (N1 + N2) * K * 2 < 2 ** 31)
+
+
+def gemm_dgrad_pair(dy1, w1, dy2, w2):
+    """dX = dY1 W1 + dY2 W2 with one rounding.  dy_i [M,N_i], w_i [N_i,K].  Shapes the
+    one-pass kernel does not take run as two products and an add."""
+    _require_gpu(dy1, w1, dy2, w2)
+    if not (dy1.dtype == w1.dtype == dy2.dtype == w2.dtype):
+        raise TypeError("operand dtypes differ")
+    M, N1 = dy1.shape
+    N2, K = w2.shape
+    if dy2.shape != (M, N2) or w1.shape != (N1, K):
+        raise ValueError("shapes do not fit: %s %s %s %s" % (tuple(dy1.shape), tuple(w1.shape),
+                                                            tuple(dy2.shape), tuple(w2.shape)))
+    if not gemm_dgrad_pair_supported(M, N1, N2, K, dy1.dtype):
+        dx = gemm_dgrad(dy1, w1)
+        dx += gemm_dgrad(dy2, w2)
+        return dx
+    dy1, ld1 = _prep_bf16(dy1)
+    dy2, ld2 = _prep_bf16(dy2)
+    if ld1 != ld2:
+        dy1, dy2 = dy1.contiguous(), dy2.contiguous()
+        if N1 != N2:  # one leading dimension for both: pad the narrower into a common stride
+            dx = gemm_dgrad(dy1, w1)
+            dx += gemm_dgrad(dy2, w2)
+            return dx
+        ld1 = N1
+    w1, lw1 = _prep_bf16(w1)
+    w2, lw2 = _prep_bf16(w2)
+    if lw1 != lw2:
+        w1, w2 = w1.contiguous(), w2.contiguous()
+        lw1 = K
+    dx = torch.empty((M, K), dtype=dy1.dtype, device=dy1.device)
+    nv.call("axn_gemm_dgrad_pair", nv.ptr(dy1), nv.ptr(w1), nv.ptr(dy2), nv.ptr(w2), nv.ptr(dx),
+            nv.dtype_code(dy1.dtype), M, N1, N2, K, ld1, lw1, K, nv.current_stream())
+    return dx
+
+
 def swiglu_bwd(dout, gate, up):
     """(dgate, dup) for out = silu(gate) * up."""
     _require_gpu(dout, gate, up)

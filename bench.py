@@ -351,9 +351,8 @@ def main():
             chk(lib.axn_gemm_dgrad(P(dy), P(wd), P(dact), Mt, H, I, H, I, I, stream))
             chk(lib.axn_gemm_wgrad(P(dy), P(act), P(dwd), Mt, H, I, H, I, I, 0, nv.BF16, stream))
             chk(lib.axn_swiglu_bwd(P(dact), P(gt), P(up), P(dgt), P(dup), nv.BF16, Mt, I, I, stream))
-            chk(lib.axn_gemm_dgrad(P(dgt), P(wg), P(dx1), Mt, I, H, I, H, H, stream))
-            chk(lib.axn_gemm_dgrad(P(dup), P(wu), P(dx2), Mt, I, H, I, H, H, stream))
-            torch.add(dx1, dx2, out=dx1)
+            chk(lib.axn_gemm_dgrad_pair(P(dgt), P(wg), P(dup), P(wu), P(dx1), nv.BF16, Mt, I, I, H, I, H, H,
+                                        stream))
             chk(lib.axn_gemm_wgrad(P(dgt), P(x), P(dwg), Mt, I, H, I, H, H, 0, nv.BF16, stream))
             chk(lib.axn_gemm_wgrad(P(dup), P(x), P(dwu), Mt, I, H, I, H, H, 0, nv.BF16, stream))
 
@@ -362,6 +361,14 @@ def main():
         t_sw = time_loop(lambda: nv.check(lib.axn_swiglu_fwd(P(gt), P(up), P(act), nv.BF16, Mt, I, I, stream)), 10)
         t_swb = time_loop(lambda: nv.check(lib.axn_swiglu_bwd(P(dact), P(gt), P(up), P(dgt), P(dup), nv.BF16,
                                                              Mt, I, I, stream)), 10)
+        def dgrad_two_calls():
+            nv.check(lib.axn_gemm_dgrad(P(dgt), P(wg), P(dx1), Mt, I, H, I, H, H, stream))
+            nv.check(lib.axn_gemm_dgrad(P(dup), P(wu), P(dx2), Mt, I, H, I, H, H, stream))
+            torch.add(dx1, dx2, out=dx1)
+
+        t_dp1 = time_loop(lambda: nv.check(lib.axn_gemm_dgrad_pair(
+            P(dgt), P(wg), P(dup), P(wu), P(dx1), nv.BF16, Mt, I, I, H, I, H, H, stream)), 10)
+        t_dp2 = time_loop(dgrad_two_calls, 10)
         t_gu1 = time_loop(gate_up_one_launch, 10)
         t_gu3 = time_loop(gate_up_three_calls, 10)
         shapes["llama_mlp_block_4096x4096x14336_swiglu"] = {
@@ -369,6 +376,8 @@ def main():
             "frac_mfma": round(fl / t / 1e12 / PEAK_BF16_TFLOPS, 4),
             "gate_up_swiglu_one_launch_us": round(t_gu1 * 1e6, 1),
             "gate_up_swiglu_three_calls_us": round(t_gu3 * 1e6, 1),
+            "gate_up_dgrad_one_pass_us": round(t_dp1 * 1e6, 1),
+            "gate_up_dgrad_two_calls_and_add_us": round(t_dp2 * 1e6, 1),
             "swiglu_fwd_gbs": round(6.0 * Mt * I / t_sw / 1e9, 1),
             "swiglu_bwd_gbs": round(10.0 * Mt * I / t_swb / 1e9, 1)}
         del x, wg, wu, wd, dy, gt, up, act, dact, dgt, dup, y, dx1, dx2, dwg, dwu, dwd

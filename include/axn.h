@@ -30,7 +30,7 @@
 extern "C" {
 #endif
 
-#define AXN_ABI_VERSION 6
+#define AXN_ABI_VERSION 7
 
 #if defined(__GNUC__)
 #define AXN_API __attribute__((visibility("default")))
@@ -170,6 +170,18 @@ AXN_API int axn_gemm_wgrad_ws(const void* dY, const void* X, void* dW, int dtype
 AXN_API int axn_gemm_swiglu_fwd(const void* X, const void* Wg, const void* Wu, void* H,
                                 void* gate_save, void* up_save, int dtype, int64_t M, int64_t N,
                                 int64_t K, int64_t ldx, int64_t ldw, int64_t ldh, void* stream);
+
+/* Input gradient of two layers that read the same input, in one pass:
+ *   dX = dY1 W1 + dY2 W2
+ * (two fully_connected.py:140 products whose results autograd would add, as for the
+ * gate and up projections of the MLP above).  dY1 [M,N1], dY2 [M,N2] (both ld lddy),
+ * W1 [N1,K], W2 [N2,K] (both ld ldw), dX [M,K] (ld lddx) of `dtype` (AXN_BF16 or
+ * AXN_F16).  The sum runs through one set of fp32 accumulators and is rounded once.
+ * Shapes: M % 128 == 0, K % 128 == 0, N1 % 64 == 0 and >= 128, N2 % 64 == 0 and >= 64,
+ * operands below 2 GiB (AXN_ESHAPE otherwise: two axn_gemm_dgrad calls and an add). */
+AXN_API int axn_gemm_dgrad_pair(const void* dY1, const void* W1, const void* dY2, const void* W2,
+                                void* dX, int dtype, int64_t M, int64_t N1, int64_t N2, int64_t K,
+                                int64_t lddy, int64_t ldw, int64_t lddx, void* stream);
 
 /* SwiGLU activation of the Llama MLP, one pass over [M,N]:
  *   out = silu(gate) * up,  silu(x) = x / (1 + exp(-x)).

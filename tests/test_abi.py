@@ -132,6 +132,20 @@ def test_gate_up_forward_argument_errors():
     assert "M % 256 == 0" in _err()
 
 
+def test_dgrad_pair_argument_errors():
+    f = nv.load().axn_gemm_dgrad_pair
+    tail = (128, 128, 128, 128, 128, 128, None)      # N2, K, lddy, ldw, lddx, stream
+    assert f(A, A, None, A, A, nv.BF16, 128, 128, *tail[:-1], None) == nv.AXN_EINVAL   # dY2 missing
+    assert f(A, A, A, A, A, nv.F32, 128, 128, *tail) == nv.AXN_EINVAL
+    assert f(A, A, A, A, A, nv.BF16, 128, 128, 0, 128, 128, 128, 128, None) == nv.AXN_EINVAL  # N2 = 0
+    assert f(A, A, A, A, A, nv.BF16, 128, 128, 12, 128, 128, 128, 128, None) == nv.AXN_ESHAPE  # N2 % 8
+    assert f(A, A, A, A, A, nv.BF16, 128, 256, 128, 128, 128, 128, 128, None) == nv.AXN_EINVAL  # lddy < N1
+    assert f(A, A, ctypes.c_void_p(0x1008), A, A, nv.BF16, 128, 128, *tail) == nv.AXN_EALIGN
+    # valid operands, but the first contraction is shorter than two stages
+    assert f(A, A, A, A, A, nv.BF16, 128, 64, 64, 128, 64, 128, 128, None) == nv.AXN_ESHAPE
+    assert "gemm_pair" in _err()
+
+
 def test_embedding_argument_errors():
     lib = nv.load()
     f, b, r = lib.axn_embedding_fwd, lib.axn_embedding_bwd, lib.axn_embedding_renorm

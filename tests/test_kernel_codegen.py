@@ -30,8 +30,9 @@ def gemm_asm(tmp_path_factory):
         end = text.index(".end_amdhsa_kernel", m.end())
         kernels[m.group(1)] = text[m.end():end]
     # 7 layout/epilogue/output variants x 3 tile shapes (256 x 256, 128 x 128, 256 x 128) x 2 element
-    # types, and the gate/up forward of each type
-    assert len(kernels) >= 44, sorted(kernels)
+    # types (and the two-term input gradient as an eighth variant), and the gate/up forward of
+    # each type
+    assert len(kernels) >= 50, sorted(kernels)
     return kernels
 
 
