@@ -106,6 +106,12 @@ struct GemmArgs {
   // the leading dimensions of A and B.
   const uint16_t* A2;
   int k_first;
+  // Two outputs (launch of one weight gradient for two layers that read the same input):
+  // output rows below m_split go to C, the others to C2 (row - m_split), same ldc and
+  // type.  m_split is a multiple of the tile height, may be <= 0 (all rows in C2) after a
+  // problem has been cut along its rows.  C2 null: one output.
+  void* C2;
+  int m_split;
 };
 
 enum GemmLayout { GEMM_NT = 0, GEMM_NN = 1, GEMM_TN = 2 };
@@ -151,8 +157,10 @@ int launch_dgelu_dbias(const void* dY, const void* Z, void* dZ, int dtype,
 // ---- SwiGLU activation of the Llama MLP and its backward -----------------------
 int launch_swiglu_fwd(const void* gate, const void* up, void* out, int dtype, int64_t M,
                       int64_t N, int64_t ld, hipStream_t stream);
+// ld: row stride of dout, gate and up; ld_out: of dgate and dup
 int launch_swiglu_bwd(const void* dout, const void* gate, const void* up, void* dgate, void* dup,
-                      int dtype, int64_t M, int64_t N, int64_t ld, hipStream_t stream);
+                      int dtype, int64_t M, int64_t N, int64_t ld, int64_t ld_out,
+                      hipStream_t stream);
 
 // ---- embedding table: row gather, dense weight gradient, max_norm -------------------
 size_t embedding_workspace_bytes(int64_t T, int64_t V);

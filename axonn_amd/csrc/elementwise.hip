@@ -165,7 +165,7 @@ __global__ void __launch_bounds__(EW_TX* EW_TY)
 template <typename T>
 __global__ void __launch_bounds__(EW_TX* EW_TY)
     swiglu_bwd_kernel(const T* dout, const T* gate, const T* up, T* dgate, T* dup, int64_t M,
-                      int64_t N, int64_t ld) {
+                      int64_t N, int64_t ld, int64_t ld_out) {
   const int tx = threadIdx.x % EW_TX, ty = threadIdx.x / EW_TX;
   const int64_t col = (int64_t)blockIdx.x * EW_COLS + tx * 8;
   if (col >= N) return;
@@ -183,8 +183,8 @@ __global__ void __launch_bounds__(EW_TX* EW_TY)
       du[e] = d[e] * g[e] * sg;
       dg[e] = d[e] * u[e] * sg * (1.0f + g[e] * (1.0f - sg));
     }
-    store8(dgate + o, dg);
-    store8(dup + o, du);
+    store8(dgate + r * ld_out + col, dg);
+    store8(dup + r * ld_out + col, du);
   }
 }
 
@@ -212,7 +212,8 @@ int launch_swiglu_fwd(const void* gate, const void* up, void* out, int dtype, in
 }
 
 int launch_swiglu_bwd(const void* dout, const void* gate, const void* up, void* dgate, void* dup,
-                      int dtype, int64_t M, int64_t N, int64_t ld, hipStream_t stream) {
+                      int dtype, int64_t M, int64_t N, int64_t ld, int64_t ld_out,
+                      hipStream_t stream) {
   const int64_t bands = (M + EW_BAND - 1) / EW_BAND;
   if (bands > 65535) {
     set_error("swiglu: too many rows (%lld)", (long long)M);
@@ -221,15 +222,15 @@ int launch_swiglu_bwd(const void* dout, const void* gate, const void* up, void* 
   const dim3 grid((unsigned)((N + EW_COLS - 1) / EW_COLS), (unsigned)bands), block(EW_TX * EW_TY);
   if (dtype == AXN_F32)
     hipLaunchKernelGGL(swiglu_bwd_kernel<float>, grid, block, 0, stream, (const float*)dout,
-                       (const float*)gate, (const float*)up, (float*)dgate, (float*)dup, M, N, ld);
+                       (const float*)gate, (const float*)up, (float*)dgate, (float*)dup, M, N, ld, ld_out);
   else if (dtype == AXN_F16)
     hipLaunchKernelGGL(swiglu_bwd_kernel<_Float16>, grid, block, 0, stream, (const _Float16*)dout,
                        (const _Float16*)gate, (const _Float16*)up, (_Float16*)dgate,
-                       (_Float16*)dup, M, N, ld);
+                       (_Float16*)dup, M, N, ld, ld_out);
   else
     hipLaunchKernelGGL(swiglu_bwd_kernel<uint16_t>, grid, block, 0, stream, (const uint16_t*)dout,
                        (const uint16_t*)gate, (const uint16_t*)up, (uint16_t*)dgate,
-                       (uint16_t*)dup, M, N, ld);
+                       (uint16_t*)dup, M, N, ld, ld_out);
   AXN_HIP_TRY(hipGetLastError());
   return AXN_OK;
 }

@@ -348,17 +348,69 @@ def gemm_dgrad_pair(dy1, w1, dy2, w2):
     return dx
 
 
-def swiglu_bwd(dout, gate, up):
-    """(dgate, dup) for out = silu(gate) * up."""
+def swiglu_bwd(dout, gate, up, side_by_side=False):
+    """(dgate, dup) for out = silu(gate) * up.  With side_by_side the two results are the
+    column blocks of one [M, 2N] buffer, returned as a third value (the layout
+    gemm_wgrad_pair reads)."""
     _require_gpu(dout, gate, up)
     dout, gate, up = _swiglu_operands("swiglu_bwd", [dout, gate, up])
     M, N = gate.shape
+    if side_by_side:
+        # 256 bytes between the rows: with a row stride of exactly 2 N elements the
+        # contraction-strided reads of the weight-gradient kernel fall onto few memory
+        # channels (Llama-3-8B shape: 704 us against 653 us with the gap)
+        ld = 2 * N + 128
+        both = torch.empty((M, ld), dtype=gate.dtype, device=gate.device)[:, :2 * N]
+        dgate, dup = both[:, :N], both[:, N:]
+        if M > 0:
+            nv.call("axn_swiglu_bwd_strided", nv.ptr(dout), nv.ptr(gate), nv.ptr(up), nv.ptr(dgate),
+                    nv.ptr(dup), nv.dtype_code(gate.dtype), M, N, N, ld, nv.current_stream())
+        return dgate, dup, both
     dgate, dup = torch.empty_like(gate), torch.empty_like(up)
     if M == 0:
         return dgate, dup
     nv.call("axn_swiglu_bwd", nv.ptr(dout), nv.ptr(gate), nv.ptr(up), nv.ptr(dgate), nv.ptr(dup),
             nv.dtype_code(gate.dtype), M, N, N, nv.current_stream())
     return dgate, dup
+
+
+def gemm_wgrad_pair_supported(M, N1, N2, K, dtype):
+    """Shapes the one-launch weight gradient of two layers takes (see axn_gemm_wgrad_pair)."""
+    return (dtype in _GEMM16 and M > 0 and M % 64 == 0 and N1 % 256 == 0 and N2 % 128 == 0
+            and K % 128 == 0 and M * (N1 + N2) * 2 < 2 ** 31 and M * K * 2 < 2 ** 31)
+
+
+def gemm_wgrad_pair(dy_both, x, n1, out1=None, out2=None, accumulate=False, out_dtype=None):
+    """dW1 = dy_both[:, :n1]^T X and dW2 = dy_both[:, n1:]^T X in one launch (optionally
+    accumulated into out1 / out2).  Callers check `gemm_wgrad_pair_supported` first."""
+    _require_gpu(dy_both, x, out1, out2)
+    if dy_both.dtype != x.dtype or dy_both.dtype not in _GEMM16:
+        raise TypeError("gemm_wgrad_pair takes bf16 or fp16 operands of one type")
+    M, NN = dy_both.shape
+    K = x.shape[1]
+    n2 = NN - n1
+    if (out1 is None) != (out2 is None):
+        raise ValueError("give both outputs or neither")
+    if out1 is not None:
+        if out1.numel() != n1 * K or out2.numel() != n2 * K or not out1.is_contiguous() \
+                or not out2.is_contiguous() or out1.dtype != out2.dtype:
+            raise ValueError("outputs must be contiguous [n1, K] and [n2, K] tensors of one type")
+        out_dtype = out1.dtype
+    elif accumulate:
+        raise ValueError("accumulate=True needs the outputs")
+    if out_dtype is None:
+        out_dtype = dy_both.dtype
+    if out_dtype not in (dy_both.dtype, torch.float32):
+        raise TypeError("dW must be %s or fp32, got %s" % (dy_both.dtype, out_dtype))
+    dy_both, lddy = _prep_bf16(dy_both)
+    x, ldx = _prep_bf16(x)
+    if out1 is None:
+        out1 = torch.empty((n1, K), dtype=out_dtype, device=x.device)
+        out2 = torch.empty((n2, K), dtype=out_dtype, device=x.device)
+    nv.call("axn_gemm_wgrad_pair", nv.ptr(dy_both), nv.ptr(x), nv.ptr(out1), nv.ptr(out2),
+            nv.dtype_code(x.dtype), M, n1, n2, K, lddy, ldx, K, 1 if accumulate else 0,
+            nv.dtype_code(out_dtype), nv.current_stream())
+    return out1, out2
 
 
 # ------------------------------------------------------------- embedding -----

@@ -330,6 +330,8 @@ def main():
         bf = dict(dtype=torch.bfloat16, device="cuda")
         gt, up, act = (torch.empty(Mt, I, **bf) for _ in range(3))
         dact, dgt, dup = (torch.empty(Mt, I, **bf) for _ in range(3))
+        ldb2 = 2 * I + 128   # 256 bytes between the rows (see ops.swiglu_bwd)
+        dboth = torch.empty(Mt, ldb2, **bf)
         y, dx1, dx2 = (torch.empty(Mt, H, **bf) for _ in range(3))
         dwg, dwu, dwd = torch.empty(I, H, **bf), torch.empty(I, H, **bf), torch.empty(H, I, **bf)
         P = lambda t: t.data_ptr()  # noqa: E731
@@ -350,17 +352,24 @@ def main():
             chk(lib.axn_gemm_fwd(P(act), P(wd), None, P(y), None, Mt, H, I, I, I, H, nv.EPI_NONE, stream))
             chk(lib.axn_gemm_dgrad(P(dy), P(wd), P(dact), Mt, H, I, H, I, I, stream))
             chk(lib.axn_gemm_wgrad(P(dy), P(act), P(dwd), Mt, H, I, H, I, I, 0, nv.BF16, stream))
-            chk(lib.axn_swiglu_bwd(P(dact), P(gt), P(up), P(dgt), P(dup), nv.BF16, Mt, I, I, stream))
-            chk(lib.axn_gemm_dgrad_pair(P(dgt), P(wg), P(dup), P(wu), P(dx1), nv.BF16, Mt, I, I, H, I, H, H,
-                                        stream))
-            chk(lib.axn_gemm_wgrad(P(dgt), P(x), P(dwg), Mt, I, H, I, H, H, 0, nv.BF16, stream))
-            chk(lib.axn_gemm_wgrad(P(dup), P(x), P(dwu), Mt, I, H, I, H, H, 0, nv.BF16, stream))
+            # dgate and dup side by side in one [Mt, 2 I] buffer: the layout of the pair kernels
+            chk(lib.axn_swiglu_bwd_strided(P(dact), P(gt), P(up), P(dboth), P(dboth) + 2 * I, nv.BF16, Mt, I,
+                                           I, ldb2, stream))
+            chk(lib.axn_gemm_dgrad_pair(P(dboth), P(wg), P(dboth) + 2 * I, P(wu), P(dx1), nv.BF16, Mt, I, I,
+                                        H, ldb2, H, H, stream))
+            chk(lib.axn_gemm_wgrad_pair(P(dboth), P(x), P(dwg), P(dwu), nv.BF16, Mt, I, I, H, ldb2, H, H, 0,
+                                        nv.BF16, stream))
 
         t = time_loop(mlp_block_step, max(args.steps // 2, 3))
         fl = 18.0 * Mt * H * I
         t_sw = time_loop(lambda: nv.check(lib.axn_swiglu_fwd(P(gt), P(up), P(act), nv.BF16, Mt, I, I, stream)), 10)
         t_swb = time_loop(lambda: nv.check(lib.axn_swiglu_bwd(P(dact), P(gt), P(up), P(dgt), P(dup), nv.BF16,
                                                              Mt, I, I, stream)), 10)
+        # the separate calls read the same values as the pair kernels (operand values set the
+        # power draw, and with it the clock)
+        dgt.copy_(dboth[:, :I])
+        dup.copy_(dboth[:, I:2 * I])
+
         def dgrad_two_calls():
             nv.check(lib.axn_gemm_dgrad(P(dgt), P(wg), P(dx1), Mt, I, H, I, H, H, stream))
             nv.check(lib.axn_gemm_dgrad(P(dup), P(wu), P(dx2), Mt, I, H, I, H, H, stream))
@@ -369,6 +378,14 @@ def main():
         t_dp1 = time_loop(lambda: nv.check(lib.axn_gemm_dgrad_pair(
             P(dgt), P(wg), P(dup), P(wu), P(dx1), nv.BF16, Mt, I, I, H, I, H, H, stream)), 10)
         t_dp2 = time_loop(dgrad_two_calls, 10)
+
+        def wgrad_two_calls():
+            nv.check(lib.axn_gemm_wgrad(P(dgt), P(x), P(dwg), Mt, I, H, I, H, H, 0, nv.BF16, stream))
+            nv.check(lib.axn_gemm_wgrad(P(dup), P(x), P(dwu), Mt, I, H, I, H, H, 0, nv.BF16, stream))
+
+        t_wp1 = time_loop(lambda: nv.check(lib.axn_gemm_wgrad_pair(
+            P(dboth), P(x), P(dwg), P(dwu), nv.BF16, Mt, I, I, H, ldb2, H, H, 0, nv.BF16, stream)), 10)
+        t_wp2 = time_loop(wgrad_two_calls, 10)
         t_gu1 = time_loop(gate_up_one_launch, 10)
         t_gu3 = time_loop(gate_up_three_calls, 10)
         shapes["llama_mlp_block_4096x4096x14336_swiglu"] = {
@@ -378,9 +395,11 @@ def main():
             "gate_up_swiglu_three_calls_us": round(t_gu3 * 1e6, 1),
             "gate_up_dgrad_one_pass_us": round(t_dp1 * 1e6, 1),
             "gate_up_dgrad_two_calls_and_add_us": round(t_dp2 * 1e6, 1),
+            "gate_up_wgrad_one_launch_us": round(t_wp1 * 1e6, 1),
+            "gate_up_wgrad_two_calls_us": round(t_wp2 * 1e6, 1),
             "swiglu_fwd_gbs": round(6.0 * Mt * I / t_sw / 1e9, 1),
             "swiglu_bwd_gbs": round(10.0 * Mt * I / t_swb / 1e9, 1)}
-        del x, wg, wu, wd, dy, gt, up, act, dact, dgt, dup, y, dx1, dx2, dwg, dwu, dwd
+        del x, wg, wu, wd, dy, gt, up, act, dact, dgt, dup, dboth, y, dx1, dx2, dwg, dwu, dwd
         torch.cuda.empty_cache()
 
         # Embedding of the Llama-3 vocabulary at the largest shape of the reference's own
