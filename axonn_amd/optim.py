@@ -130,10 +130,15 @@ class CPUAdam(Optimizer):
             self.exp_avg_sq = torch.zeros(total, dtype=torch.float32, device=device)
             offset = 0
             self._views = []
+            self._params = all_params
+            self._grad_views = []   # flat 1-D views, one per parameter: what the scan walks
             for p in all_params:
                 n = p.numel()
-                p.grad = self.model_grads_fp16[offset:offset + n].view(p.shape)
+                flat_view = self.model_grads_fp16[offset:offset + n]
+                p.grad = flat_view.view(p.shape)
                 self._views.append((offset, n))
+                if n:
+                    self._grad_views.append(flat_view)
                 offset += n
         self._writes_lowp = self._lowp_dtype != torch.float32
 
@@ -159,16 +164,47 @@ class CPUAdam(Optimizer):
         lo, hi = self.group_offsets[group_no], self.group_offsets[group_no + 1]
         return lo, hi
 
+    def _relink_gradients(self):
+        """The step reads the flat gradient buffer; a parameter's `.grad` is a view into
+        it.  Code that rebinds `.grad` (`model.zero_grad()` sets it to None by default, a
+        cast makes a new tensor) breaks that link without an error: backward would then
+        write elsewhere and the step would apply zeros.  A gradient that has moved is
+        copied into its slice and the view is installed again; a missing one is zeroed
+        (a parameter without a gradient takes no step in the reference either,
+        axonn/optim.py:103-105 walks p.grad)."""
+        flat = self.model_grads_fp16
+        base, esz = flat.data_ptr(), flat.element_size()
+        for p, (offset, n) in zip(self._params, self._views):
+            g = p.grad
+            if g is not None and g.data_ptr() == base + offset * esz and g.numel() == n \
+                    and g.dtype == flat.dtype and g.is_contiguous():
+                continue
+            view = flat[offset:offset + n].view(p.shape)
+            if g is None:
+                view.zero_()
+            else:
+                if g.numel() != n:
+                    raise RuntimeError("a parameter's gradient changed its size (%d -> %d elements)"
+                                       % (n, g.numel()))
+                view.copy_(g)
+            p.grad = view
+
     @torch.no_grad()
     def step(self, closure=None):
         assert closure is None, "AxoNN CPUAdam does not support closure yet"
+        self._relink_gradients()
         inv_scale = 1.0 / self.scaler.loss_scale
         grads = self.model_grads_fp16
         max_norm = float(self.max_grad_norm) if self.max_grad_norm else 0.0
         need_scan = self.dynamic_loss_scale or max_norm > 0.0
         scan = None
         if need_scan:
-            scan = ops.mt_scan([grads], inv_scale, max_norm, result=self._scan)
+            # The overflow test is the reference's, per parameter: a tensor's sum, in
+            # the gradient dtype, is inf or nan (axonn/inter_layer.py:447-460 walks the
+            # parameters; the legacy class walks 16 M-element buckets,
+            # axonn/optim.py:158-161).  One sum over the whole flat buffer would trip on
+            # fp16 as soon as all scaled gradients together sum past 65504.
+            scan = ops.mt_scan(self._grad_views, inv_scale, max_norm, result=self._scan)
             self._scan = scan
         t = self.step_count + 1
         for group_no, group in enumerate(self.param_groups):

@@ -425,3 +425,200 @@ def test_cpuadam_parameter_groups_follow_torch_adam():
         assert float((got - want).abs().max() / want.abs().max()) <= P_TOL
     assert torch.equal(a.detach(), opt.model_params_fp32[:3001].bfloat16())
     assert torch.equal(b.detach().reshape(-1), opt.model_params_fp32[3001:].bfloat16())
+
+
+def test_cpuadam_overflow_flag_is_per_parameter_not_per_flat_buffer():
+    """fp16 gradients whose per-parameter sums stay inside the fp16 range while the sum
+    over the whole flat buffer does not: the reference tests each parameter
+    (axonn/inter_layer.py:447-460), so the step must be applied and the loss scale kept."""
+    from axonn_amd.optim import CPUAdam
+
+    params = [torch.nn.Parameter((torch.randn(1000) * 0.02).half().cuda()) for _ in range(8)]
+    opt = CPUAdam(params, lr=1e-3)
+    assert opt.dynamic_loss_scale and opt.loss_scale == 65536.0
+    for p in params:
+        p.grad.fill_(60.0)                   # 1000 x 60 = 60000 per parameter: finite in fp16
+    grads = [p.grad.double().cpu().numpy() for p in params]
+    overflow, _ = oo.unscale_gradients(grads, "f16", 65536.0)
+    assert overflow is False                                     # the reference's flag
+    assert oo.check_nan(np.concatenate(grads), "f16") is True    # a whole-buffer sum would trip
+    p32 = [opt.model_params_fp32[o:o + n].cpu().numpy().copy() for o, n in opt._views]
+    zeros = [np.zeros_like(a) for a in p32]
+    res = oo.mixed_precision_step([g.astype(np.float32) for g in grads], p32, zeros, zeros, 1,
+                                  65536.0, g_dtype="f16", p_dtype="f16")
+    opt.step()
+    assert not opt.last_step_skipped and opt.step_count == 1 and opt.loss_scale == 65536.0
+    got, ref = opt.model_params_fp32.cpu().numpy(), np.concatenate(res["p"])
+    assert np.max(np.abs(got - ref)) / np.max(np.abs(ref)) <= P_TOL
+    # a parameter whose own sum leaves the range does trip the flag, as in the reference
+    params[3].grad.fill_(70.0)               # 70000 > 65504
+    grads = [p.grad.double().cpu().numpy() for p in params]
+    assert oo.unscale_gradients(grads, "f16", 65536.0)[0] is True
+    before = opt.model_params_fp32.clone()
+    opt.step()
+    assert opt.last_step_skipped and opt.step_count == 1 and opt.loss_scale == 32768.0
+    assert torch.equal(opt.model_params_fp32, before)
+
+
+def test_cpuadam_large_fp16_buffer_of_finite_gradients_is_not_skipped():
+    """Twelve parameters of 40000 fp16 gradients with mean 1: every parameter sums to about
+    40000, the flat buffer to about 480000."""
+    from axonn_amd.optim import CPUAdam
+
+    torch.manual_seed(31)
+    params = [torch.nn.Parameter(torch.zeros(40000 + 3 * i, dtype=torch.float16, device="cuda"))
+              for i in range(12)]
+    opt = CPUAdam(params, max_grad_norm=1.0)
+    for p in params:
+        p.grad.copy_((torch.randn(p.numel()) + 1.0).half())
+    grads = [p.grad.double().cpu().numpy() for p in params]
+    assert oo.unscale_gradients(grads, "f16", 65536.0)[0] is False
+    assert abs(float(np.concatenate(grads).sum())) > 4e5
+    opt.step()
+    assert not opt.last_step_skipped and opt.step_count == 1
+    assert opt.scaler.no_overflow_iters == 1 and opt.loss_scale == 65536.0
+    want = float(np.sqrt(sum(((g / 65536.0) ** 2).sum() for g in grads)))
+    assert abs(float(opt.grad_norm()) - want) <= 1e-5 * want
+
+
+def test_cpuadam_survives_rebound_gradients():
+    """`model.zero_grad()` sets gradients to None by default and backward then makes new
+    tensors: the step must still see them (they are copied back into the flat buffer)."""
+    from axonn_amd.inter_layer import LossScaler
+    from axonn_amd.optim import CPUAdam
+
+    torch.manual_seed(32)
+    model = torch.nn.Linear(24, 40).cuda().bfloat16()
+    opt = CPUAdam(model.parameters(), lr=1e-2, loss_scaler=LossScaler(loss_scale=1.0),
+                  dynamic_loss_scale=False)
+    params = list(model.parameters())
+    p32 = [opt.model_params_fp32[o:o + n].cpu().numpy().copy() for o, n in opt._views]
+    m = [np.zeros_like(a) for a in p32]
+    v = [np.zeros_like(a) for a in p32]
+    for step in (1, 2):
+        model.zero_grad()                       # set_to_none=True: the views are gone
+        assert all(p.grad is None for p in params)
+        x = torch.randn(16, 24).bfloat16().cuda()
+        model(x).float().pow(2).mean().backward()
+        grads = [p.grad.float().cpu().numpy().reshape(-1).copy() for p in params]
+        res = oo.mixed_precision_step(grads, p32, m, v, step, 1.0, lr=1e-2)
+        opt.step()
+        p32, m, v = res["p"], res["m"], res["v"]
+        got, ref = opt.model_params_fp32.cpu().numpy(), np.concatenate(p32)
+        assert np.max(np.abs(got - ref)) / np.max(np.abs(ref)) <= P_TOL
+        base = opt.model_grads_fp16.data_ptr()
+        assert all(p.grad.data_ptr() == base + o * 2 for p, (o, n) in zip(params, opt._views))
+    # a parameter that received no gradient takes a zero gradient
+    model.zero_grad()
+    params[0].grad = torch.ones_like(params[0])
+    opt.step()
+    assert torch.count_nonzero(opt.model_grads_fp16[opt._views[1][0]:]) == 0
+
+
+def test_full_size_adam_config():
+    """The optimizer configuration at its full size: 1.3e9 elements in 64 ragged tensors
+    packed back to back, bf16 gradients ~ N(0, 1e-3) x 65536, clip norm 1, steps 1 and 2;
+    then one +inf in tensor 17.  Checked through a sampled oracle (20000 elements, both
+    steps), the exact rounding of the low-precision copy, the norm against a float64 sum,
+    and bit-identity of the whole state on the skip path."""
+    from axonn_amd import ops
+
+    rng = np.random.default_rng(0)
+    frac = rng.random(64)
+    sizes = np.clip((frac / frac.sum() * 1.3e9).astype(np.int64), 100000, 60000000) | 1  # odd: ragged
+    sizes[np.argmax(sizes)] += 1300000000 - int(sizes.sum())
+    sizes = [int(s) for s in sizes]
+    total = sum(sizes)
+    assert total == 1300000000 and min(sizes) >= 100000
+    g = torch.Generator(device="cuda").manual_seed(1)
+    P = torch.empty(total, device="cuda").normal_(0, 0.02, generator=g)
+    G = torch.empty(total, dtype=torch.bfloat16, device="cuda")
+    sumsq = 0.0
+    for lo in range(0, total, 1 << 27):        # slabs: no 5 GB fp32 temporary
+        hi = min(total, lo + (1 << 27))
+        t = torch.empty(hi - lo, device="cuda").normal_(0, 1e-3 * 65536.0, generator=g)
+        G[lo:hi] = t.bfloat16()
+        sumsq += float(((G[lo:hi].double() / 65536.0) ** 2).sum())
+        del t
+    M = torch.zeros(total, device="cuda")
+    V = torch.zeros(total, device="cuda")
+    PL = torch.zeros(total, dtype=torch.bfloat16, device="cuda")
+    idx = torch.from_numpy(np.sort(rng.choice(total, 20000, replace=False))).cuda()
+    # the sample includes the first and last element of every tensor (the ragged heads and tails)
+    edges = np.cumsum([0] + sizes)
+    idx = torch.unique(torch.cat([idx, torch.from_numpy(edges[:-1]).cuda(),
+                                  torch.from_numpy(edges[1:] - 1).cuda()]))
+    p_s, m_s, v_s = P[idx].cpu().numpy(), M[idx].cpu().numpy(), V[idx].cpu().numpy()
+    vs = lambda t: flat_views(t, sizes)
+    want_norm = float(np.sqrt(sumsq))
+    for step in (1, 2):
+        scan = ops.mt_scan(vs(G), 1.0 / 65536.0, 1.0)
+        assert int(scan.found_inf.item()) == 0
+        assert abs(float(scan.total_norm.item()) - want_norm) <= 1e-6 * want_norm
+        coef = float(scan.clip_coef.item())
+        assert abs(coef - 1.0 / (want_norm + 1e-6)) <= 1e-6 * coef
+        ops.mt_adam(vs(G), vs(P), vs(M), vs(V), vs(PL),
+                    ops.adam_hparams(step, 1e-3, 0.9, 0.999, 1e-8, 0.0), 1.0 / 65536.0, scan)
+        gs = ((G[idx].float() / 65536.0).cpu().numpy() * np.float32(coef)).astype(np.float32)
+        p_s, m_s, v_s = oo.adam_update(p_s, gs, m_s, v_s, step)
+        got = P[idx].cpu().numpy()
+        assert np.max(np.abs(got - p_s)) / np.max(np.abs(p_s)) <= P_TOL
+        assert np.allclose(M[idx].cpu().numpy(), m_s, rtol=1e-5, atol=1e-12)
+        assert np.allclose(V[idx].cpu().numpy(), v_s, rtol=1e-5, atol=1e-16)
+        for lo in range(0, total, 1 << 28):
+            hi = min(total, lo + (1 << 28))
+            assert torch.equal(PL[lo:hi], P[lo:hi].bfloat16())
+    # variant B: one +inf in tensor 17 -> flag set, nothing written
+    G[int(edges[17]) + 12345] = float("inf")
+    csum = lambda t: t.view(torch.int32).sum(dtype=torch.int64).item()  # wrap-around checksum of the bits
+    before = [csum(P), csum(M), csum(V), csum(PL.view(torch.int16).view(torch.int32))]
+    Pc = P[: 1 << 24].clone()
+    scan = ops.mt_scan(vs(G), 1.0 / 65536.0, 1.0)
+    ops.mt_adam(vs(G), vs(P), vs(M), vs(V), vs(PL), ops.adam_hparams(3, 1e-3, 0.9, 0.999, 1e-8, 0.0),
+                1.0 / 65536.0, scan)
+    assert int(scan.found_inf.item()) == 1
+    assert [csum(P), csum(M), csum(V), csum(PL.view(torch.int16).view(torch.int32))] == before
+    assert torch.equal(P[: 1 << 24], Pc)
+
+
+@pytest.mark.parametrize("p", [1.0, 3.0, 0.5, 2.5, 0.0, -1.5])
+def test_clip_grad_norm_any_finite_order(p):
+    """Orders other than 2 (gradient_normalization.py:18-34 passes norm_type through):
+    against the oracle and torch.nn.utils.clip_grad_norm_ on ragged fp32 gradients, and on
+    a bf16 / fp32 mix against the float64 closed form."""
+    from axonn_amd.intra_layer import clip_grad_norm_
+    from axonn_amd.intra_layer.gradient_normalization import get_total_norm
+
+    torch.manual_seed(40)
+    ps = [torch.nn.Parameter(torch.randn(n).cuda()) for n in (33, 70001, 12, 4096)]
+    qs = [torch.nn.Parameter(p_.detach().clone()) for p_ in ps]
+    for a, b in zip(ps, qs):
+        a.grad = torch.randn_like(a) * 0.5 + 0.01
+        b.grad = a.grad.clone()
+    grads = [a.grad.double().cpu().numpy() for a in ps]
+    want, clipped = oo.clip_grad_norm_(grads, 0.05, "f32", norm_type=p)
+    assert abs(float(get_total_norm([a.grad for a in ps], p)) - want) <= 2e-5 * abs(want)
+    got = clip_grad_norm_(ps, 0.05, norm_type=p)
+    ref = torch.nn.utils.clip_grad_norm_(qs, 0.05, norm_type=p, foreach=False)
+    assert abs(float(got) - want) <= 2e-5 * abs(want)
+    assert abs(float(got) - float(ref)) <= 2e-5 * abs(float(ref))
+    for a, b, c in zip(ps, qs, clipped):
+        assert torch.allclose(a.grad, b.grad, rtol=3e-5, atol=0)
+        assert np.allclose(a.grad.double().cpu().numpy(), c, rtol=3e-5, atol=0)
+    if p > 0:   # mixed dtypes: one accumulating call per dtype
+        gs = [torch.randn(5000).cuda().bfloat16(), torch.randn(333).cuda(), torch.randn(64).cuda().half()]
+        flat = np.abs(np.concatenate([g.double().cpu().numpy() for g in gs]))
+        w = float(np.sum(flat ** p) ** (1.0 / p))
+        assert abs(float(get_total_norm(gs, p)) - w) <= 2e-5 * w
+
+
+def test_order_zero_counts_gradients_with_a_nonzero_element():
+    from axonn_amd.intra_layer.gradient_normalization import get_total_norm
+
+    gs = [torch.zeros(100).cuda(), torch.zeros(70000).cuda(), torch.zeros(9).cuda()]
+    assert float(get_total_norm(gs, 0.0)) == 0.0
+    gs[1][69999] = -2.0
+    gs[2][0] = 1e-30
+    assert float(get_total_norm(gs, 0.0)) == 2.0
+    want = torch.norm(torch.stack([torch.norm(g, 0.0) for g in gs]), 0.0)
+    assert float(want) == 2.0
