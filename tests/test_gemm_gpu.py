@@ -550,3 +550,94 @@ def test_every_launch_rule_boundary(tm, tn):
     dw = ops.gemm_wgrad(G, A, out_dtype=torch.float32)
     ref = G.float().t() @ A.float()
     assert float((dw - ref).abs().max()) <= 1e-4 * float(ref.abs().max())
+
+
+def test_mlp_shard_config_fused_epilogue_four_micro_batches():
+    """One GPU's shard of the 12B-style MLP exactly as the configuration states it:
+    8192 tokens x 2560 inputs, W shard [5120, 2560] with bias, GELU fused into the forward
+    epilogue, backward through dGELU + dbias, dgrad and a weight gradient accumulated over
+    4 micro-batches (seeds 0..3) - into a bf16 gradient (the parameter's dtype, as the
+    reference accumulates: overlap_communication.py:38-47) and into an fp32 one.  Checked
+    against the oracle on sampled rows / columns of every result, the full column sums of
+    the bias gradient, and the additivity of dW over micro-batches."""
+    from axonn_amd import ops
+
+    M, N, K = 8192, 5120, 2560
+    gw = torch.Generator(device="cuda").manual_seed(100)
+    W = (torch.randn(N, K, generator=gw, device="cuda") * 0.02).bfloat16()
+    b = (torch.randn(N, generator=gw, device="cuda") * 0.1)
+    Wn, bn = np64(W), b.double().cpu().numpy()
+    rs = np.random.default_rng(7)
+    rows = np.sort(rs.choice(M, 40, replace=False))
+    nrows = np.sort(rs.choice(N, 40, replace=False))
+    ti, tn = torch.from_numpy(rows).cuda(), torch.from_numpy(nrows).cuda()
+
+    dw16 = torch.zeros(N, K, dtype=torch.bfloat16, device="cuda")
+    dw32 = torch.zeros(N, K, dtype=torch.float32, device="cuda")
+    db = torch.zeros(N, dtype=torch.float32, device="cuda")
+    dw_rows_ref = np.zeros((len(nrows), K))          # float64 sum over micro-batches
+    dw16_rows_ref = None                             # the reference's bf16 accumulation order
+    db_ref = np.zeros(N)
+    singles = []
+    for mb in range(4):
+        g = torch.Generator(device="cuda").manual_seed(mb)
+        X = torch.randn(M, K, generator=g, device="cuda").bfloat16()
+        dY = (torch.randn(M, N, generator=g, device="cuda") * 1e-3).bfloat16()
+        y, z = ops.gemm_fwd(X, W, bias=b, activation="gelu", save_z=True)
+        dz, _ = ops.dgelu_dbias(dY, z, want_dbias=True, dbias_out=db, accumulate=True)
+        dx = ops.gemm_dgrad(dz, W)
+        ops.gemm_wgrad(dz, X, out=dw16, accumulate=True)
+        ops.gemm_wgrad(dz, X, out=dw32, accumulate=True)
+        # oracle on the sampled token rows
+        yo, zo = ol.linear_forward(np64(X[ti]), Wn.reshape(-1), (N, K), bias=bn, activation="gelu")
+        assert rel(np64(y[ti]), yo) < BF16_TOL and rel(np64(z[ti]), zo) < BF16_TOL
+        # backward from the saved (rounded) pre-activation, as autograd would
+        bw = ol.linear_backward(np64(X[ti]), Wn.reshape(-1), (N, K), np64(dY[ti]), z=np64(z[ti]),
+                                activation="gelu", has_bias=True)
+        assert rel(np64(dz[ti]), bw["dz"]) < BF16_TOL
+        assert rel(np64(dx[ti]), np64(dz[ti]) @ Wn) < BF16_TOL
+        # rows `nrows` of dW need every token: dZ columns from the kernel's (checked) dZ
+        dzc = np64(dz[:, tn])
+        part = dzc.T @ np64(X)
+        dw_rows_ref += part
+        dw16_rows_ref = ol.accumulate(dw16_rows_ref, part, "bf16")
+        # bias gradient: column sums of dZ over all tokens, oracle dGELU on the full matrix
+        dz_full = np64(dY) * ol.dgelu(np64(z))
+        db_ref += dz_full.sum(0)
+        if mb < 2:
+            singles.append(ops.gemm_wgrad(dz, X, out_dtype=torch.float32))
+            if mb == 1:   # additivity: accumulating equals adding the separate gradients
+                two = ops.gemm_wgrad(dz, X, out=singles[0].clone(), accumulate=True)
+                assert rel(np64(two), np64(singles[0]) + np64(singles[1])) < 1e-6
+        del dz_full, dzc
+    assert rel(dw32[tn].cpu().numpy(), dw_rows_ref) < 1e-4
+    assert rel(np64(dw16[tn]), dw_rows_ref) < BF16_TOL
+    # bf16 accumulation rounds after every micro-batch, exactly like the reference's add_
+    assert rel(np64(dw16[tn]), dw16_rows_ref) < 4e-3
+    assert rel(db.cpu().numpy(), db_ref) < 2e-3
+
+
+@pytest.mark.parametrize("name", ["down", "mlp_shard", "skinny"])
+def test_every_block_of_long_contraction_shapes(name):
+    """Element-wise over every 16 x 16 block of the output (the unit a lane group owns) at
+    the down projection's contraction of 14336 and at the shard and skinny shapes: the
+    largest deviation inside each block stays within bf16 rounding of the fp32 product, so
+    a single misplaced fragment cannot hide in a norm."""
+    from axonn_amd import ops
+
+    M, N, K = FULL[name]
+    g = torch.Generator(device="cuda").manual_seed(9)
+    X = torch.randn(M, K, generator=g, device="cuda").bfloat16()
+    W = (torch.randn(N, K, generator=g, device="cuda") * 0.02).bfloat16()
+    dY = (torch.randn(M, N, generator=g, device="cuda") * 1e-3).bfloat16()
+
+    def blocks_ok(got, ref, tol):
+        err = (got.float() - ref).abs()
+        r, c = err.shape
+        bmax = err.reshape(r // 16, 16, c // 16, 16).amax(dim=(1, 3))
+        return float((bmax / ref.abs().max()).max()) <= tol
+
+    assert blocks_ok(ops.gemm_fwd(X, W)[0], X.float() @ W.float().t(), 1e-2)
+    assert blocks_ok(ops.gemm_dgrad(dY, W), dY.float() @ W.float(), 1e-2)
+    assert blocks_ok(ops.gemm_wgrad(dY, X), dY.float().t() @ X.float(), 1e-2)
+    assert blocks_ok(ops.gemm_wgrad(dY, X, out_dtype=torch.float32), dY.float().t() @ X.float(), 1e-4)
