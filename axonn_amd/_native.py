@@ -21,7 +21,7 @@ AXN_ELIMIT = -5
 BF16, F16, F32 = 0, 1, 2
 EPI_NONE, EPI_BIAS, EPI_BIAS_GELU, EPI_GELU = 0, 1, 2, 3
 
-ABI_VERSION = 8
+ABI_VERSION = 9
 
 # Every symbol include/axn.h declares: name -> (restype, argtypes)
 _c = ctypes
@@ -83,9 +83,11 @@ SYMBOLS = {
     "axn_gemm_wgrad_f32": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _int, _vp]),
     "axn_mt_scan_workspace_bytes": (_sz, [_i64, _i64]),
     "axn_mt_scan": (_int, [_pp, _pi64, _i64, _int, _f32, _f32, _int, _vp, _vp, _sz, _vp]),
+    "axn_mt_scan_norm": (_int, [_pp, _pi64, _i64, _int, _f32, _f32, _f32, _int, _vp, _vp, _sz, _vp]),
     "axn_mt_adam": (_int, [_pp, _pp, _pp, _pp, _pp, _pi64, _i64, _int, _int, _f32, _vp,
                            _c.POINTER(AdamHParams), _vp]),
     "axn_mt_scale": (_int, [_pp, _pi64, _i64, _int, _f32, _vp, _int, _vp]),
+    "axn_stream_probe": (_int, [_int, _vp, _vp, _sz, _vp]),
 }
 
 _lib = None

@@ -1,6 +1,7 @@
 // The C ABI of libaxn_gfx950.so (declared in axn.h): argument validation and
 // dispatch only.  Validation runs before any HIP call so that bad arguments are
 // reported the same way on a host without a GPU.
+#include <cmath>
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
@@ -593,25 +594,55 @@ size_t axn_mt_scan_workspace_bytes(int64_t n, int64_t total) {
   return mt_scan_workspace_bytes(n, total);
 }
 
-int axn_mt_scan(const void* const* h_g, const int64_t* h_sizes, int64_t n,
-                int g_dtype, float inv_scale, float max_norm, int accumulate,
-                axn_scan_result* result, void* workspace, size_t workspace_bytes,
-                void* stream) {
-  const char* name = "axn_mt_scan";
+namespace {
+int check_scan_args(const char* name, const void* const* h_g, const int64_t* h_sizes, int64_t n,
+                    int g_dtype, float norm_type, int accumulate, axn_scan_result* result) {
   int rc = check_sizes(name, h_sizes, n);
   if (rc) return rc;
   REQUIRE(known_dtype(g_dtype), AXN_EINVAL, "%s: unknown gradient dtype %d", name, g_dtype);
   REQUIRE(n == 0 || h_g != nullptr, AXN_EINVAL, "%s: null pointer array", name);
   REQUIRE(result != nullptr, AXN_EINVAL, "%s: result is null", name);
   REQUIRE(((uintptr_t)result & 7u) == 0, AXN_EALIGN, "%s: result must be 8-byte aligned", name);
-  REQUIRE(workspace != nullptr || workspace_bytes == 0, AXN_EINVAL, "%s: null workspace", name);
-  REQUIRE(((uintptr_t)workspace & 15u) == 0, AXN_EALIGN,
-          "%s: workspace must be 16-byte aligned", name);
+  REQUIRE(std::isfinite(norm_type), AXN_EINVAL,
+          "%s: the norm's order must be finite (got %g)", name, (double)norm_type);
   rc = check_list(name, h_g, "g", h_sizes, n, g_dtype == AXN_F32 ? 4 : 2);
   if (rc) return rc;
   REQUIRE(accumulate == 0 || accumulate == 1, AXN_EINVAL, "%s: accumulate must be 0 or 1", name);
-  return launch_mt_scan(h_g, h_sizes, n, g_dtype, inv_scale, max_norm, accumulate, result,
-                        workspace, workspace_bytes, (hipStream_t)stream);
+  return AXN_OK;
+}
+}  // namespace
+
+int axn_mt_scan_norm(const void* const* h_g, const int64_t* h_sizes, int64_t n,
+                     int g_dtype, float inv_scale, float max_norm, float norm_type,
+                     int accumulate, axn_scan_result* result, void* workspace,
+                     size_t workspace_bytes, void* stream) {
+  const char* name = "axn_mt_scan";
+  int rc = check_scan_args(name, h_g, h_sizes, n, g_dtype, norm_type, accumulate, result);
+  if (rc) return rc;
+  REQUIRE(workspace != nullptr || workspace_bytes == 0, AXN_EINVAL, "%s: null workspace", name);
+  REQUIRE(((uintptr_t)workspace & 15u) == 0, AXN_EALIGN,
+          "%s: workspace must be 16-byte aligned", name);
+  return launch_mt_scan(h_g, h_sizes, n, g_dtype, inv_scale, max_norm, norm_type, accumulate,
+                        result, workspace, workspace_bytes, (hipStream_t)stream);
+}
+
+int axn_mt_scan(const void* const* h_g, const int64_t* h_sizes, int64_t n,
+                int g_dtype, float inv_scale, float max_norm, int accumulate,
+                axn_scan_result* result, void* workspace, size_t workspace_bytes,
+                void* stream) {
+  return axn_mt_scan_norm(h_g, h_sizes, n, g_dtype, inv_scale, max_norm, 2.0f, accumulate, result,
+                          workspace, workspace_bytes, stream);
+}
+
+int axn_stream_probe(int kind, const void* src, void* dst, size_t bytes, void* stream) {
+  const char* name = "axn_stream_probe";
+  REQUIRE(kind == AXN_PROBE_READ || kind == AXN_PROBE_FILL || kind == AXN_PROBE_COPY, AXN_EINVAL,
+          "%s: unknown kind %d", name, kind);
+  REQUIRE(dst != nullptr, AXN_EINVAL, "%s: dst is null", name);
+  REQUIRE(kind == AXN_PROBE_FILL || src != nullptr, AXN_EINVAL, "%s: src is null", name);
+  REQUIRE(((uintptr_t)src & 15u) == 0 && ((uintptr_t)dst & (kind == AXN_PROBE_READ ? 3u : 15u)) == 0,
+          AXN_EALIGN, "%s: pointers must be 16-byte aligned", name);
+  return launch_stream_probe(kind, src, dst, bytes, (hipStream_t)stream);
 }
 
 int axn_mt_adam(const void* const* h_g, void* const* h_p, void* const* h_m,

@@ -178,8 +178,8 @@ int launch_embedding_renorm(const int64_t* ids, void* W, int dtype, int64_t T, i
 // ---- multi-tensor optimizer ------------------------------------------------
 size_t mt_scan_workspace_bytes(int64_t n, int64_t total);
 int launch_mt_scan(const void* const* h_g, const int64_t* h_sizes, int64_t n,
-                   int g_dtype, float inv_scale, float max_norm, int accumulate,
-                   axn_scan_result* result, void* ws, size_t ws_bytes,
+                   int g_dtype, float inv_scale, float max_norm, float norm_type,
+                   int accumulate, axn_scan_result* result, void* ws, size_t ws_bytes,
                    hipStream_t stream);
 int launch_mt_adam(const void* const* h_g, void* const* h_p, void* const* h_m,
                    void* const* h_v, void* const* h_plow, const int64_t* h_sizes,
@@ -189,5 +189,8 @@ int launch_mt_adam(const void* const* h_g, void* const* h_p, void* const* h_m,
 int launch_mt_scale(void* const* h_g, const int64_t* h_sizes, int64_t n,
                     int g_dtype, float inv_scale, const axn_scan_result* scan,
                     int use_clip, hipStream_t stream);
+
+// Streaming yardsticks (axn_stream_probe).
+int launch_stream_probe(int kind, const void* src, void* dst, size_t bytes, hipStream_t stream);
 
 }  // namespace axn

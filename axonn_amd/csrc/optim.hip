@@ -22,8 +22,8 @@
 // scalar accesses.
 #include "axn_internal.h"
 
+#include <atomic>
 #include <cmath>
-#include <vector>
 
 namespace axn {
 namespace {
@@ -32,7 +32,7 @@ namespace {
 #define AXN_SCAN_CHUNK 65536
 #endif
 #ifndef AXN_ADAM_CHUNK
-#define AXN_ADAM_CHUNK 4096
+#define AXN_ADAM_CHUNK 8192
 #endif
 #ifndef AXN_ADAM_UNROLL
 #define AXN_ADAM_UNROLL 1
@@ -42,6 +42,12 @@ namespace {
 #endif
 #ifndef AXN_ADAM_NT_STORE
 #define AXN_ADAM_NT_STORE 1
+#endif
+#ifndef AXN_ADAM_NT_LOAD
+#define AXN_ADAM_NT_LOAD 0
+#endif
+#ifndef AXN_ADAM_WGS_PER_CU
+#define AXN_ADAM_WGS_PER_CU 4096
 #endif
 
 constexpr int MT_MAX = 64;         // tensors per launch
@@ -217,9 +223,22 @@ __device__ __forceinline__ int wave_or(int x) {
   return x;
 }
 
-template <int DT>
+// |u|^p of the norm's order p, by mode: the 2-norm and the 1-norm have their own
+// instructions, order 0 counts the non-zero elements (torch.norm's meaning of p = 0),
+// any other order goes through exp2(p log2 |u|) (|0|^p is 0 for p > 0 and +inf for p < 0,
+// as in torch).
+enum NormMode { NORM_2 = 0, NORM_1 = 1, NORM_0 = 2, NORM_P = 3 };
+template <int MODE>
+__device__ __forceinline__ float norm_term(float u, float p) {
+  if (MODE == NORM_2) return u * u;
+  if (MODE == NORM_1) return fabsf(u);
+  if (MODE == NORM_0) return u != 0.0f ? 1.0f : 0.0f;
+  return powf(fabsf(u), p);
+}
+
+template <int DT, int MODE>
 __global__ void __launch_bounds__(MT_THREADS)
-    mt_scan_kernel(const MtTable tab, float inv_scale, ScanPartial* partial,
+    mt_scan_kernel(const MtTable tab, float inv_scale, float norm_type, ScanPartial* partial,
                    int block_base) {
   typedef typename Lowp<DT>::raw raw;
   const int t = find_tensor(tab, blockIdx.x);
@@ -234,8 +253,7 @@ __global__ void __launch_bounds__(MT_THREADS)
     bad |= Lowp<DT>::nonfinite(x) ? 1 : 0;
     const float f = Lowp<DT>::to_float(x);
     sm += f;
-    const float u = f * inv_scale;
-    sq += u * u;
+    sq += norm_term<MODE>(f * inv_scale, norm_type);
   };
   if (tab.vec_ok[t]) {
     if (c == 0 && tid < tab.head[t]) one(((const raw*)g)[tid]);
@@ -292,7 +310,7 @@ __device__ __forceinline__ double wave_sum_d(double x) {
 __global__ void __launch_bounds__(1024)
     mt_scan_finalize_kernel(const MtTable tab, const ScanPartial* partial,
                             int block_base, double sum_limit, float max_norm,
-                            int first, axn_scan_result* out) {
+                            float norm_type, int first, axn_scan_result* out) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   __shared__ double s_sq[16];
   __shared__ int s_bad[16];
@@ -312,6 +330,9 @@ __global__ void __launch_bounds__(1024)
     tbad = wave_or(tbad);
     // The tensor's sum, rounded to the gradient dtype, is non-finite.
     if (!(fabs(tsm) < sum_limit)) tbad = 1;
+    // order 0: the norm over the stacked per-tensor norms counts the tensors whose own
+    // count of non-zero elements is not zero
+    if (norm_type == 0.0f) tsq = tsq != 0.0 ? 1.0 : 0.0;
     sq += tsq;
     bad |= tbad;
   }
@@ -327,7 +348,9 @@ __global__ void __launch_bounds__(1024)
       total += s_sq[w];
       flag |= s_bad[w];
     }
-    const float norm = (float)sqrt(total);
+    const float norm = norm_type == 2.0f ? (float)sqrt(total)
+                       : norm_type == 1.0f || norm_type == 0.0f ? (float)total
+                       : (float)pow(total, 1.0 / (double)norm_type);
     float coef = 1.0f;
     if (max_norm > 0.0f) {
       coef = max_norm / (norm + 1e-6f);
@@ -362,10 +385,17 @@ __device__ __forceinline__ void adam_math(float g, float& p, float& m, float& v,
   asm volatile("" : "+v"(p));
 }
 
+// One workgroup per chunk up to a cap of AXN_ADAM_WGS_PER_CU workgroups per CU, beyond
+// which workgroups walk the chunk list with a stride of the grid size.  The cap is far
+// above what the optimizer configurations reach, on purpose: measured on MI355X (1.3e9
+// elements, 64 tensors) a grid of one workgroup per chunk, which the dispatcher hands out
+// in order so that the chip works on one compact window of every stream, updates at
+// 5.23 TB/s; 256 workgroups per CU at 5.18, 64 at 5.08, 4 to 16 at 5.05 - workgroups
+// that stay resident drift apart and the window widens.
 template <int GDT, int PDT, bool HAS_PLOW>
 __global__ void __launch_bounds__(MT_THREADS)
     mt_adam_kernel(const MtTable tab, const AdamScalars s,
-                   const axn_scan_result* scan) {
+                   const axn_scan_result* scan, int total_chunks) {
   typedef typename Lowp<GDT>::raw graw;
   typedef typename Lowp<PDT>::raw praw;
   float gmul = 1.0f;
@@ -373,80 +403,85 @@ __global__ void __launch_bounds__(MT_THREADS)
     if (scan->found_inf != 0) return;  // overflow: the whole step is skipped
     gmul = scan->clip_coef;
   }
-  const int t = find_tensor(tab, blockIdx.x);
-  const int c = blockIdx.x - tab.chunk_start[t];
-  const Range rg = chunk_range(tab, t, c);
-  const void* g = tab.g[t];
-  float* p = (float*)tab.p[t];
-  float* m = (float*)tab.m[t];
-  float* v = (float*)tab.v[t];
-  void* plow = tab.plow[t];
   const int tid = threadIdx.x;
+  int t = find_tensor(tab, blockIdx.x);
+  for (int b = blockIdx.x; b < total_chunks; b += gridDim.x) {
+    while (tab.chunk_start[t + 1] <= b) ++t;  // uniform: chunk ids only grow
+    const int c = b - tab.chunk_start[t];
+    const Range rg = chunk_range(tab, t, c);
+    const void* g = tab.g[t];
+    float* p = (float*)tab.p[t];
+    float* m = (float*)tab.m[t];
+    float* v = (float*)tab.v[t];
+    void* plow = tab.plow[t];
 
-  auto one = [&](int64_t i) {
-    float pp = p[i], mm = m[i], vv = v[i];
-    adam_math(Lowp<GDT>::to_float(((const graw*)g)[i]), pp, mm, vv, s, gmul);
-    p[i] = pp;
-    m[i] = mm;
-    v[i] = vv;
-    if (HAS_PLOW) ((praw*)plow)[i] = Lowp<PDT>::from_float(pp);
-  };
+    auto one = [&](int64_t i) {
+      float pp = p[i], mm = m[i], vv = v[i];
+      adam_math(Lowp<GDT>::to_float(((const graw*)g)[i]), pp, mm, vv, s, gmul);
+      p[i] = pp;
+      m[i] = mm;
+      v[i] = vv;
+      if (HAS_PLOW) ((praw*)plow)[i] = Lowp<PDT>::from_float(pp);
+    };
 
-  if (tab.vec_ok[t]) {
-    if (c == 0 && tid < tab.head[t]) one(tid);
-    const int64_t nvec = (rg.end - rg.begin) / MT_VEC;
-    int64_t i = tid;
-    // Main body: ADAM_UNROLL independent vectors per lane in flight.
-    for (; i + (ADAM_UNROLL - 1) * MT_THREADS < nvec; i += ADAM_UNROLL * MT_THREADS) {
-      graw gr[ADAM_UNROLL][8];
-      float pp[ADAM_UNROLL][8], mm[ADAM_UNROLL][8], vv[ADAM_UNROLL][8];
+    if (tab.vec_ok[t]) {
+      if (c == 0 && tid < tab.head[t]) one(tid);
+      const int64_t nvec = (rg.end - rg.begin) / MT_VEC;
+      int64_t i = tid;
+      // Main body: ADAM_UNROLL independent vectors per lane in flight.
+      for (; i + (ADAM_UNROLL - 1) * MT_THREADS < nvec; i += ADAM_UNROLL * MT_THREADS) {
+        graw gr[ADAM_UNROLL][8];
+        float pp[ADAM_UNROLL][8], mm[ADAM_UNROLL][8], vv[ADAM_UNROLL][8];
 #pragma unroll
-      for (int u = 0; u < ADAM_UNROLL; ++u) {
-        const int64_t e0 = rg.begin + (i + u * MT_THREADS) * MT_VEC;
-        load8<GDT, AXN_ADAM_NT_G != 0>(g, e0, gr[u]);
-        loadf8<false>(p + e0, pp[u]);
-        loadf8<false>(m + e0, mm[u]);
-        loadf8<false>(v + e0, vv[u]);
-      }
-#pragma unroll
-      for (int u = 0; u < ADAM_UNROLL; ++u) {
-        const int64_t e0 = rg.begin + (i + u * MT_THREADS) * MT_VEC;
-        praw pl[8];
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          adam_math(Lowp<GDT>::to_float(gr[u][e]), pp[u][e], mm[u][e], vv[u][e], s, gmul);
-          if (HAS_PLOW) pl[e] = Lowp<PDT>::from_float(pp[u][e]);
+        for (int u = 0; u < ADAM_UNROLL; ++u) {
+          const int64_t e0 = rg.begin + (i + u * MT_THREADS) * MT_VEC;
+          load8<GDT, AXN_ADAM_NT_G != 0>(g, e0, gr[u]);
+          loadf8<AXN_ADAM_NT_LOAD != 0>(p + e0, pp[u]);
+          loadf8<AXN_ADAM_NT_LOAD != 0>(m + e0, mm[u]);
+          loadf8<AXN_ADAM_NT_LOAD != 0>(v + e0, vv[u]);
         }
-        storef8<AXN_ADAM_NT_STORE != 0>(p + e0, pp[u]);
-        storef8<AXN_ADAM_NT_STORE != 0>(m + e0, mm[u]);
-        storef8<AXN_ADAM_NT_STORE != 0>(v + e0, vv[u]);
-        if (HAS_PLOW) store8<PDT, AXN_ADAM_NT_STORE != 0>(plow, e0, pl);
-      }
-    }
-    for (; i < nvec; i += MT_THREADS) {
-      const int64_t e0 = rg.begin + i * MT_VEC;
-      graw gr[8];
-      float pp[8], mm[8], vv[8];
-      praw pl[8];
-      load8<GDT, AXN_ADAM_NT_G != 0>(g, e0, gr);
-      loadf8<false>(p + e0, pp);
-      loadf8<false>(m + e0, mm);
-      loadf8<false>(v + e0, vv);
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        adam_math(Lowp<GDT>::to_float(gr[e]), pp[e], mm[e], vv[e], s, gmul);
-        if (HAS_PLOW) pl[e] = Lowp<PDT>::from_float(pp[e]);
+        for (int u = 0; u < ADAM_UNROLL; ++u) {
+          const int64_t e0 = rg.begin + (i + u * MT_THREADS) * MT_VEC;
+          praw pl[8];
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            adam_math(Lowp<GDT>::to_float(gr[u][e]), pp[u][e], mm[u][e], vv[u][e], s, gmul);
+            if (HAS_PLOW) pl[e] = Lowp<PDT>::from_float(pp[u][e]);
+          }
+          storef8<AXN_ADAM_NT_STORE != 0>(p + e0, pp[u]);
+          storef8<AXN_ADAM_NT_STORE != 0>(m + e0, mm[u]);
+          storef8<AXN_ADAM_NT_STORE != 0>(v + e0, vv[u]);
+          if (HAS_PLOW) store8<PDT, AXN_ADAM_NT_STORE != 0>(plow, e0, pl);
+        }
       }
-      storef8<AXN_ADAM_NT_STORE != 0>(p + e0, pp);
-      storef8<AXN_ADAM_NT_STORE != 0>(m + e0, mm);
-      storef8<AXN_ADAM_NT_STORE != 0>(v + e0, vv);
-      if (HAS_PLOW) store8<PDT, AXN_ADAM_NT_STORE != 0>(plow, e0, pl);
+      if (ADAM_UNROLL > 1) {
+        for (; i < nvec; i += MT_THREADS) {
+          const int64_t e0 = rg.begin + i * MT_VEC;
+          graw gr[8];
+          float pp[8], mm[8], vv[8];
+          praw pl[8];
+          load8<GDT, AXN_ADAM_NT_G != 0>(g, e0, gr);
+          loadf8<AXN_ADAM_NT_LOAD != 0>(p + e0, pp);
+          loadf8<AXN_ADAM_NT_LOAD != 0>(m + e0, mm);
+          loadf8<AXN_ADAM_NT_LOAD != 0>(v + e0, vv);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            adam_math(Lowp<GDT>::to_float(gr[e]), pp[e], mm[e], vv[e], s, gmul);
+            if (HAS_PLOW) pl[e] = Lowp<PDT>::from_float(pp[e]);
+          }
+          storef8<AXN_ADAM_NT_STORE != 0>(p + e0, pp);
+          storef8<AXN_ADAM_NT_STORE != 0>(m + e0, mm);
+          storef8<AXN_ADAM_NT_STORE != 0>(v + e0, vv);
+          if (HAS_PLOW) store8<PDT, AXN_ADAM_NT_STORE != 0>(plow, e0, pl);
+        }
+      }
+      const int64_t tail = rg.begin + nvec * MT_VEC;
+      if (tail + tid < rg.end) one(tail + tid);
+    } else {
+      const int64_t b0 = (c == 0) ? 0 : rg.begin;
+      for (int64_t i = b0 + tid; i < rg.end; i += MT_THREADS) one(i);
     }
-    const int64_t tail = rg.begin + nvec * MT_VEC;
-    if (tail + tid < rg.end) one(tail + tid);
-  } else {
-    const int64_t b = (c == 0) ? 0 : rg.begin;
-    for (int64_t i = b + tid; i < rg.end; i += MT_THREADS) one(i);
   }
 }
 
@@ -484,6 +519,33 @@ __global__ void __launch_bounds__(MT_THREADS)
     const int64_t b = (c == 0) ? 0 : rg.begin;
     for (int64_t i = b + tid; i < rg.end; i += MT_THREADS) ((raw*)g)[i] = f(((raw*)g)[i]);
   }
+}
+
+// ------------------------------------------------------------- probes ------
+// Plain streaming kernels in the optimizer's access pattern (16-byte vectors, grid-stride,
+// non-temporal stores): what the memory system gives a read, a fill and a copy on this
+// GPU, measured beside the optimizer step by benchmarks.
+__global__ void __launch_bounds__(MT_THREADS)
+    probe_read_kernel(const f32x4* __restrict__ src, int64_t nvec, float* sink) {
+  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+  for (int64_t i = (int64_t)blockIdx.x * MT_THREADS + threadIdx.x; i < nvec;
+       i += (int64_t)gridDim.x * MT_THREADS)
+    acc += ld<true>(src + i);
+  // never true for finite data: keeps the loads alive without a store per lane
+  if (acc[0] + acc[1] + acc[2] + acc[3] == 1.2345678e38f) *sink = acc[0];
+}
+__global__ void __launch_bounds__(MT_THREADS)
+    probe_fill_kernel(f32x4* __restrict__ dst, int64_t nvec) {
+  const f32x4 x = {0.f, 0.f, 0.f, 0.f};
+  for (int64_t i = (int64_t)blockIdx.x * MT_THREADS + threadIdx.x; i < nvec;
+       i += (int64_t)gridDim.x * MT_THREADS)
+    st<true>(x, dst + i);
+}
+__global__ void __launch_bounds__(MT_THREADS)
+    probe_copy_kernel(const f32x4* src, f32x4* dst, int64_t nvec) {
+  for (int64_t i = (int64_t)blockIdx.x * MT_THREADS + threadIdx.x; i < nvec;
+       i += (int64_t)gridDim.x * MT_THREADS)
+    st<true>(ld<false>(src + i), dst + i);
 }
 
 // ------------------------------------------------------------- host side ----
@@ -526,25 +588,27 @@ struct Group {
   int blocks;
 };
 
-// Splits the tensor list into launch groups and fills the argument tables.
-// `ptr_sets[k][i]` is pointer k of tensor i (k = 0 is always the gradient).
-int build_groups(const void* const* const* ptr_sets, const int* elem_sizes,
-                 int nsets, const int64_t* h_sizes, int64_t n, int chunk,
-                 std::vector<Group>& out) {
-  out.clear();
+// Walks the tensor list in launch groups (at most MT_MAX tensors, below 2^31 chunks)
+// and hands each filled argument table to `emit`, which returns a status; the first
+// non-zero status ends the walk.  `ptr_sets[k][i]` is pointer k of tensor i (k = 0 is
+// always the gradient).  Nothing is allocated: the one table lives on the stack.
+template <class Emit>
+int for_each_group(const void* const* const* ptr_sets, const int* elem_sizes, int nsets,
+                   const int64_t* h_sizes, int64_t n, int chunk, Emit&& emit) {
   Group cur;
   cur.tab = MtTable();
   cur.blocks = 0;
   int k = 0;
-  auto flush = [&]() {
-    if (k == 0) return;
+  auto flush = [&]() -> int {
+    if (k == 0) return AXN_OK;
     cur.tab.n = k;
     cur.tab.chunk = chunk;
     cur.tab.chunk_start[k] = cur.blocks;
-    out.push_back(cur);
+    const int rc = emit(cur);
     cur.tab = MtTable();
     cur.blocks = 0;
     k = 0;
+    return rc;
   };
   for (int64_t i = 0; i < n; ++i) {
     const int64_t sz = h_sizes[i];
@@ -563,7 +627,10 @@ int build_groups(const void* const* const* ptr_sets, const int* elem_sizes,
                 (long long)i, (long long)sz);
       return AXN_ELIMIT;
     }
-    if (k == MT_MAX || (long long)cur.blocks + chunks > 0x7fffffffLL) flush();
+    if (k == MT_MAX || (long long)cur.blocks + chunks > 0x7fffffffLL) {
+      const int rc = flush();
+      if (rc != AXN_OK) return rc;
+    }
     cur.tab.g[k] = ptrs[0];
     cur.tab.p[k] = const_cast<void*>(ptrs[1]);
     cur.tab.m[k] = const_cast<void*>(ptrs[2]);
@@ -576,8 +643,7 @@ int build_groups(const void* const* const* ptr_sets, const int* elem_sizes,
     cur.blocks += (int)chunks;
     ++k;
   }
-  flush();
-  return AXN_OK;
+  return flush();
 }
 
 double sum_limit_of(int dt) {
@@ -587,6 +653,38 @@ double sum_limit_of(int dt) {
     case AXN_BF16: return 3.3961775292304601e38;   // 2^127 * (2 - 2^-8)
     default: return 3.4028235677973366e38;         // 2^127 * (2 - 2^-24)
   }
+}
+
+// CUs of the current device (the persistent kernels size their grids by it).
+int cu_count() {
+  static std::atomic<int> cached[64];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+  int n = cached[dev].load(std::memory_order_relaxed);
+  if (n == 0) {
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+      n = 256;
+    cached[dev].store(n, std::memory_order_relaxed);
+  }
+  return n;
+}
+
+template <int DT>
+void scan_dispatch(const Group& gr, float inv_scale, float norm_type, ScanPartial* partial,
+                   int base, hipStream_t stream) {
+  const dim3 grid(gr.blocks), block(MT_THREADS);
+  if (norm_type == 2.0f)
+    hipLaunchKernelGGL((mt_scan_kernel<DT, NORM_2>), grid, block, 0, stream, gr.tab, inv_scale,
+                       norm_type, partial, base);
+  else if (norm_type == 1.0f)
+    hipLaunchKernelGGL((mt_scan_kernel<DT, NORM_1>), grid, block, 0, stream, gr.tab, inv_scale,
+                       norm_type, partial, base);
+  else if (norm_type == 0.0f)
+    hipLaunchKernelGGL((mt_scan_kernel<DT, NORM_0>), grid, block, 0, stream, gr.tab, inv_scale,
+                       norm_type, partial, base);
+  else
+    hipLaunchKernelGGL((mt_scan_kernel<DT, NORM_P>), grid, block, 0, stream, gr.tab, inv_scale,
+                       norm_type, partial, base);
 }
 
 }  // namespace
@@ -599,78 +697,74 @@ size_t mt_scan_workspace_bytes(int64_t n, int64_t total) {
 }
 
 int launch_mt_scan(const void* const* h_g, const int64_t* h_sizes, int64_t n,
-                   int g_dtype, float inv_scale, float max_norm, int accumulate,
-                   axn_scan_result* result, void* ws, size_t ws_bytes,
+                   int g_dtype, float inv_scale, float max_norm, float norm_type,
+                   int accumulate, axn_scan_result* result, void* ws, size_t ws_bytes,
                    hipStream_t stream) {
   const void* const* sets[1] = {h_g};
   const int es[1] = {dtype_size(g_dtype)};
-  std::vector<Group> groups;
-  int rc = build_groups(sets, es, 1, h_sizes, n, SCAN_CHUNK, groups);
-  if (rc != AXN_OK) return rc;
+  // first walk: what the partial results need
   int64_t need = 0;
-  for (auto& gr : groups) need += gr.blocks;
+  int rc = for_each_group(sets, es, 1, h_sizes, n, SCAN_CHUNK, [&](const Group& gr) {
+    need += gr.blocks;
+    return (int)AXN_OK;
+  });
+  if (rc != AXN_OK) return rc;
   if ((size_t)need * sizeof(ScanPartial) > ws_bytes) {
     set_error("mt_scan: workspace too small (%zu bytes given, %zu needed)",
               ws_bytes, (size_t)need * sizeof(ScanPartial));
     return AXN_EINVAL;
   }
   ScanPartial* partial = (ScanPartial*)ws;
-  if (groups.empty()) {
+  if (need == 0) {
     // Nothing to scan: norm 0, no overflow.
     MtTable empty = MtTable();
     empty.n = 0;
     empty.chunk = SCAN_CHUNK;
     hipLaunchKernelGGL(mt_scan_finalize_kernel, dim3(1), dim3(1024), 0, stream,
-                       empty, partial, 0, sum_limit_of(g_dtype), max_norm,
+                       empty, partial, 0, sum_limit_of(g_dtype), max_norm, norm_type,
                        accumulate ? 0 : 1, result);
     AXN_HIP_TRY(hipGetLastError());
     return AXN_OK;
   }
   int base = 0;
   bool first = !accumulate;
-  for (auto& gr : groups) {
+  return for_each_group(sets, es, 1, h_sizes, n, SCAN_CHUNK, [&](const Group& gr) {
     switch (g_dtype) {
-      case AXN_BF16:
-        hipLaunchKernelGGL(mt_scan_kernel<AXN_BF16>, dim3(gr.blocks), dim3(MT_THREADS),
-                           0, stream, gr.tab, inv_scale, partial, base);
-        break;
-      case AXN_F16:
-        hipLaunchKernelGGL(mt_scan_kernel<AXN_F16>, dim3(gr.blocks), dim3(MT_THREADS),
-                           0, stream, gr.tab, inv_scale, partial, base);
-        break;
-      default:
-        hipLaunchKernelGGL(mt_scan_kernel<AXN_F32>, dim3(gr.blocks), dim3(MT_THREADS),
-                           0, stream, gr.tab, inv_scale, partial, base);
-        break;
+      case AXN_BF16: scan_dispatch<AXN_BF16>(gr, inv_scale, norm_type, partial, base, stream); break;
+      case AXN_F16: scan_dispatch<AXN_F16>(gr, inv_scale, norm_type, partial, base, stream); break;
+      default: scan_dispatch<AXN_F32>(gr, inv_scale, norm_type, partial, base, stream); break;
     }
     AXN_HIP_TRY(hipGetLastError());
     hipLaunchKernelGGL(mt_scan_finalize_kernel, dim3(1), dim3(1024), 0, stream,
-                       gr.tab, partial, base, sum_limit_of(g_dtype), max_norm,
+                       gr.tab, partial, base, sum_limit_of(g_dtype), max_norm, norm_type,
                        first ? 1 : 0, result);
     AXN_HIP_TRY(hipGetLastError());
     base += gr.blocks;
     first = false;
-  }
-  return AXN_OK;
+    return (int)AXN_OK;
+  });
 }
 
+namespace {
 template <int GDT>
 int adam_dispatch(const Group& gr, const AdamScalars& s, int plow_dtype,
                   bool has_plow, const axn_scan_result* scan, hipStream_t stream) {
-  const dim3 grid(gr.blocks), block(MT_THREADS);
+  const long long cap = (long long)cu_count() * AXN_ADAM_WGS_PER_CU;
+  const dim3 grid((unsigned)(gr.blocks < cap ? gr.blocks : cap)), block(MT_THREADS);
   if (!has_plow) {
     hipLaunchKernelGGL((mt_adam_kernel<GDT, AXN_BF16, false>), grid, block, 0,
-                       stream, gr.tab, s, scan);
+                       stream, gr.tab, s, scan, gr.blocks);
   } else if (plow_dtype == AXN_BF16) {
     hipLaunchKernelGGL((mt_adam_kernel<GDT, AXN_BF16, true>), grid, block, 0,
-                       stream, gr.tab, s, scan);
+                       stream, gr.tab, s, scan, gr.blocks);
   } else {
     hipLaunchKernelGGL((mt_adam_kernel<GDT, AXN_F16, true>), grid, block, 0,
-                       stream, gr.tab, s, scan);
+                       stream, gr.tab, s, scan, gr.blocks);
   }
   AXN_HIP_TRY(hipGetLastError());
   return AXN_OK;
 }
+}  // namespace
 
 int launch_mt_adam(const void* const* h_g, void* const* h_p, void* const* h_m,
                    void* const* h_v, void* const* h_plow, const int64_t* h_sizes,
@@ -680,21 +774,41 @@ int launch_mt_adam(const void* const* h_g, void* const* h_p, void* const* h_m,
   const void* const* sets[5] = {h_g, (const void* const*)h_p, (const void* const*)h_m,
                                 (const void* const*)h_v, (const void* const*)h_plow};
   const int es[5] = {dtype_size(g_dtype), 4, 4, 4, dtype_size(plow_dtype)};
-  std::vector<Group> groups;
-  int rc = build_groups(sets, es, 5, h_sizes, n, ADAM_CHUNK, groups);
-  if (rc != AXN_OK) return rc;
   AdamScalars s;
   s.hp = hp;
   s.inv_scale = inv_scale;
   const bool has_plow = h_plow != nullptr;
-  for (auto& gr : groups) {
+  return for_each_group(sets, es, 5, h_sizes, n, ADAM_CHUNK, [&](const Group& gr) {
     switch (g_dtype) {
-      case AXN_BF16: rc = adam_dispatch<AXN_BF16>(gr, s, plow_dtype, has_plow, scan, stream); break;
-      case AXN_F16: rc = adam_dispatch<AXN_F16>(gr, s, plow_dtype, has_plow, scan, stream); break;
-      default: rc = adam_dispatch<AXN_F32>(gr, s, plow_dtype, has_plow, scan, stream); break;
+      case AXN_BF16: return adam_dispatch<AXN_BF16>(gr, s, plow_dtype, has_plow, scan, stream);
+      case AXN_F16: return adam_dispatch<AXN_F16>(gr, s, plow_dtype, has_plow, scan, stream);
+      default: return adam_dispatch<AXN_F32>(gr, s, plow_dtype, has_plow, scan, stream);
     }
-    if (rc != AXN_OK) return rc;
+  });
+}
+
+int launch_stream_probe(int kind, const void* src, void* dst, size_t bytes, hipStream_t stream) {
+  const int64_t nvec = (int64_t)(bytes / 16);
+  if (nvec == 0) return AXN_OK;
+  // enough workgroups to keep every CU's memory pipeline full, few enough to stay resident
+  long long blocks = (nvec + MT_THREADS - 1) / MT_THREADS;
+  const long long cap = (long long)cu_count() * 32;
+  if (blocks > cap) blocks = cap;
+  const dim3 grid((unsigned)blocks), block(MT_THREADS);
+  switch (kind) {
+    case AXN_PROBE_READ:
+      hipLaunchKernelGGL(probe_read_kernel, grid, block, 0, stream, (const f32x4*)src, nvec,
+                         (float*)dst);
+      break;
+    case AXN_PROBE_FILL:
+      hipLaunchKernelGGL(probe_fill_kernel, grid, block, 0, stream, (f32x4*)dst, nvec);
+      break;
+    default:
+      hipLaunchKernelGGL(probe_copy_kernel, grid, block, 0, stream, (const f32x4*)src, (f32x4*)dst,
+                         nvec);
+      break;
   }
+  AXN_HIP_TRY(hipGetLastError());
   return AXN_OK;
 }
 
@@ -703,10 +817,7 @@ int launch_mt_scale(void* const* h_g, const int64_t* h_sizes, int64_t n,
                     int use_clip, hipStream_t stream) {
   const void* const* sets[1] = {(const void* const*)h_g};
   const int es[1] = {dtype_size(g_dtype)};
-  std::vector<Group> groups;
-  int rc = build_groups(sets, es, 1, h_sizes, n, SCALE_CHUNK, groups);
-  if (rc != AXN_OK) return rc;
-  for (auto& gr : groups) {
+  return for_each_group(sets, es, 1, h_sizes, n, SCALE_CHUNK, [&](const Group& gr) {
     const dim3 grid(gr.blocks), block(MT_THREADS);
     switch (g_dtype) {
       case AXN_BF16:
@@ -723,8 +834,8 @@ int launch_mt_scale(void* const* h_g, const int64_t* h_sizes, int64_t n,
         break;
     }
     AXN_HIP_TRY(hipGetLastError());
-  }
-  return AXN_OK;
+    return (int)AXN_OK;
+  });
 }
 
 }  // namespace axn

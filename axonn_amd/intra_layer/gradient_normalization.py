@@ -1,13 +1,14 @@
-"""Gradient clipping by global 2-norm, same signature and return value as
+"""Gradient clipping by a global p-norm, same signature and return value as
 axonn/intra_layer/gradient_normalization.py:37-95.
 
-The reference takes one `torch.norm` per gradient, all-reduces the squared norm
-of every tensor-parallel group and multiplies every gradient by the clamped
-coefficient.  With one rank per group the total is the 2-norm over all
-gradients; here one multi-tensor kernel reads the gradients once (sum of squares
-in fp32 per workgroup, fp64 across workgroups), leaves norm and coefficient on
-the device, and a second multi-tensor kernel scales the gradients in place - no
-host synchronisation.
+The reference takes one `torch.norm(g, p)` per gradient, all-reduces the p-th power
+of every tensor-parallel group's norm and multiplies every gradient by the clamped
+coefficient.  With one rank per group the total is the p-norm over all gradients
+(for p = 0, torch.norm's count: the number of gradients with a non-zero element);
+here one multi-tensor kernel reads the gradients once (sum of |g|^p in fp32 per
+workgroup, fp64 across workgroups), leaves norm and coefficient on the device, and
+a second multi-tensor kernel scales the gradients in place - no host
+synchronisation.  Any finite p; p = inf raises as in the reference (:38-39).
 """
 
 from collections import defaultdict
@@ -19,12 +20,12 @@ from .. import ops
 
 
 def get_total_norm(tensors, norm_type=2.0, error_if_nonfinite=False):
-    """2-norm over a list of tensors (gradient_normalization.py:18-34)."""
-    if float(norm_type) != 2.0:
-        raise NotImplementedError("only the 2-norm is implemented on the GPU path")
+    """p-norm over a list of tensors (gradient_normalization.py:18-34)."""
+    if norm_type == inf or norm_type == -inf:
+        raise NotImplementedError
     if len(tensors) == 0:
         return torch.tensor(0.0)
-    result = _scan(tensors, 0.0)
+    result = _scan(tensors, 0.0, norm_type)
     total = result.total_norm.clone()
     if error_if_nonfinite and not bool(torch.isfinite(total)):
         raise RuntimeError(
@@ -36,21 +37,20 @@ def get_total_norm(tensors, norm_type=2.0, error_if_nonfinite=False):
     return total
 
 
-def _scan(grads, max_norm):
+def _scan(grads, max_norm, norm_type=2.0):
     by_dtype = defaultdict(list)
     for g in grads:
         by_dtype[g.dtype].append(g.detach())
     result = None
     for group in by_dtype.values():
-        result = ops.mt_scan(group, 1.0, max_norm, result=result, accumulate=result is not None)
+        result = ops.mt_scan(group, 1.0, max_norm, result=result, accumulate=result is not None,
+                             norm_type=norm_type)
     return result
 
 
 def clip_grad_norm_(parameters, max_norm, norm_type=2.0, error_if_nonfinite=False):
     if norm_type == inf:
         raise NotImplementedError
-    if float(norm_type) != 2.0:
-        raise NotImplementedError("only the 2-norm is implemented on the GPU path")
     if isinstance(parameters, torch.Tensor):
         parameters = [parameters]
     grads = []
@@ -62,9 +62,10 @@ def clip_grad_norm_(parameters, max_norm, norm_type=2.0, error_if_nonfinite=Fals
         if p.grad is not None:
             grads.append(p.grad)
     max_norm = float(max_norm)
+    norm_type = float(norm_type)
     if len(grads) == 0:
         return torch.tensor(0.0)
-    result = _scan(grads, max_norm)
+    result = _scan(grads, max_norm, norm_type)
     total_norm = result.total_norm.clone()
     if error_if_nonfinite and not bool(torch.isfinite(total_norm)):
         raise RuntimeError(

@@ -535,9 +535,9 @@ def _check_list(tensors, dtype=None):
             raise TypeError("expected %s, got %s" % (dtype, t.dtype))
 
 
-def mt_scan(grads, inv_scale=1.0, max_norm=0.0, result=None, accumulate=False):
-    """Overflow flag, sum of squares, 2-norm and clip coefficient of a list of
-    gradients of ONE dtype, left on the device in a ScanResult."""
+def mt_scan(grads, inv_scale=1.0, max_norm=0.0, result=None, accumulate=False, norm_type=2.0):
+    """Overflow flag, sum of |g|^p, p-norm and clip coefficient of a list of gradients of
+    ONE dtype, left on the device in a ScanResult."""
     if len(grads) == 0:
         raise ValueError("empty gradient list")
     dt = grads[0].dtype
@@ -546,12 +546,20 @@ def mt_scan(grads, inv_scale=1.0, max_norm=0.0, result=None, accumulate=False):
     if result is None:
         result = ScanResult(device)
         accumulate = False
+    norm_type = float(norm_type)
+    if norm_type in (float("inf"), float("-inf")) or norm_type != norm_type:
+        raise NotImplementedError("the norm's order must be finite")
     total = sum(g.numel() for g in grads)
     ws_bytes = nv.load().axn_mt_scan_workspace_bytes(len(grads), total)
     ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=device)
-    nv.call("axn_mt_scan", nv.ptr_array(grads), nv.size_array(grads), len(grads),
-            nv.dtype_code(dt), float(inv_scale), float(max_norm), 1 if accumulate else 0,
-            result.ptr(), nv.ptr(ws), ws_bytes, nv.current_stream())
+    if norm_type == 2.0:
+        nv.call("axn_mt_scan", nv.ptr_array(grads), nv.size_array(grads), len(grads),
+                nv.dtype_code(dt), float(inv_scale), float(max_norm), 1 if accumulate else 0,
+                result.ptr(), nv.ptr(ws), ws_bytes, nv.current_stream())
+    else:
+        nv.call("axn_mt_scan_norm", nv.ptr_array(grads), nv.size_array(grads), len(grads),
+                nv.dtype_code(dt), float(inv_scale), float(max_norm), norm_type,
+                1 if accumulate else 0, result.ptr(), nv.ptr(ws), ws_bytes, nv.current_stream())
     return result
 
 

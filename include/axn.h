@@ -30,7 +30,7 @@
 extern "C" {
 #endif
 
-#define AXN_ABI_VERSION 8
+#define AXN_ABI_VERSION 9
 
 #if defined(__GNUC__)
 #define AXN_API __attribute__((visibility("default")))
@@ -293,8 +293,9 @@ AXN_API int axn_gemm_wgrad_f32(const float* dY, const float* X, float* dW, int64
 /* Device-resident result of the gradient scan, consumed by axn_mt_adam and
  * axn_mt_scale without a host round trip.  32 bytes. */
 typedef struct axn_scan_result {
-  double sumsq;       /* sum over all tensors of (g * inv_scale)^2            */
-  float total_norm;   /* sqrt(sumsq)                                          */
+  double sumsq;       /* sum over all tensors of |g * inv_scale|^p (p = 2 unless
+                         axn_mt_scan_norm names another order)                */
+  float total_norm;   /* sumsq^(1/p)                                          */
   float clip_coef;    /* min(1, max_norm / (total_norm + 1e-6)); 1 if no clip */
   int32_t found_inf;  /* 1 if the overflow check fired, else 0                */
   int32_t reserved[3];
@@ -322,6 +323,19 @@ AXN_API int axn_mt_scan(const void* const* h_g, const int64_t* h_sizes, int64_t 
                 int g_dtype, float inv_scale, float max_norm, int accumulate,
                 axn_scan_result* result, void* workspace,
                 size_t workspace_bytes, void* stream);
+
+/* The same scan with the norm's order as an argument: total_norm = (sum |g * inv_scale|^p)^(1/p)
+ * for any finite p = norm_type, which is what the reference's clipping accepts
+ * (axonn/intra_layer/gradient_normalization.py:18-34 takes torch.norm(g, norm_type) per
+ * gradient and the norm_type-norm of those; :74-87 the coefficient).  p = 0 follows
+ * torch.norm's meaning there: the number of gradients that have a non-zero element.
+ * p = inf is not taken (the reference raises NotImplementedError, :38-39): AXN_EINVAL.
+ * axn_mt_scan is this call with norm_type = 2.  Calls that accumulate into one result
+ * must name the same order. */
+AXN_API int axn_mt_scan_norm(const void* const* h_g, const int64_t* h_sizes, int64_t n,
+                     int g_dtype, float inv_scale, float max_norm, float norm_type,
+                     int accumulate, axn_scan_result* result, void* workspace,
+                     size_t workspace_bytes, void* stream);
 
 /* Scalar hyper-parameters of one Adam step.  The bias corrections are
  * computed by the caller in double precision, as torch does
@@ -363,6 +377,19 @@ AXN_API int axn_mt_adam(const void* const* h_g, void* const* h_p, void* const* h
 AXN_API int axn_mt_scale(void* const* h_g, const int64_t* h_sizes, int64_t n,
                  int g_dtype, float inv_scale, const axn_scan_result* scan,
                  int use_clip, void* stream);
+
+/* ------------------------------------------------------------------------
+ * Measurement aid, no counterpart in the reference: plain streaming kernels in the
+ * optimizer kernels' access pattern (16-byte vectors per lane, grid-stride, non-temporal
+ * stores), so that a benchmark can put the optimizer step's rate beside what the memory
+ * system of the same GPU gives a plain read, fill or copy.
+ *   AXN_PROBE_READ: reads `bytes` from src (dst: 4 writable bytes, never written for
+ *                   finite data); AXN_PROBE_FILL: writes `bytes` of zeros to dst;
+ *   AXN_PROBE_COPY: copies `bytes` from src to dst (src == dst: in place).
+ * Pointers 16-byte aligned; bytes is rounded down to a multiple of 16.
+ * ------------------------------------------------------------------------ */
+typedef enum axn_probe_kind { AXN_PROBE_READ = 0, AXN_PROBE_FILL = 1, AXN_PROBE_COPY = 2 } axn_probe_kind;
+AXN_API int axn_stream_probe(int kind, const void* src, void* dst, size_t bytes, void* stream);
 
 #ifdef __cplusplus
 }

@@ -102,13 +102,24 @@ def unscale_gradients(grads, dtype, loss_scale):
 
 
 # ----------------------------------------------------------- grad norm -------
-def get_total_norm(tensors, dtype="f64"):
-    """gradient_normalization.py:18-34 for norm_type 2: the norm of the stacked
-    per-tensor norms, each torch.norm returning the tensor's dtype."""
+def _norm(x, norm_type):
+    """torch.norm(x, p) of a flat float64 vector for finite p: (sum |x|^p)^(1/p); p = 0
+    counts the non-zero elements."""
+    x = np.abs(np.asarray(x, dtype=np.float64).reshape(-1))
+    if norm_type == 0:
+        return float(np.count_nonzero(x))
+    with np.errstate(divide="ignore", over="ignore"):
+        return float(np.sum(x ** norm_type) ** (1.0 / norm_type))
+
+
+def get_total_norm(tensors, dtype="f64", norm_type=2.0):
+    """gradient_normalization.py:18-34: the norm_type-norm of the stacked per-tensor
+    norm_type-norms, each torch.norm returning the tensor's dtype.  The reference passes
+    any finite order through to torch.norm (inf is refused earlier, :38-39)."""
     if len(tensors) == 0:
         return 0.0
-    per = [round_to(np.sqrt(np.sum(np.asarray(t, dtype=np.float64) ** 2)), dtype) for t in tensors]
-    return float(round_to(np.sqrt(np.sum(np.asarray(per) ** 2)), dtype))
+    per = [round_to(_norm(t, norm_type), dtype) for t in tensors]
+    return float(round_to(_norm(np.asarray(per), norm_type), dtype))
 
 
 def clip_coef(total_norm, max_norm):
@@ -117,12 +128,13 @@ def clip_coef(total_norm, max_norm):
     return min(c, 1.0) if c == c else c
 
 
-def clip_grad_norm_(grads, max_norm, dtype="f64"):
-    """gradient_normalization.py:37-95 on one rank, norm_type 2: every process
-    group has one member, so the total is the norm over all gradients; every
-    gradient is multiplied by the clamped coefficient, also when it is 1.
+def clip_grad_norm_(grads, max_norm, dtype="f64", norm_type=2.0):
+    """gradient_normalization.py:37-95 on one rank: every process group has one member
+    (the all-reduce of norm^p over a group and the 1/p power after it, :74-81, give the
+    group's norm back), so the total is the norm over all gradients; every gradient is
+    multiplied by the clamped coefficient, also when it is 1.
     Returns (total_norm, clipped grads)."""
-    total = get_total_norm(grads, dtype)
+    total = get_total_norm(grads, dtype, norm_type)
     c = clip_coef(total, max_norm)
     c = float(round_to(c, "f32"))  # the coefficient is a float32 tensor in torch
     return total, [round_to(np.asarray(g, dtype=np.float64) * c, dtype) for g in grads]

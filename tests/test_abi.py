@@ -233,6 +233,29 @@ def test_multi_tensor_argument_errors():
     assert lib.axn_mt_scale(ptrs, sizes, -1, nv.BF16, 1.0, None, 0, None) == nv.AXN_EINVAL
 
 
+def test_scan_variants_argument_errors():
+    """The norm's order must be finite."""
+    lib = nv.load()
+    ptrs = (ctypes.c_void_p * 2)(0x1000, 0x2000)
+    sizes = (ctypes.c_int64 * 2)(4, 4)
+    res = ctypes.c_void_p(0x3000)
+    for bad in (float("inf"), float("-inf"), float("nan")):
+        assert lib.axn_mt_scan_norm(ptrs, sizes, 2, nv.BF16, 1.0, 0.0, bad, 0, res, A, 4096,
+                                    None) == nv.AXN_EINVAL
+        assert "finite" in _err()
+    assert lib.axn_mt_scan_norm(ptrs, sizes, 2, nv.BF16, 1.0, 0.0, 3.0, 0, res, A, 0,
+                                None) == nv.AXN_EINVAL          # workspace too small
+
+
+def test_stream_probe_argument_errors():
+    lib = nv.load()
+    assert lib.axn_stream_probe(7, A, A, 1024, None) == nv.AXN_EINVAL
+    assert lib.axn_stream_probe(2, None, A, 1024, None) == nv.AXN_EINVAL
+    assert lib.axn_stream_probe(1, None, None, 1024, None) == nv.AXN_EINVAL
+    assert lib.axn_stream_probe(2, ctypes.c_void_p(0x1008), A, 1024, None) == nv.AXN_EALIGN
+    assert lib.axn_stream_probe(1, None, A, 0, None) == nv.AXN_OK     # nothing to do, nothing launched
+
+
 def test_adam_hparams_struct_layout():
     assert ctypes.sizeof(nv.AdamHParams) == 32
     assert nv.SCAN_RESULT_BYTES == 32

@@ -154,8 +154,12 @@ def test_adam_hparams_use_double_precision_bias_corrections():
 def test_clip_grad_norm_argument_handling():
     with pytest.raises(NotImplementedError):
         clip_grad_norm_([], 1.0, norm_type=float("inf"))
+    from axonn_amd.intra_layer.gradient_normalization import get_total_norm
+
     with pytest.raises(NotImplementedError):
-        clip_grad_norm_([], 1.0, norm_type=1.0)
+        get_total_norm([torch.zeros(2)], float("inf"))
+    assert float(clip_grad_norm_([], 1.0, norm_type=1.0)) == 0.0        # any finite order is taken
+    assert float(get_total_norm([], 3.0)) == 0.0
     assert float(clip_grad_norm_([torch.nn.Parameter(torch.zeros(2))], 1.0)) == 0.0  # no grads
 
 

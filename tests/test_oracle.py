@@ -268,6 +268,33 @@ def test_norm_of_norms_equals_flat_norm():
     assert oo.get_total_norm([]) == 0.0
 
 
+@pytest.mark.parametrize("p", [1.0, 3.0, 0.5, 4.0, 1.5, -1.0, 0.0])
+def test_clip_of_any_finite_order_matches_torch(p):
+    """The reference hands norm_type to torch.norm per gradient and once more over the
+    stacked results (gradient_normalization.py:18-34); torch.nn.utils.clip_grad_norm_
+    computes the same quantity, and for p != 0 it equals the p-norm of all elements."""
+    torch.manual_seed(60)
+    params = [torch.nn.Parameter(torch.zeros(n)) for n in (5, 17, 64)]
+    for q in params:
+        q.grad = torch.randn_like(q) * 0.3
+    params[1].grad[3] = 0.0
+    grads = [q.grad.clone().double().numpy() for q in params]
+    want = torch.norm(torch.stack([torch.norm(q.grad.detach(), p) for q in params]), p)   # :21-24
+    total = torch.nn.utils.clip_grad_norm_(params, 0.05, norm_type=p, foreach=False)
+    t, clipped = oo.clip_grad_norm_(grads, 0.05, "f32", norm_type=p)
+    assert abs(t - float(want)) <= 2e-6 * abs(float(want))
+    assert abs(t - float(total)) <= 2e-6 * abs(float(total))
+    for c, q in zip(clipped, params):
+        assert np.allclose(c, q.grad.double().numpy(), rtol=1e-6, atol=0)
+    flat = np.abs(np.concatenate(grads))
+    if p == 0.0:
+        assert t == 3.0                       # three gradients with a non-zero element
+    elif p > 0:
+        assert abs(t - float(np.sum(flat ** p) ** (1.0 / p))) <= 1e-6 * t
+    else:
+        assert t == 0.0                       # a zero element: |0|^p = inf, inf^(1/p) = 0
+
+
 # ------------------------------------------------------------------ Adam -----
 @pytest.mark.parametrize("wd", [0.0, 0.01])
 def test_adam_matches_torch_optim_adam_over_steps(wd):
