@@ -84,6 +84,7 @@ SYMBOLS = {
     "axn_mt_scan_workspace_bytes": (_sz, [_i64, _i64]),
     "axn_mt_scan": (_int, [_pp, _pi64, _i64, _int, _f32, _f32, _int, _vp, _vp, _sz, _vp]),
     "axn_mt_scan_norm": (_int, [_pp, _pi64, _i64, _int, _f32, _f32, _f32, _int, _vp, _vp, _sz, _vp]),
+    "axn_mt_scan_noalloc": (_int, [_pp, _pi64, _i64, _int, _f32, _f32, _int, _vp, _vp]),
     "axn_mt_adam": (_int, [_pp, _pp, _pp, _pp, _pp, _pi64, _i64, _int, _int, _f32, _vp,
                            _c.POINTER(AdamHParams), _vp]),
     "axn_mt_scale": (_int, [_pp, _pi64, _i64, _int, _f32, _vp, _int, _vp]),

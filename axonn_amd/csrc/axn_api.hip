@@ -634,6 +634,16 @@ int axn_mt_scan(const void* const* h_g, const int64_t* h_sizes, int64_t n,
                           workspace, workspace_bytes, stream);
 }
 
+int axn_mt_scan_noalloc(const void* const* h_g, const int64_t* h_sizes, int64_t n,
+                        int g_dtype, float inv_scale, float max_norm, int accumulate,
+                        axn_scan_result* result, void* stream) {
+  int rc = check_scan_args("axn_mt_scan_noalloc", h_g, h_sizes, n, g_dtype, 2.0f, accumulate,
+                           result);
+  if (rc) return rc;
+  return launch_mt_scan_noalloc(h_g, h_sizes, n, g_dtype, inv_scale, max_norm, 2.0f, accumulate,
+                                result, (hipStream_t)stream);
+}
+
 int axn_stream_probe(int kind, const void* src, void* dst, size_t bytes, void* stream) {
   const char* name = "axn_stream_probe";
   REQUIRE(kind == AXN_PROBE_READ || kind == AXN_PROBE_FILL || kind == AXN_PROBE_COPY, AXN_EINVAL,

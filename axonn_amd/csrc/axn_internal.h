@@ -181,6 +181,10 @@ int launch_mt_scan(const void* const* h_g, const int64_t* h_sizes, int64_t n,
                    int g_dtype, float inv_scale, float max_norm, float norm_type,
                    int accumulate, axn_scan_result* result, void* ws, size_t ws_bytes,
                    hipStream_t stream);
+// The same with the partial results in the library's own device array (no workspace).
+int launch_mt_scan_noalloc(const void* const* h_g, const int64_t* h_sizes, int64_t n,
+                           int g_dtype, float inv_scale, float max_norm, float norm_type,
+                           int accumulate, axn_scan_result* result, hipStream_t stream);
 int launch_mt_adam(const void* const* h_g, void* const* h_p, void* const* h_m,
                    void* const* h_v, void* const* h_plow, const int64_t* h_sizes,
                    int64_t n, int g_dtype, int plow_dtype, float inv_scale,

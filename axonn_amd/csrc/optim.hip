@@ -24,6 +24,7 @@
 
 #include <atomic>
 #include <cmath>
+#include <mutex>
 
 namespace axn {
 namespace {
@@ -688,6 +689,41 @@ void scan_dispatch(const Group& gr, float inv_scale, float norm_type, ScanPartia
 }
 
 }  // namespace
+}  // namespace axn
+
+// Scratch of axn_mt_scan_noalloc: the per-chunk partial results of the scan, in device
+// memory that exists for the life of the process (1 MiB per GPU the library runs on).
+// This name is a host-side handle only; the device address is looked up per device.
+static __device__ __align__(256) unsigned char scratch[AXN_MT_SCAN_SCRATCH_BYTES];
+
+namespace axn {
+namespace {
+
+// Device address of `scratch` on the current device, looked up once per device.
+int scan_scratch(void** out) {
+  static std::mutex mu;
+  static void* ptrs[64];
+  int dev = 0;
+  AXN_HIP_TRY(hipGetDevice(&dev));
+  if (dev < 0 || dev >= 64) {
+    set_error("axn_mt_scan_noalloc: device index %d out of range", dev);
+    return AXN_ELIMIT;
+  }
+  std::lock_guard<std::mutex> lock(mu);
+  if (ptrs[dev] == nullptr) {
+    void* p = nullptr;
+    AXN_HIP_TRY(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    if (p == nullptr) {
+      set_error("axn_mt_scan_noalloc: no device address for the scratch array");
+      return AXN_EHIP;
+    }
+    ptrs[dev] = p;
+  }
+  *out = ptrs[dev];
+  return AXN_OK;
+}
+
+}  // namespace
 
 size_t mt_scan_workspace_bytes(int64_t n, int64_t total) {
   if (n < 0 || total < 0) return 0;
@@ -743,6 +779,32 @@ int launch_mt_scan(const void* const* h_g, const int64_t* h_sizes, int64_t n,
     first = false;
     return (int)AXN_OK;
   });
+}
+
+int launch_mt_scan_noalloc(const void* const* h_g, const int64_t* h_sizes, int64_t n,
+                           int g_dtype, float inv_scale, float max_norm, float norm_type,
+                           int accumulate, axn_scan_result* result, hipStream_t stream) {
+  // the size limit is checked before anything touches the device
+  const void* const* sets[1] = {h_g};
+  const int es[1] = {dtype_size(g_dtype)};
+  int64_t need = 0;
+  int rc = for_each_group(sets, es, 1, h_sizes, n, SCAN_CHUNK, [&](const Group& gr) {
+    need += gr.blocks;
+    return (int)AXN_OK;
+  });
+  if (rc != AXN_OK) return rc;
+  if ((size_t)need * sizeof(ScanPartial) > (size_t)AXN_MT_SCAN_SCRATCH_BYTES) {
+    set_error("axn_mt_scan_noalloc: the gradients make %lld chunks of %d elements, the built-in "
+              "scratch holds %lld; use axn_mt_scan with a workspace",
+              (long long)need, SCAN_CHUNK,
+              (long long)(AXN_MT_SCAN_SCRATCH_BYTES / sizeof(ScanPartial)));
+    return AXN_ELIMIT;
+  }
+  void* ws = nullptr;
+  rc = scan_scratch(&ws);
+  if (rc != AXN_OK) return rc;
+  return launch_mt_scan(h_g, h_sizes, n, g_dtype, inv_scale, max_norm, norm_type, accumulate,
+                        result, ws, (size_t)AXN_MT_SCAN_SCRATCH_BYTES, stream);
 }
 
 namespace {

@@ -535,9 +535,12 @@ def _check_list(tensors, dtype=None):
             raise TypeError("expected %s, got %s" % (dtype, t.dtype))
 
 
-def mt_scan(grads, inv_scale=1.0, max_norm=0.0, result=None, accumulate=False, norm_type=2.0):
+def mt_scan(grads, inv_scale=1.0, max_norm=0.0, result=None, accumulate=False, norm_type=2.0,
+            workspace=True):
     """Overflow flag, sum of |g|^p, p-norm and clip coefficient of a list of gradients of
-    ONE dtype, left on the device in a ScanResult."""
+    ONE dtype, left on the device in a ScanResult.  workspace=False takes the entry point
+    that keeps its partial results in the library's own device array (no allocation here
+    or there; 2-norm only, sizes up to the array's limit)."""
     if len(grads) == 0:
         raise ValueError("empty gradient list")
     dt = grads[0].dtype
@@ -549,6 +552,13 @@ def mt_scan(grads, inv_scale=1.0, max_norm=0.0, result=None, accumulate=False, n
     norm_type = float(norm_type)
     if norm_type in (float("inf"), float("-inf")) or norm_type != norm_type:
         raise NotImplementedError("the norm's order must be finite")
+    if not workspace:
+        if norm_type != 2.0:
+            raise ValueError("the entry point without a workspace computes the 2-norm")
+        nv.call("axn_mt_scan_noalloc", nv.ptr_array(grads), nv.size_array(grads), len(grads),
+                nv.dtype_code(dt), float(inv_scale), float(max_norm), 1 if accumulate else 0,
+                result.ptr(), nv.current_stream())
+        return result
     total = sum(g.numel() for g in grads)
     ws_bytes = nv.load().axn_mt_scan_workspace_bytes(len(grads), total)
     ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=device)

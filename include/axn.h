@@ -337,6 +337,25 @@ AXN_API int axn_mt_scan_norm(const void* const* h_g, const int64_t* h_sizes, int
                      int accumulate, axn_scan_result* result, void* workspace,
                      size_t workspace_bytes, void* stream);
 
+/* axn_mt_scan for callers that cannot allocate device memory and have no workspace to
+ * hand over (code under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc).  No counterpart in the reference.  Arguments and results as axn_mt_scan
+ * without the workspace: the per-chunk partial results go to an array of
+ * AXN_MT_SCAN_SCRATCH_BYTES that is part of the library's device image (each GPU the
+ * library runs on holds its own copy until the process ends).  The call allocates and
+ * frees nothing, on the device or through a library.
+ * Limit: axn_mt_scan_workspace_bytes(n, total) <= AXN_MT_SCAN_SCRATCH_BYTES, i.e. about
+ * 4.29e9 gradient elements in up to a few thousand tensors; beyond it the call returns
+ * AXN_ELIMIT before it touches the device.
+ * All calls on one GPU share that GPU's array: calls that may overlap in time on one GPU
+ * (different streams, different host threads) race and must be serialised by the caller.
+ * Nothing in the array needs to start at zero (every partial result a call reads it has
+ * written itself), so the array is never cleared. */
+#define AXN_MT_SCAN_SCRATCH_BYTES 1048576
+AXN_API int axn_mt_scan_noalloc(const void* const* h_g, const int64_t* h_sizes, int64_t n,
+                        int g_dtype, float inv_scale, float max_norm, int accumulate,
+                        axn_scan_result* result, void* stream);
+
 /* Scalar hyper-parameters of one Adam step.  The bias corrections are
  * computed by the caller in double precision, as torch does
  * (torch/optim/adam.py::_single_tensor_adam, reached from

@@ -234,7 +234,8 @@ def test_multi_tensor_argument_errors():
 
 
 def test_scan_variants_argument_errors():
-    """The norm's order must be finite."""
+    """The norm's order must be finite; the entry point without a workspace rejects what
+    its built-in array cannot hold before it touches the device."""
     lib = nv.load()
     ptrs = (ctypes.c_void_p * 2)(0x1000, 0x2000)
     sizes = (ctypes.c_int64 * 2)(4, 4)
@@ -245,6 +246,15 @@ def test_scan_variants_argument_errors():
         assert "finite" in _err()
     assert lib.axn_mt_scan_norm(ptrs, sizes, 2, nv.BF16, 1.0, 0.0, 3.0, 0, res, A, 0,
                                 None) == nv.AXN_EINVAL          # workspace too small
+    assert lib.axn_mt_scan_noalloc(ptrs, sizes, 2, 9, 1.0, 0.0, 0, res, None) == nv.AXN_EINVAL
+    assert lib.axn_mt_scan_noalloc(ptrs, sizes, 2, nv.BF16, 1.0, 0.0, 0, None, None) == nv.AXN_EINVAL
+    # 65536 chunks of 65536 elements fit the 1 MiB array; three tensors of 2^31 elements do not
+    limit = 1048576
+    assert lib.axn_mt_scan_workspace_bytes(3, 3 * 2 ** 31) > limit
+    ptrs3 = (ctypes.c_void_p * 3)(0x1000, 0x2000, 0x4000)
+    sizes3 = (ctypes.c_int64 * 3)(2 ** 31, 2 ** 31, 2 ** 31)
+    assert lib.axn_mt_scan_noalloc(ptrs3, sizes3, 3, nv.BF16, 1.0, 0.0, 0, res, None) == nv.AXN_ELIMIT
+    assert "scratch" in _err() and "axn_mt_scan" in _err()
 
 
 def test_stream_probe_argument_errors():
