@@ -21,7 +21,7 @@ AXN_ELIMIT = -5
 BF16, F16, F32 = 0, 1, 2
 EPI_NONE, EPI_BIAS, EPI_BIAS_GELU, EPI_GELU = 0, 1, 2, 3
 
-ABI_VERSION = 9
+ABI_VERSION = 10
 
 # Every symbol include/axn.h declares: name -> (restype, argtypes)
 _c = ctypes
@@ -67,8 +67,6 @@ SYMBOLS = {
     "axn_dgelu_dbias": (_int, [_vp, _vp, _vp, _int, _vp, _i64, _i64, _i64, _int, _vp, _sz, _vp]),
     "axn_gemm_swiglu_fwd": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _int, _i64, _i64, _i64, _i64, _i64, _i64, _vp]),
     "axn_gemm_dgrad_pair": (_int, [_vp, _vp, _vp, _vp, _vp, _int, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _vp]),
-    "axn_gemm_wgrad_pair": (_int, [_vp, _vp, _vp, _vp, _int, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _int, _int, _vp]),
-    "axn_swiglu_bwd_strided": (_int, [_vp, _vp, _vp, _vp, _vp, _int, _i64, _i64, _i64, _i64, _vp]),
     "axn_dgelu_dbias_workspace_bytes": (_sz, [_i64, _i64]),
     "axn_swiglu_fwd": (_int, [_vp, _vp, _vp, _int, _i64, _i64, _i64, _vp]),
     "axn_swiglu_bwd": (_int, [_vp, _vp, _vp, _vp, _vp, _int, _i64, _i64, _i64, _vp]),

@@ -367,41 +367,6 @@ int axn_gemm_dgrad_pair(const void* dY1, const void* W1, const void* dY2, const 
   return launch_gemm_pair(g, dtype == AXN_F16, (hipStream_t)stream);
 }
 
-int axn_gemm_wgrad_pair(const void* dY, const void* X, void* dW1, void* dW2, int dtype, int64_t M,
-                        int64_t N1, int64_t N2, int64_t K, int64_t lddy, int64_t ldx, int64_t lddw,
-                        int beta, int dw_dtype, void* stream) {
-  const char* name = "axn_gemm_wgrad_pair";
-  REQUIRE(dtype == AXN_BF16 || dtype == AXN_F16, AXN_EINVAL, "%s: dtype must be bf16 or fp16", name);
-  REQUIRE(N1 >= 1 && N2 >= 1 && N1 <= 0x7fffffff - N2, AXN_EINVAL, "%s: N1 and N2 must be >= 1", name);
-  int rc = check_gemm(name, dY, X, dW1, M, N1 + N2, K, lddy, ldx, lddw, N1 + N2, K, K);
-  if (rc) return rc;
-  REQUIRE(dW2 != nullptr, AXN_EINVAL, "%s: null operand pointer", name);
-  REQUIRE(aligned16(dW2), AXN_EALIGN, "%s: operand pointers must be 16-byte aligned", name);
-  REQUIRE(beta == 0 || beta == 1, AXN_EINVAL, "%s: beta must be 0 or 1", name);
-  REQUIRE(dw_dtype == dtype || dw_dtype == AXN_F32, AXN_EINVAL, "%s: dW must be %s or fp32", name,
-          dtype == AXN_F16 ? "fp16" : "bf16");
-  REQUIRE(N1 % 256 == 0 && N2 % 128 == 0 && K % 128 == 0 && M % 64 == 0, AXN_ESHAPE,
-          "%s: needs N1 %% 256 == 0, N2 %% 128 == 0, K %% 128 == 0, M %% 64 == 0 (got M=%lld, N1=%lld, "
-          "N2=%lld, K=%lld)", name, (long long)M, (long long)N1, (long long)N2, (long long)K);
-  GemmArgs g = {};
-  g.A = (const uint16_t*)dY;  // [M][N1 + N2]: contraction-major, output rows = N1 + N2
-  g.B = (const uint16_t*)X;
-  g.C = dW1;
-  g.C2 = dW2;
-  g.m_split = (int)N1;
-  g.M = (int)(N1 + N2);
-  g.N = (int)K;
-  g.Kc = (int)M;
-  g.lda = lddy;
-  g.ldb = ldx;
-  g.ldc = lddw;
-  g.beta = beta;
-  return dtype == AXN_F16 ? launch_gemm_f16(GEMM_TN, g, AXN_EPI_NONE, dw_dtype == AXN_F32,
-                                            (hipStream_t)stream)
-                          : launch_gemm_bf16(GEMM_TN, g, AXN_EPI_NONE, dw_dtype == AXN_F32,
-                                             (hipStream_t)stream);
-}
-
 size_t axn_dgelu_dbias_workspace_bytes(int64_t M, int64_t N) {
   return dgelu_dbias_workspace_bytes(M, N);
 }
@@ -456,20 +421,6 @@ int axn_swiglu_bwd(const void* dout, const void* gate, const void* up, void* dga
   REQUIRE(aligned16(dout) && aligned16(gate) && aligned16(up) && aligned16(dgate) && aligned16(dup),
           AXN_EALIGN, "%s: pointers must be 16-byte aligned", name);
   return launch_swiglu_bwd(dout, gate, up, dgate, dup, dtype, M, N, ld, ld, (hipStream_t)stream);
-}
-
-int axn_swiglu_bwd_strided(const void* dout, const void* gate, const void* up, void* dgate,
-                           void* dup, int dtype, int64_t M, int64_t N, int64_t ld, int64_t ld_out,
-                           void* stream) {
-  const char* name = "axn_swiglu_bwd_strided";
-  REQUIRE(dout && gate && up && dgate && dup, AXN_EINVAL, "%s: null pointer", name);
-  int rc = check_swiglu(name, dtype, M, N, ld);
-  if (rc) return rc;
-  REQUIRE(ld_out >= N && ld_out % 8 == 0, AXN_EALIGN,
-          "%s: ld_out must be >= N and a multiple of 8", name);
-  REQUIRE(aligned16(dout) && aligned16(gate) && aligned16(up) && aligned16(dgate) && aligned16(dup),
-          AXN_EALIGN, "%s: pointers must be 16-byte aligned", name);
-  return launch_swiglu_bwd(dout, gate, up, dgate, dup, dtype, M, N, ld, ld_out, (hipStream_t)stream);
 }
 
 static int elem_bytes_of(int dtype) { return dtype == AXN_F32 ? 4 : 2; }
@@ -542,7 +493,7 @@ int axn_embedding_renorm(const int64_t* ids, void* W, int dtype, int64_t T, int6
                          size_t workspace_bytes, void* stream) {
   const char* name = "axn_embedding_renorm";
   REQUIRE(W && (ids || T == 0), AXN_EINVAL, "%s: null pointer", name);
-  REQUIRE(dtype == AXN_BF16 || dtype == AXN_F32, AXN_EINVAL, "%s: dtype must be bf16 or fp32",
+  REQUIRE(known_dtype(dtype), AXN_EINVAL, "%s: dtype must be bf16, fp16 or fp32",
           name);
   int rc = check_embedding(name, T, V, H);
   if (rc) return rc;

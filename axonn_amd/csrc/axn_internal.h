@@ -106,12 +106,6 @@ struct GemmArgs {
   // the leading dimensions of A and B.
   const uint16_t* A2;
   int k_first;
-  // Two outputs (launch of one weight gradient for two layers that read the same input):
-  // output rows below m_split go to C, the others to C2 (row - m_split), same ldc and
-  // type.  m_split is a multiple of the tile height, may be <= 0 (all rows in C2) after a
-  // problem has been cut along its rows.  C2 null: one output.
-  void* C2;
-  int m_split;
 };
 
 enum GemmLayout { GEMM_NT = 0, GEMM_NN = 1, GEMM_TN = 2 };

@@ -114,6 +114,23 @@ struct Vec<uint16_t> {
   }
 };
 
+template <>
+struct Vec<_Float16> {
+  static constexpr int N = 8;
+  typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+  static __device__ __forceinline__ void load_cached(const _Float16* p, float (&x)[8]) {
+    const f16x8 v = *(const f16x8*)p;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) x[e] = (float)v[e];
+  }
+  static __device__ __forceinline__ void store(_Float16* p, const float (&x)[8]) {
+    f16x8 v;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] = (_Float16)x[e];
+    *(f16x8*)p = v;
+  }
+};
+
 // Loads VEC consecutive elements as fp32 (VEC = 4 or 8), 16 bytes per instruction
 // where the type allows.  Gradient rows are read once: non-temporal.
 template <int VEC>
@@ -412,6 +429,9 @@ int launch_embedding_renorm(const int64_t* ids, void* W, int dtype, int64_t T, i
   if (dtype == AXN_F32)
     hipLaunchKernelGGL(embedding_renorm_kernel<float>, grid, block, 0, stream, w.row_start,
                        (float*)W, V, H, ldw, max_norm, norm_type);
+  else if (dtype == AXN_F16)
+    hipLaunchKernelGGL(embedding_renorm_kernel<_Float16>, grid, block, 0, stream, w.row_start,
+                       (_Float16*)W, V, H, ldw, max_norm, norm_type);
   else
     hipLaunchKernelGGL(embedding_renorm_kernel<uint16_t>, grid, block, 0, stream, w.row_start,
                        (uint16_t*)W, V, H, ldw, max_norm, norm_type);

@@ -746,11 +746,7 @@ __device__ __forceinline__ void solo_gemm(const GemmArgs& g) {
   } else {
     GemmArgs go = g;  // a split writes its own fp32 partial product
     if (OUT_F32 && g.splits > 1) go.C = (float*)g.C + (int64_t)split * g.M * g.ldc;
-    int out_row = orow;
-    if (g.C2 != nullptr && m0 >= g.m_split) {  // the tile belongs to the second output
-      go.C = g.C2;
-      out_row -= g.m_split;
-    }
+    const int out_row = orow;
 #pragma unroll
     for (int i = 0; i < FRM; ++i)
 #pragma unroll
@@ -988,10 +984,6 @@ int launch_whole(const GemmArgs& g, hipStream_t stream) {
     set_error("gemm_pair: needs whole 128 x 128 tiles, contractions that are multiples of 64 and "
               "operands below 2 GiB (got M=%d, N=%d, K=%d)", g.M, g.N, g.Kc);
     return AXN_ESHAPE;
-  } else if (g.C2 != nullptr) {  // two outputs: the tile kernels only
-    set_error("gemm with two outputs: needs whole 128 x 128 tiles, a contraction that is a multiple "
-              "of 64 and operands below 2 GiB (got M=%d, N=%d, K=%d)", g.M, g.N, g.Kc);
-    return AXN_ESHAPE;
   } else {
     if (whole128) return launch_cfg<128, 128, 2, 2, AK, BKM, EPI, OUT_F32, false, HALF>(g, stream);
     return launch_cfg<128, 128, 2, 2, AK, BKM, EPI, OUT_F32, true, HALF>(g, stream);
@@ -1022,7 +1014,6 @@ int launch_shape(const GemmArgs& g, hipStream_t stream) {
         g2.B = BKM ? g.B + n1 * g.ldb : g.B + n1;
         if (g.B2 != nullptr) g2.B2 = BKM ? g.B2 + n1 * g.ldb : g.B2 + n1;
         g2.C = (char*)g.C + n1 * esz;
-        if (g.C2 != nullptr) g2.C2 = (char*)g.C2 + n1 * esz;
         if (g.bias != nullptr) g2.bias = g.bias + n1;
         if (g.Z != nullptr) g2.Z = g.Z + n1;
         cut = true;
@@ -1033,7 +1024,6 @@ int launch_shape(const GemmArgs& g, hipStream_t stream) {
         g2.A = AK ? g.A + m1 * g.lda : g.A + m1;
         if (g.A2 != nullptr) g2.A2 = AK ? g.A2 + m1 * g.lda : g.A2 + m1;
         g2.C = (char*)g.C + m1 * g.ldc * esz;
-        g2.m_split = g.m_split - (int)m1;  // <= 0: every row of the rest belongs to C2
         if (g.Z != nullptr) g2.Z = g.Z + m1 * g.ldc;
         cut = true;
       }

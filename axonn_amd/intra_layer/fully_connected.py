@@ -68,9 +68,11 @@ def _weight_grad(grad_2d, input_2d, original_weight):
         out_dtype = grad_2d.dtype  # the kernels write dW in the operands' type or in fp32
     if overlap_communication.OVERLAP_REDUCE_SCATTER:
         grad = original_weight.grad
+        # the kernel writes 16-byte vectors: a gradient that is a view at an odd offset
+        # of a flat buffer (axonn/utils.py:11-30 packs without padding) takes the later add
         fusable = (
             grad is not None and grad.is_contiguous() and grad.dtype == out_dtype
-            and grad.numel() == original_weight.numel()
+            and grad.numel() == original_weight.numel() and grad.data_ptr() % 16 == 0
         )
         if fusable:
             ops.gemm_wgrad(grad_2d, input_2d, out=grad, accumulate=True)
@@ -84,36 +86,6 @@ def _weight_grad(grad_2d, input_2d, original_weight):
         return None
     dw = ops.gemm_wgrad(grad_2d, input_2d, out_dtype=out_dtype).reshape(-1)
     return _reduce_scatter(dw, dim=0, process_group=None, overlap_comm=False)
-
-
-def _weight_grad_pair(grad_both, n1, input_2d, weight1, weight2):
-    """`_weight_grad` for two layers that read the same input, as one launch: grad_both
-    holds the two output gradients side by side ([tokens, n1 + n2]).  Falls back to two
-    launches where the pair of gradients cannot be written by one."""
-    out_dtype = weight1.dtype
-    if out_dtype not in (torch.float32, grad_both.dtype):
-        out_dtype = grad_both.dtype
-    if weight2.dtype != weight1.dtype:
-        return (_weight_grad(grad_both[:, :n1], input_2d, weight1),
-                _weight_grad(grad_both[:, n1:], input_2d, weight2))
-    if overlap_communication.OVERLAP_REDUCE_SCATTER:
-        g1, g2 = weight1.grad, weight2.grad
-
-        def fusable(g, w):
-            return g is not None and g.is_contiguous() and g.dtype == out_dtype and g.numel() == w.numel()
-
-        if fusable(g1, weight1) and fusable(g2, weight2):
-            ops.gemm_wgrad_pair(grad_both, input_2d, n1, out1=g1, out2=g2, accumulate=True)
-            return None, None
-        if g1 is None and g2 is None and out_dtype == weight1.dtype:
-            d1, d2 = ops.gemm_wgrad_pair(grad_both, input_2d, n1, out_dtype=out_dtype)
-            weight1.grad, weight2.grad = d1.reshape(weight1.shape), d2.reshape(weight2.shape)
-            return None, None
-        return (_weight_grad(grad_both[:, :n1], input_2d, weight1),
-                _weight_grad(grad_both[:, n1:], input_2d, weight2))
-    d1, d2 = ops.gemm_wgrad_pair(grad_both, input_2d, n1, out_dtype=out_dtype)
-    return (_reduce_scatter(d1.reshape(-1), dim=0, process_group=None, overlap_comm=False),
-            _reduce_scatter(d2.reshape(-1), dim=0, process_group=None, overlap_comm=False))
 
 
 class AsyncLinear(Function):

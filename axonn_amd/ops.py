@@ -49,6 +49,21 @@ def _prep_bf16(t):
     return t, ld
 
 
+def _pad8(t, dim):
+    """`t` with dimension `dim` (0 or 1) of a 2-D tensor zero-padded up to a multiple of 8."""
+    r = (-t.shape[dim]) % 8
+    if r == 0:
+        return t
+    return torch.nn.functional.pad(t, (0, r) if dim == 1 else (0, 0, 0, r))
+
+
+def _ragged16(dtype, *dims):
+    """The 16-bit MFMA kernels move 16-byte vectors: feature counts that are not multiples
+    of 8 (a 10-class head, a vocabulary of 50257) run on operands zero-padded to the next
+    multiple (zeros add nothing to a product) and the result is cut back."""
+    return dtype in _GEMM16 and any(d % 8 for d in dims)
+
+
 # ------------------------------------------------------------------ GEMMs ----
 # 16-bit operand types of the MFMA kernels -> suffix of their entry points
 _GEMM16 = {torch.bfloat16: "", torch.float16: "_f16"}
@@ -86,6 +101,10 @@ def gemm_fwd(x, w, bias=None, activation=None, save_z=False):
     if M == 0:  # an empty batch: nothing to launch (the library takes M >= 1)
         y = torch.empty((0, N), dtype=x.dtype, device=x.device)
         return y, (torch.empty_like(y) if want_z else None)
+    if _ragged16(x.dtype, N, K):
+        bp = None if bias is None else _pad8(bias.reshape(1, -1), 1).reshape(-1)
+        y, z = gemm_fwd(_pad8(x, 1), _pad8(_pad8(w, 1), 0), bp, activation, save_z)
+        return y[:, :N].contiguous(), (None if z is None else z[:, :N].contiguous())
     if x.dtype in _GEMM16:
         x, ldx = _prep_bf16(x)
         w, ldw = _prep_bf16(w)
@@ -121,6 +140,8 @@ def gemm_dgrad(dy, w):
         raise TypeError("the Linear kernels take bf16, fp16 or fp32 operands, got %s" % dy.dtype)
     if M == 0:
         return torch.empty((0, K), dtype=dy.dtype, device=dy.device)
+    if _ragged16(dy.dtype, N, K):
+        return gemm_dgrad(_pad8(dy, 1), _pad8(_pad8(w, 1), 0))[:, :K].contiguous()
     if dy.dtype in _GEMM16:
         dy, lddy = _prep_bf16(dy)
         w, ldw = _prep_bf16(w)
@@ -164,6 +185,17 @@ def gemm_wgrad(dy, x, out=None, accumulate=False, out_dtype=None):
         if out is None:
             return torch.zeros((N, K), dtype=out_dtype, device=dy.device)
         return out if accumulate else out.zero_()
+    if _ragged16(dy.dtype, N, K):
+        # the kernel accumulates into a padded copy of the gradient, which is cut back
+        tmp = None
+        if out is not None:
+            tmp = _pad8(_pad8(out.view(N, K), 1), 0) if accumulate else \
+                torch.empty((N + (-N) % 8, K + (-K) % 8), dtype=out.dtype, device=out.device)
+        full = gemm_wgrad(_pad8(dy, 1), _pad8(x, 1), out=tmp, accumulate=accumulate, out_dtype=out_dtype)
+        if out is None:
+            return full[:N, :K].contiguous()
+        out.view(N, K).copy_(full[:N, :K])
+        return out
     if dy.dtype in _GEMM16:
         if out_dtype not in (dy.dtype, torch.float32):
             raise TypeError("dW must be %s or fp32, got %s" % (dy.dtype, out_dtype))
@@ -198,6 +230,20 @@ def dgelu_dbias(dy, z=None, want_dbias=True, dbias_out=None, accumulate=False):
     _require_gpu(dy, z, dbias_out)
     if dy.dtype not in (torch.bfloat16, torch.float16, torch.float32):
         raise TypeError("bf16, fp16 or fp32 expected, got %s" % dy.dtype)
+    if dy.dim() == 2 and dy.shape[1] % 8:   # ragged width: zero-padded columns, results cut back
+        N = dy.shape[1]
+        acc = None
+        if want_dbias and dbias_out is not None:
+            acc = _pad8(dbias_out.reshape(1, -1), 1).reshape(-1) if accumulate else \
+                torch.empty(N + (-N) % 8, dtype=torch.float32, device=dy.device)
+        dz, db = dgelu_dbias(_pad8(dy, 1), None if z is None else _pad8(z, 1), want_dbias, acc,
+                             accumulate)
+        if db is not None and dbias_out is not None:
+            dbias_out.copy_(db[:N])
+            db = dbias_out
+        elif db is not None:
+            db = db[:N].contiguous()
+        return (dz[:, :N].contiguous() if z is not None else dy), db
     dy, ld = _rows(dy)
     if dy.data_ptr() % 16 or ld % 8:
         dy = dy.contiguous().clone()
@@ -337,6 +383,12 @@ def gemm_dgrad_pair(dy1, w1, dy2, w2):
             dx += gemm_dgrad(dy2, w2)
             return dx
         ld1 = N1
+    if M * ld1 * 2 >= 2 ** 31:
+        # row-strided operands (column blocks of a wider buffer) can span 2 GiB where dense
+        # ones would not: the one-pass kernel addresses an operand with 32-bit offsets
+        dx = gemm_dgrad(dy1, w1)
+        dx += gemm_dgrad(dy2, w2)
+        return dx
     w1, lw1 = _prep_bf16(w1)
     w2, lw2 = _prep_bf16(w2)
     if lw1 != lw2:
@@ -348,69 +400,17 @@ def gemm_dgrad_pair(dy1, w1, dy2, w2):
     return dx
 
 
-def swiglu_bwd(dout, gate, up, side_by_side=False):
-    """(dgate, dup) for out = silu(gate) * up.  With side_by_side the two results are the
-    column blocks of one [M, 2N] buffer, returned as a third value (the layout
-    gemm_wgrad_pair reads)."""
+def swiglu_bwd(dout, gate, up):
+    """(dgate, dup) for out = silu(gate) * up."""
     _require_gpu(dout, gate, up)
     dout, gate, up = _swiglu_operands("swiglu_bwd", [dout, gate, up])
     M, N = gate.shape
-    if side_by_side:
-        # 256 bytes between the rows: with a row stride of exactly 2 N elements the
-        # contraction-strided reads of the weight-gradient kernel fall onto few memory
-        # channels (Llama-3-8B shape: 704 us against 653 us with the gap)
-        ld = 2 * N + 128
-        both = torch.empty((M, ld), dtype=gate.dtype, device=gate.device)[:, :2 * N]
-        dgate, dup = both[:, :N], both[:, N:]
-        if M > 0:
-            nv.call("axn_swiglu_bwd_strided", nv.ptr(dout), nv.ptr(gate), nv.ptr(up), nv.ptr(dgate),
-                    nv.ptr(dup), nv.dtype_code(gate.dtype), M, N, N, ld, nv.current_stream())
-        return dgate, dup, both
     dgate, dup = torch.empty_like(gate), torch.empty_like(up)
     if M == 0:
         return dgate, dup
     nv.call("axn_swiglu_bwd", nv.ptr(dout), nv.ptr(gate), nv.ptr(up), nv.ptr(dgate), nv.ptr(dup),
             nv.dtype_code(gate.dtype), M, N, N, nv.current_stream())
     return dgate, dup
-
-
-def gemm_wgrad_pair_supported(M, N1, N2, K, dtype):
-    """Shapes the one-launch weight gradient of two layers takes (see axn_gemm_wgrad_pair)."""
-    return (dtype in _GEMM16 and M > 0 and M % 64 == 0 and N1 % 256 == 0 and N2 % 128 == 0
-            and K % 128 == 0 and M * (N1 + N2) * 2 < 2 ** 31 and M * K * 2 < 2 ** 31)
-
-
-def gemm_wgrad_pair(dy_both, x, n1, out1=None, out2=None, accumulate=False, out_dtype=None):
-    """dW1 = dy_both[:, :n1]^T X and dW2 = dy_both[:, n1:]^T X in one launch (optionally
-    accumulated into out1 / out2).  Callers check `gemm_wgrad_pair_supported` first."""
-    _require_gpu(dy_both, x, out1, out2)
-    if dy_both.dtype != x.dtype or dy_both.dtype not in _GEMM16:
-        raise TypeError("gemm_wgrad_pair takes bf16 or fp16 operands of one type")
-    M, NN = dy_both.shape
-    K = x.shape[1]
-    n2 = NN - n1
-    if (out1 is None) != (out2 is None):
-        raise ValueError("give both outputs or neither")
-    if out1 is not None:
-        if out1.numel() != n1 * K or out2.numel() != n2 * K or not out1.is_contiguous() \
-                or not out2.is_contiguous() or out1.dtype != out2.dtype:
-            raise ValueError("outputs must be contiguous [n1, K] and [n2, K] tensors of one type")
-        out_dtype = out1.dtype
-    elif accumulate:
-        raise ValueError("accumulate=True needs the outputs")
-    if out_dtype is None:
-        out_dtype = dy_both.dtype
-    if out_dtype not in (dy_both.dtype, torch.float32):
-        raise TypeError("dW must be %s or fp32, got %s" % (dy_both.dtype, out_dtype))
-    dy_both, lddy = _prep_bf16(dy_both)
-    x, ldx = _prep_bf16(x)
-    if out1 is None:
-        out1 = torch.empty((n1, K), dtype=out_dtype, device=x.device)
-        out2 = torch.empty((n2, K), dtype=out_dtype, device=x.device)
-    nv.call("axn_gemm_wgrad_pair", nv.ptr(dy_both), nv.ptr(x), nv.ptr(out1), nv.ptr(out2),
-            nv.dtype_code(x.dtype), M, n1, n2, K, lddy, ldx, K, 1 if accumulate else 0,
-            nv.dtype_code(out_dtype), nv.current_stream())
-    return out1, out2
 
 
 # ------------------------------------------------------------- embedding -----
@@ -488,8 +488,8 @@ def embedding_renorm_(weight, ids, max_norm, norm_type=2.0):
     scaled to max_norm (torch.embedding_renorm_)."""
     _require_gpu(ids, weight)
     _embedding_table("embedding_renorm_", weight)
-    if weight.dtype not in (torch.bfloat16, torch.float32):
-        raise TypeError("embedding_renorm_: bf16 or fp32 table expected, got %s" % weight.dtype)
+    if weight.dtype not in (torch.bfloat16, torch.float16, torch.float32):
+        raise TypeError("embedding_renorm_: bf16, fp16 or fp32 table expected, got %s" % weight.dtype)
     flat = _embedding_ids(ids)
     V, H = weight.shape
     ws, nbytes = _embedding_workspace(flat.numel(), V, weight.device)

@@ -64,6 +64,11 @@ def parse():
     ap.add_argument("--no-library-baseline", action="store_true")
     ap.add_argument("--no-extra-shapes", action="store_true")
     ap.add_argument("--adam-elements", type=float, default=1.3e9)
+    ap.add_argument("--shapes", default=None,
+                    help="comma list of the extra shapes to run (fp16, mlp_shard, skinny, llama_mlp, "
+                         "embedding, small_mlp); default: all")
+    ap.add_argument("--no-main-set", action="store_true",
+                    help="skip the Llama-3-8B-shaped set (value is null): for profiles of the other shapes")
     ap.add_argument("--no-launch-events", action="store_true",
                     help="do not bracket every launch with events (no per-kernel figures)")
     return ap.parse_args()
@@ -119,7 +124,13 @@ def main():
                                     L.dW.data_ptr(), L.M, L.N, L.K, L.N, L.K, L.K, beta, nv.BF16,
                                     stream))
 
-    layers = [Layer(n, M, N, K, i, torch) for i, (n, M, N, K) in enumerate(LLAMA_SET)]
+    selected = None if args.shapes is None else set(args.shapes.split(","))
+
+    def want(name):
+        return not args.no_extra_shapes and (selected is None or name in selected)
+
+    main_set = not args.no_main_set
+    layers = [Layer(n, M, N, K, i, torch) for i, (n, M, N, K) in enumerate(LLAMA_SET)] if main_set else []
     total_flops = sum(L.flops for L in layers)
 
     # One plain copy of known size (1 GiB read + 1 GiB written), outside every timed
@@ -158,13 +169,13 @@ def main():
             timed("dgrad", dgrad, L) if record else dgrad(L)
             timed("wgrad", wgrad, L) if record else wgrad(L)
 
-    for _ in range(args.warmup):
+    for _ in range(args.warmup if main_set else 0):
         step(False)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     # Events bracket the launches of every fourth timed step: recorded on every step they cost
     # 0.7-1.5 % of the step, and the per-kernel averages need no more samples than that.
-    for i in range(args.steps):
+    for i in range(args.steps if main_set else 0):
         step(i % EVENT_EVERY == 0)
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
@@ -172,7 +183,7 @@ def main():
     value = total_flops / (elapsed / args.steps) / 1e12
 
     roofline = None
-    if not args.no_launch_events:
+    if main_set and not args.no_launch_events:
         kinds = {}
         for kind, lst in spans.items():
             tot_ms = sum(s.elapsed_time(e) for s, e, _ in lst)
@@ -210,7 +221,7 @@ def main():
     # operands, same order, timed the same way: a yardstick on this box, not a code path
     # of the library under test.
     library = None
-    if not args.no_library_baseline:
+    if main_set and not args.no_library_baseline:
         def library_step():
             for L in layers:
                 torch.matmul(L.X, L.W.t(), out=L.Y)
@@ -243,7 +254,7 @@ def main():
         return s.elapsed_time(e) / n * 1e-3
 
     shapes = {}
-    if not args.no_extra_shapes:
+    if main_set and want("fp16"):
         # The same step on fp16 operands (the reference's default autocast type): the same
         # kernels with v_mfma_f32_16x16x32_f16.
         half = [(L.X.half(), L.W.half(), L.dY.half(), torch.empty_like(L.Y, dtype=torch.float16),
@@ -268,171 +279,159 @@ def main():
     del layers
     torch.cuda.empty_cache()
     if not args.no_extra_shapes:
-        # 12B-style MLP shard: bias + GELU fused, dW accumulated over 4 micro-batches
-        L = Layer("mlp_shard", 8192, 5120, 2560, 10, torch, bias=True)
-        ws_bytes = lib.axn_dgelu_dbias_workspace_bytes(L.M, L.N)
-        ws = torch.empty(ws_bytes, dtype=torch.uint8, device="cuda")
+        if want("mlp_shard"):
+            # 12B-style MLP shard: bias + GELU fused, dW accumulated over 4 micro-batches
+            L = Layer("mlp_shard", 8192, 5120, 2560, 10, torch, bias=True)
+            ws_bytes = lib.axn_dgelu_dbias_workspace_bytes(L.M, L.N)
+            ws = torch.empty(ws_bytes, dtype=torch.uint8, device="cuda")
 
-        def mlp_shard_step():
-            for mb in range(4):
-                fwd(L, nv.EPI_BIAS_GELU)
-                nv.check(lib.axn_dgelu_dbias(L.dY.data_ptr(), L.Z.data_ptr(), L.dZ.data_ptr(),
-                                             nv.BF16, L.db.data_ptr(), L.M, L.N, L.N,
-                                             1 if mb else 0, ws.data_ptr(), ws_bytes, stream))
-                dgrad(L, L.dZ)
-                wgrad(L, 1 if mb else 0, L.dZ)
+            def mlp_shard_step():
+                for mb in range(4):
+                    fwd(L, nv.EPI_BIAS_GELU)
+                    nv.check(lib.axn_dgelu_dbias(L.dY.data_ptr(), L.Z.data_ptr(), L.dZ.data_ptr(),
+                                                 nv.BF16, L.db.data_ptr(), L.M, L.N, L.N,
+                                                 1 if mb else 0, ws.data_ptr(), ws_bytes, stream))
+                    dgrad(L, L.dZ)
+                    wgrad(L, 1 if mb else 0, L.dZ)
 
-        t = time_loop(mlp_shard_step, max(args.steps // 4, 3)) / 4
-        shapes["mlp_shard_8192x5120x2560_bias_gelu"] = {
-            "us_per_microbatch": round(t * 1e6, 1), "tflops": round(L.flops / t / 1e12, 1),
-            "frac_mfma": round(L.flops / t / 1e12 / PEAK_BF16_TFLOPS, 4)}
-        del L, ws
-        # Skinny shard at the ridge of the roofline: its operands (90 MB a set) would stay in
-        # the 256 MB memory-side cache from one iteration to the next, so the loop walks over
-        # six sets (540 MB) and every GEMM finds its operands in HBM.
-        sets = [Layer("skinny", 512, 8192, 3584, 11 + i, torch) for i in range(6)]
-        L = sets[0]
-        # few output tiles: the entry points that may split the contraction over workgroups
-        ws_bytes = max(lib.axn_gemm_workspace_bytes(op, L.M, L.N, L.K) for op in (0, 1, 2))
-        ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device="cuda")
-        turn = {"i": 0}
+            t = time_loop(mlp_shard_step, max(args.steps // 4, 3)) / 4
+            shapes["mlp_shard_8192x5120x2560_bias_gelu"] = {
+                "us_per_microbatch": round(t * 1e6, 1), "tflops": round(L.flops / t / 1e12, 1),
+                "frac_mfma": round(L.flops / t / 1e12 / PEAK_BF16_TFLOPS, 4)}
+            del L, ws
+        if want("skinny"):
+            # Skinny shard at the ridge of the roofline: its operands (90 MB a set) would stay in
+            # the 256 MB memory-side cache from one iteration to the next, so the loop walks over
+            # six sets (540 MB) and every GEMM finds its operands in HBM.
+            sets = [Layer("skinny", 512, 8192, 3584, 11 + i, torch) for i in range(6)]
+            L = sets[0]
+            # few output tiles: the entry points that may split the contraction over workgroups
+            ws_bytes = max(lib.axn_gemm_workspace_bytes(op, L.M, L.N, L.K) for op in (0, 1, 2))
+            ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device="cuda")
+            turn = {"i": 0}
 
-        def skinny_step():
-            S = sets[turn["i"] % len(sets)]
-            turn["i"] += 1
-            a = (nv.BF16, S.M, S.N, S.K)
-            nv.check(lib.axn_gemm_fwd_ws(S.X.data_ptr(), S.W.data_ptr(), S.Y.data_ptr(), *a,
-                                         S.K, S.K, S.N, ws.data_ptr(), ws_bytes, stream))
-            nv.check(lib.axn_gemm_dgrad_ws(S.dY.data_ptr(), S.W.data_ptr(), S.dX.data_ptr(), *a,
-                                           S.N, S.K, S.K, ws.data_ptr(), ws_bytes, stream))
-            nv.check(lib.axn_gemm_wgrad_ws(S.dY.data_ptr(), S.X.data_ptr(), S.dW.data_ptr(), *a,
-                                           S.N, S.K, S.K, 0, nv.BF16, ws.data_ptr(), ws_bytes, stream))
+            def skinny_step():
+                S = sets[turn["i"] % len(sets)]
+                turn["i"] += 1
+                a = (nv.BF16, S.M, S.N, S.K)
+                nv.check(lib.axn_gemm_fwd_ws(S.X.data_ptr(), S.W.data_ptr(), S.Y.data_ptr(), *a,
+                                             S.K, S.K, S.N, ws.data_ptr(), ws_bytes, stream))
+                nv.check(lib.axn_gemm_dgrad_ws(S.dY.data_ptr(), S.W.data_ptr(), S.dX.data_ptr(), *a,
+                                               S.N, S.K, S.K, ws.data_ptr(), ws_bytes, stream))
+                nv.check(lib.axn_gemm_wgrad_ws(S.dY.data_ptr(), S.X.data_ptr(), S.dW.data_ptr(), *a,
+                                               S.N, S.K, S.K, 0, nv.BF16, ws.data_ptr(), ws_bytes, stream))
 
-        t = time_loop(skinny_step, max(args.steps, 12), w=6)
-        nbytes = 6.0 * (L.M * L.K + L.N * L.K + L.M * L.N)
-        shapes["skinny_512x8192x3584"] = {
-            "us": round(t * 1e6, 1), "tflops": round(L.flops / t / 1e12, 1),
-            "frac_mfma": round(L.flops / t / 1e12 / PEAK_BF16_TFLOPS, 4),
-            "gbs": round(nbytes / t / 1e9, 1), "frac_hbm": round(nbytes / t / 1e9 / PEAK_HBM_GBS, 4),
-            "operands": "cold (6 operand sets in turn)"}
-        del L, ws, sets
-        torch.cuda.empty_cache()
+            t = time_loop(skinny_step, max(args.steps, 12), w=6)
+            nbytes = 6.0 * (L.M * L.K + L.N * L.K + L.M * L.N)
+            shapes["skinny_512x8192x3584"] = {
+                "us": round(t * 1e6, 1), "tflops": round(L.flops / t / 1e12, 1),
+                "frac_mfma": round(L.flops / t / 1e12 / PEAK_BF16_TFLOPS, 4),
+                "gbs": round(nbytes / t / 1e9, 1), "frac_hbm": round(nbytes / t / 1e9 / PEAK_HBM_GBS, 4),
+                "operands": "cold (6 operand sets in turn)"}
+            del L, ws, sets
+            torch.cuda.empty_cache()
 
-        # Llama-3-8B MLP block, 4096 tokens: gate/up/down projections with the one-pass
-        # SwiGLU between them, forward + backward (9 GEMMs, 2 elementwise passes, and
-        # torch's add of the two input-gradient contributions).
-        Mt, H, I = 4096, 4096, 14336
-        g = torch.Generator(device="cuda").manual_seed(12)
-        x = torch.randn(Mt, H, generator=g, device="cuda").bfloat16()
-        wg, wu = ((torch.randn(I, H, generator=g, device="cuda") * 0.02).bfloat16() for _ in range(2))
-        wd = (torch.randn(H, I, generator=g, device="cuda") * 0.02).bfloat16()
-        dy = (torch.randn(Mt, H, generator=g, device="cuda") * 1e-3).bfloat16()
-        bf = dict(dtype=torch.bfloat16, device="cuda")
-        gt, up, act = (torch.empty(Mt, I, **bf) for _ in range(3))
-        dact, dgt, dup = (torch.empty(Mt, I, **bf) for _ in range(3))
-        ldb2 = 2 * I + 128   # 256 bytes between the rows (see ops.swiglu_bwd)
-        dboth = torch.empty(Mt, ldb2, **bf)
-        y, dx1, dx2 = (torch.empty(Mt, H, **bf) for _ in range(3))
-        dwg, dwu, dwd = torch.empty(I, H, **bf), torch.empty(I, H, **bf), torch.empty(H, I, **bf)
-        P = lambda t: t.data_ptr()  # noqa: E731
+        if want("llama_mlp"):
+            # Llama-3-8B MLP block, 4096 tokens: gate/up/down projections with the one-pass
+            # SwiGLU between them, forward + backward (9 GEMMs, 2 elementwise passes, and
+            # torch's add of the two input-gradient contributions).
+            Mt, H, I = 4096, 4096, 14336
+            g = torch.Generator(device="cuda").manual_seed(12)
+            x = torch.randn(Mt, H, generator=g, device="cuda").bfloat16()
+            wg, wu = ((torch.randn(I, H, generator=g, device="cuda") * 0.02).bfloat16() for _ in range(2))
+            wd = (torch.randn(H, I, generator=g, device="cuda") * 0.02).bfloat16()
+            dy = (torch.randn(Mt, H, generator=g, device="cuda") * 1e-3).bfloat16()
+            bf = dict(dtype=torch.bfloat16, device="cuda")
+            gt, up, act = (torch.empty(Mt, I, **bf) for _ in range(3))
+            dact, dgt, dup = (torch.empty(Mt, I, **bf) for _ in range(3))
+            y, dx1, dx2 = (torch.empty(Mt, H, **bf) for _ in range(3))
+            dwg, dwu, dwd = torch.empty(I, H, **bf), torch.empty(I, H, **bf), torch.empty(H, I, **bf)
+            P = lambda t: t.data_ptr()  # noqa: E731
 
-        def gate_up_three_calls():
-            chk = nv.check
-            chk(lib.axn_gemm_fwd(P(x), P(wg), None, P(gt), None, Mt, I, H, H, H, I, nv.EPI_NONE, stream))
-            chk(lib.axn_gemm_fwd(P(x), P(wu), None, P(up), None, Mt, I, H, H, H, I, nv.EPI_NONE, stream))
-            chk(lib.axn_swiglu_fwd(P(gt), P(up), P(act), nv.BF16, Mt, I, I, stream))
+            def gate_up_three_calls():
+                chk = nv.check
+                chk(lib.axn_gemm_fwd(P(x), P(wg), None, P(gt), None, Mt, I, H, H, H, I, nv.EPI_NONE, stream))
+                chk(lib.axn_gemm_fwd(P(x), P(wu), None, P(up), None, Mt, I, H, H, H, I, nv.EPI_NONE, stream))
+                chk(lib.axn_swiglu_fwd(P(gt), P(up), P(act), nv.BF16, Mt, I, I, stream))
 
-        def gate_up_one_launch():
-            nv.check(lib.axn_gemm_swiglu_fwd(P(x), P(wg), P(wu), P(act), P(gt), P(up), nv.BF16, Mt, I, H,
-                                             H, H, I, stream))
+            def gate_up_one_launch():
+                nv.check(lib.axn_gemm_swiglu_fwd(P(x), P(wg), P(wu), P(act), P(gt), P(up), nv.BF16, Mt, I, H,
+                                                 H, H, I, stream))
 
-        def mlp_block_step():
-            chk = nv.check
-            gate_up_one_launch()
-            chk(lib.axn_gemm_fwd(P(act), P(wd), None, P(y), None, Mt, H, I, I, I, H, nv.EPI_NONE, stream))
-            chk(lib.axn_gemm_dgrad(P(dy), P(wd), P(dact), Mt, H, I, H, I, I, stream))
-            chk(lib.axn_gemm_wgrad(P(dy), P(act), P(dwd), Mt, H, I, H, I, I, 0, nv.BF16, stream))
-            # dgate and dup side by side in one [Mt, 2 I] buffer: the layout of the pair kernels
-            chk(lib.axn_swiglu_bwd_strided(P(dact), P(gt), P(up), P(dboth), P(dboth) + 2 * I, nv.BF16, Mt, I,
-                                           I, ldb2, stream))
-            chk(lib.axn_gemm_dgrad_pair(P(dboth), P(wg), P(dboth) + 2 * I, P(wu), P(dx1), nv.BF16, Mt, I, I,
-                                        H, ldb2, H, H, stream))
-            chk(lib.axn_gemm_wgrad_pair(P(dboth), P(x), P(dwg), P(dwu), nv.BF16, Mt, I, I, H, ldb2, H, H, 0,
-                                        nv.BF16, stream))
+            def mlp_block_step():
+                chk = nv.check
+                gate_up_one_launch()
+                chk(lib.axn_gemm_fwd(P(act), P(wd), None, P(y), None, Mt, H, I, I, I, H, nv.EPI_NONE, stream))
+                chk(lib.axn_gemm_dgrad(P(dy), P(wd), P(dact), Mt, H, I, H, I, I, stream))
+                chk(lib.axn_gemm_wgrad(P(dy), P(act), P(dwd), Mt, H, I, H, I, I, 0, nv.BF16, stream))
+                chk(lib.axn_swiglu_bwd(P(dact), P(gt), P(up), P(dgt), P(dup), nv.BF16, Mt, I, I, stream))
+                chk(lib.axn_gemm_dgrad_pair(P(dgt), P(wg), P(dup), P(wu), P(dx1), nv.BF16, Mt, I, I, H, I, H, H,
+                                            stream))
+                chk(lib.axn_gemm_wgrad(P(dgt), P(x), P(dwg), Mt, I, H, I, H, H, 0, nv.BF16, stream))
+                chk(lib.axn_gemm_wgrad(P(dup), P(x), P(dwu), Mt, I, H, I, H, H, 0, nv.BF16, stream))
 
-        t = time_loop(mlp_block_step, max(args.steps // 2, 3))
-        fl = 18.0 * Mt * H * I
-        t_sw = time_loop(lambda: nv.check(lib.axn_swiglu_fwd(P(gt), P(up), P(act), nv.BF16, Mt, I, I, stream)), 10)
-        t_swb = time_loop(lambda: nv.check(lib.axn_swiglu_bwd(P(dact), P(gt), P(up), P(dgt), P(dup), nv.BF16,
-                                                             Mt, I, I, stream)), 10)
-        # the separate calls read the same values as the pair kernels (operand values set the
-        # power draw, and with it the clock)
-        dgt.copy_(dboth[:, :I])
-        dup.copy_(dboth[:, I:2 * I])
+            t = time_loop(mlp_block_step, max(args.steps // 2, 3))
+            fl = 18.0 * Mt * H * I
+            t_sw = time_loop(lambda: nv.check(lib.axn_swiglu_fwd(P(gt), P(up), P(act), nv.BF16, Mt, I, I, stream)), 10)
+            t_swb = time_loop(lambda: nv.check(lib.axn_swiglu_bwd(P(dact), P(gt), P(up), P(dgt), P(dup), nv.BF16,
+                                                                 Mt, I, I, stream)), 10)
 
-        def dgrad_two_calls():
-            nv.check(lib.axn_gemm_dgrad(P(dgt), P(wg), P(dx1), Mt, I, H, I, H, H, stream))
-            nv.check(lib.axn_gemm_dgrad(P(dup), P(wu), P(dx2), Mt, I, H, I, H, H, stream))
-            torch.add(dx1, dx2, out=dx1)
+            def dgrad_two_calls():
+                nv.check(lib.axn_gemm_dgrad(P(dgt), P(wg), P(dx1), Mt, I, H, I, H, H, stream))
+                nv.check(lib.axn_gemm_dgrad(P(dup), P(wu), P(dx2), Mt, I, H, I, H, H, stream))
+                torch.add(dx1, dx2, out=dx1)
 
-        t_dp1 = time_loop(lambda: nv.check(lib.axn_gemm_dgrad_pair(
-            P(dgt), P(wg), P(dup), P(wu), P(dx1), nv.BF16, Mt, I, I, H, I, H, H, stream)), 10)
-        t_dp2 = time_loop(dgrad_two_calls, 10)
+            t_dp1 = time_loop(lambda: nv.check(lib.axn_gemm_dgrad_pair(
+                P(dgt), P(wg), P(dup), P(wu), P(dx1), nv.BF16, Mt, I, I, H, I, H, H, stream)), 10)
+            t_dp2 = time_loop(dgrad_two_calls, 10)
 
-        def wgrad_two_calls():
-            nv.check(lib.axn_gemm_wgrad(P(dgt), P(x), P(dwg), Mt, I, H, I, H, H, 0, nv.BF16, stream))
-            nv.check(lib.axn_gemm_wgrad(P(dup), P(x), P(dwu), Mt, I, H, I, H, H, 0, nv.BF16, stream))
+            t_gu1 = time_loop(gate_up_one_launch, 10)
+            t_gu3 = time_loop(gate_up_three_calls, 10)
+            shapes["llama_mlp_block_4096x4096x14336_swiglu"] = {
+                "us": round(t * 1e6, 1), "tflops": round(fl / t / 1e12, 1),
+                "frac_mfma": round(fl / t / 1e12 / PEAK_BF16_TFLOPS, 4),
+                "gate_up_swiglu_one_launch_us": round(t_gu1 * 1e6, 1),
+                "gate_up_swiglu_three_calls_us": round(t_gu3 * 1e6, 1),
+                "gate_up_dgrad_one_pass_us": round(t_dp1 * 1e6, 1),
+                "gate_up_dgrad_two_calls_and_add_us": round(t_dp2 * 1e6, 1),
+                "swiglu_fwd_gbs": round(6.0 * Mt * I / t_sw / 1e9, 1),
+                "swiglu_bwd_gbs": round(10.0 * Mt * I / t_swb / 1e9, 1)}
+            del x, wg, wu, wd, dy, gt, up, act, dact, dgt, dup, y, dx1, dx2, dwg, dwu, dwd
+            torch.cuda.empty_cache()
 
-        t_wp1 = time_loop(lambda: nv.check(lib.axn_gemm_wgrad_pair(
-            P(dboth), P(x), P(dwg), P(dwu), nv.BF16, Mt, I, I, H, ldb2, H, H, 0, nv.BF16, stream)), 10)
-        t_wp2 = time_loop(wgrad_two_calls, 10)
-        t_gu1 = time_loop(gate_up_one_launch, 10)
-        t_gu3 = time_loop(gate_up_three_calls, 10)
-        shapes["llama_mlp_block_4096x4096x14336_swiglu"] = {
-            "us": round(t * 1e6, 1), "tflops": round(fl / t / 1e12, 1),
-            "frac_mfma": round(fl / t / 1e12 / PEAK_BF16_TFLOPS, 4),
-            "gate_up_swiglu_one_launch_us": round(t_gu1 * 1e6, 1),
-            "gate_up_swiglu_three_calls_us": round(t_gu3 * 1e6, 1),
-            "gate_up_dgrad_one_pass_us": round(t_dp1 * 1e6, 1),
-            "gate_up_dgrad_two_calls_and_add_us": round(t_dp2 * 1e6, 1),
-            "gate_up_wgrad_one_launch_us": round(t_wp1 * 1e6, 1),
-            "gate_up_wgrad_two_calls_us": round(t_wp2 * 1e6, 1),
-            "swiglu_fwd_gbs": round(6.0 * Mt * I / t_sw / 1e9, 1),
-            "swiglu_bwd_gbs": round(10.0 * Mt * I / t_swb / 1e9, 1)}
-        del x, wg, wu, wd, dy, gt, up, act, dact, dgt, dup, dboth, y, dx1, dx2, dwg, dwu, dwd
-        torch.cuda.empty_cache()
+        if want("embedding"):
+            # Embedding of the Llama-3 vocabulary at the largest shape of the reference's own
+            # test of the layer (B 8, S 2048, H 2048, V 128256, fp32): row gather forward and
+            # the dense weight gradient (sort of the token positions + one pass that writes
+            # every row of dW once).
+            Te, He, Ve = 8 * 2048, 2048, 128256
+            g = torch.Generator(device="cuda").manual_seed(13)
+            table = torch.randn(Ve, He, generator=g, device="cuda")
+            ids = torch.randint(0, Ve, (Te,), generator=g, device="cuda")
+            dye = torch.randn(Te, He, generator=g, device="cuda") * 1e-3
+            oute = torch.empty(Te, He, device="cuda")
+            dtab = torch.empty(Ve, He, device="cuda")
+            ws_bytes = lib.axn_embedding_workspace_bytes(Te, Ve)
+            wse = torch.empty(ws_bytes, dtype=torch.uint8, device="cuda")
+            t_ef = time_loop(lambda: nv.check(lib.axn_embedding_fwd(
+                P(ids), P(table), P(oute), nv.F32, Te, Ve, He, He, He, None, stream)), 20)
+            t_eb = time_loop(lambda: nv.check(lib.axn_embedding_bwd(
+                P(ids), P(dye), P(dtab), nv.F32, nv.F32, Te, Ve, He, He, He, -1, 0, 0, P(wse), ws_bytes,
+                stream)), 20)
+            fwd_bytes = 8.0 * Te * He + 8.0 * Te            # rows in, rows out, ids
+            bwd_bytes = 4.0 * Te * He + 4.0 * Ve * He + 8.0 * Te  # dY in, every dW row out, ids
+            shapes["embedding_16384x2048x128256_f32"] = {
+                "fwd_us": round(t_ef * 1e6, 1), "fwd_gbs": round(fwd_bytes / t_ef / 1e9, 1),
+                "bwd_us": round(t_eb * 1e6, 1), "bwd_gbs": round(bwd_bytes / t_eb / 1e9, 1),
+                "bwd_frac_hbm": round(bwd_bytes / t_eb / 1e9 / PEAK_HBM_GBS, 4)}
+            del table, ids, dye, oute, dtab, wse
+            torch.cuda.empty_cache()
 
-        # Embedding of the Llama-3 vocabulary at the largest shape of the reference's own
-        # test of the layer (B 8, S 2048, H 2048, V 128256, fp32): row gather forward and
-        # the dense weight gradient (sort of the token positions + one pass that writes
-        # every row of dW once).
-        Te, He, Ve = 8 * 2048, 2048, 128256
-        g = torch.Generator(device="cuda").manual_seed(13)
-        table = torch.randn(Ve, He, generator=g, device="cuda")
-        ids = torch.randint(0, Ve, (Te,), generator=g, device="cuda")
-        dye = torch.randn(Te, He, generator=g, device="cuda") * 1e-3
-        oute = torch.empty(Te, He, device="cuda")
-        dtab = torch.empty(Ve, He, device="cuda")
-        ws_bytes = lib.axn_embedding_workspace_bytes(Te, Ve)
-        wse = torch.empty(ws_bytes, dtype=torch.uint8, device="cuda")
-        t_ef = time_loop(lambda: nv.check(lib.axn_embedding_fwd(
-            P(ids), P(table), P(oute), nv.F32, Te, Ve, He, He, He, None, stream)), 20)
-        t_eb = time_loop(lambda: nv.check(lib.axn_embedding_bwd(
-            P(ids), P(dye), P(dtab), nv.F32, nv.F32, Te, Ve, He, He, He, -1, 0, 0, P(wse), ws_bytes,
-            stream)), 20)
-        fwd_bytes = 8.0 * Te * He + 8.0 * Te            # rows in, rows out, ids
-        bwd_bytes = 4.0 * Te * He + 4.0 * Ve * He + 8.0 * Te  # dY in, every dW row out, ids
-        shapes["embedding_16384x2048x128256_f32"] = {
-            "fwd_us": round(t_ef * 1e6, 1), "fwd_gbs": round(fwd_bytes / t_ef / 1e9, 1),
-            "bwd_us": round(t_eb * 1e6, 1), "bwd_gbs": round(bwd_bytes / t_eb / 1e9, 1),
-            "bwd_frac_hbm": round(bwd_bytes / t_eb / 1e9 / PEAK_HBM_GBS, 4)}
-        del table, ids, dye, oute, dtab, wse
-        torch.cuda.empty_cache()
-
-        # The reference's CPU-runnable configuration: batch 64, 1024 -> 4096 GELU -> 1024 in
-        # fp32, MSE loss, one Adam step, through the package's modules (launch-bound: a
-        # sanity figure, not a roofline target).
-        shapes["mlp_64x1024x4096x1024_fp32_train_step"] = small_mlp_step(torch, time_loop)
+        if want("small_mlp"):
+            # The reference's CPU-runnable configuration: batch 64, 1024 -> 4096 GELU -> 1024 in
+            # fp32, MSE loss, one Adam step, through the package's modules (launch-bound: a
+            # sanity figure, not a roofline target).
+            shapes["mlp_64x1024x4096x1024_fp32_train_step"] = small_mlp_step(torch, time_loop)
 
     adam = None
     if not args.no_adam:
@@ -440,7 +439,7 @@ def main():
 
     cpu = None
     if not args.no_cpu_baseline:
-        cpu = cpu_baseline(torch)
+        cpu = cpu_baseline(torch) if main_set else None
         if adam is not None:
             adam["cpu_baseline"] = cpu_adam_baseline(torch)
         key = "mlp_64x1024x4096x1024_fp32_train_step"
@@ -449,14 +448,16 @@ def main():
 
     out = {
         "metric": "Linear fwd+bwd TFLOP/s on the Llama-3-8B-shaped set (Adam step GB/s under 'adam')",
-        "value": round(value, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps,
-        "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True,
+        "value": round(value, 2) if main_set else None, "unit": "TFLOP/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4) if main_set else None, "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {
             "workload": "llama3-8b-shaped Linear set, 4096 tokens: qkv 4096->6144, o 4096->4096, "
                         "gate+up 4096->14336 (x2), down 14336->4096; fwd+bwd, bf16 in/out, fp32 "
                         "accumulate, no bias; X~N(0,1), W~N(0,0.02), dY~N(0,1e-3)",
-            "flops_per_step": total_flops, "frac_of_mfma_peak": round(value / PEAK_BF16_TFLOPS, 4),
+            "flops_per_step": total_flops,
+            "frac_of_mfma_peak": round(value / PEAK_BF16_TFLOPS, 4) if main_set else None,
         },
         "roofline": roofline,
         "cpu_baseline": cpu,
@@ -612,10 +613,20 @@ def bench_adam(args, torch, nv, lib, stream, time_loop):
     a = torch.empty(1 << 30, dtype=torch.float32, device="cuda").normal_()
     b = torch.empty_like(a)
     nb = a.numel() * 4.0
+    def probe(kind, src, dst):
+        return time_loop(lambda: nv.check(lib.axn_stream_probe(kind, src.data_ptr(), dst.data_ptr(),
+                                                               int(nb), stream)), 5, 2)
+
     out["hbm_reference_streams"] = {
         "copy_gbs": round(2 * nb / time_loop(lambda: b.copy_(a), 5, 2) / 1e9, 1),
         "elementwise_1r1w_gbs": round(2 * nb / time_loop(lambda: torch.mul(a, 2.0, out=b), 5, 2) / 1e9, 1),
         "fill_gbs": round(nb / time_loop(lambda: b.fill_(1.0), 5, 2) / 1e9, 1),
+        # the library's own plain streams in the optimizer kernels' access pattern
+        # (axn_stream_probe: 16-byte vectors, grid-stride, non-temporal stores)
+        "probe_read_gbs": round(nb / probe(0, a, b) / 1e9, 1),
+        "probe_fill_gbs": round(nb / probe(1, a, b) / 1e9, 1),
+        "probe_copy_gbs": round(2 * nb / probe(2, a, b) / 1e9, 1),
+        "probe_copy_in_place_gbs": round(2 * nb / probe(2, a, a) / 1e9, 1),
         "unit": "GB/s",
     }
     del a, b

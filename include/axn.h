@@ -30,7 +30,7 @@
 extern "C" {
 #endif
 
-#define AXN_ABI_VERSION 9
+#define AXN_ABI_VERSION 10
 
 #if defined(__GNUC__)
 #define AXN_API __attribute__((visibility("default")))
@@ -183,18 +183,6 @@ AXN_API int axn_gemm_dgrad_pair(const void* dY1, const void* W1, const void* dY2
                                 void* dX, int dtype, int64_t M, int64_t N1, int64_t N2, int64_t K,
                                 int64_t lddy, int64_t ldw, int64_t lddx, void* stream);
 
-/* Weight gradients of two layers that read the same input, in one launch:
- *   dW1 (+)= dY[:, :N1]^T X,   dW2 (+)= dY[:, N1:]^T X
- * (two fully_connected.py:147-151 products; one launch covers the tiles of both outputs,
- * so that neither leaves a partly filled last round).  dY [M, N1+N2] holds both output
- * gradients side by side (ld lddy), X [M,K] (ld ldx), dW1 [N1,K] and dW2 [N2,K] (both ld
- * lddw) of dw_dtype (`dtype` or AXN_F32); beta as in axn_gemm_wgrad, for both outputs.
- * Shapes: N1 % 256 == 0, N2 % 128 == 0, K % 128 == 0, M % 64 == 0, operands below 2 GiB
- * (AXN_ESHAPE otherwise: two axn_gemm_wgrad calls). */
-AXN_API int axn_gemm_wgrad_pair(const void* dY, const void* X, void* dW1, void* dW2, int dtype,
-                                int64_t M, int64_t N1, int64_t N2, int64_t K, int64_t lddy,
-                                int64_t ldx, int64_t lddw, int beta, int dw_dtype, void* stream);
-
 /* SwiGLU activation of the Llama MLP, one pass over [M,N]:
  *   out = silu(gate) * up,  silu(x) = x / (1 + exp(-x)).
  * The reference's Llama patch (axonn/models/transformers/modify_llama.py:76-95)
@@ -215,13 +203,6 @@ AXN_API int axn_swiglu_fwd(const void* gate, const void* up, void* out, int dtyp
 AXN_API int axn_swiglu_bwd(const void* dout, const void* gate, const void* up,
                    void* dgate, void* dup, int dtype, int64_t M, int64_t N,
                    int64_t ld, void* stream);
-
-/* The same with a row stride of its own for the two results (ld_out >= N, % 8 == 0): dgate
- * and dup may be the two column blocks of one [M, 2N] buffer, which is the layout
- * axn_gemm_wgrad_pair and axn_gemm_dgrad_pair read. */
-AXN_API int axn_swiglu_bwd_strided(const void* dout, const void* gate, const void* up,
-                                   void* dgate, void* dup, int dtype, int64_t M, int64_t N,
-                                   int64_t ld, int64_t ld_out, void* stream);
 
 /* ------------------------------------------------------------------------
  * Embedding table.  T = tokens, V = rows of the (local) table, H = (local)
@@ -265,7 +246,7 @@ AXN_API int axn_embedding_bwd(const int64_t* ids, const void* dY, void* dW, int 
 /* max_norm of F.embedding (torch.embedding_renorm_, applied to the table in
  * place before the lookup): every row named by at least one id whose
  * norm_type-norm exceeds max_norm is scaled by max_norm / (norm + 1e-7).
- * W [V,H] of dtype AXN_BF16 or AXN_F32; max_norm > 0, norm_type > 0. */
+ * W [V,H] of any axn_dtype; max_norm > 0, norm_type > 0. */
 AXN_API int axn_embedding_renorm(const int64_t* ids, void* W, int dtype, int64_t T,
                          int64_t V, int64_t H, int64_t ldw, float max_norm,
                          float norm_type, void* workspace, size_t workspace_bytes,

@@ -146,23 +146,6 @@ def test_dgrad_pair_argument_errors():
     assert "gemm_pair" in _err()
 
 
-def test_wgrad_pair_and_strided_swiglu_argument_errors():
-    lib = nv.load()
-    f = lib.axn_gemm_wgrad_pair
-    ok = (nv.BF16, 64, 256, 128, 128, 384, 128, 128, 0, nv.BF16, None)
-    assert f(A, A, A, None, *ok) == nv.AXN_EINVAL                         # second output missing
-    assert f(A, A, A, A, nv.F32, *ok[1:]) == nv.AXN_EINVAL
-    assert f(A, A, A, A, nv.BF16, 64, 256, 128, 128, 256, 128, 128, 0, nv.BF16, None) == nv.AXN_EINVAL  # lddy < N1+N2
-    assert f(A, A, A, A, nv.BF16, 64, 256, 128, 128, 384, 128, 128, 2, nv.BF16, None) == nv.AXN_EINVAL  # beta
-    assert f(A, A, A, A, nv.BF16, 64, 256, 128, 128, 384, 128, 128, 0, nv.F16, None) == nv.AXN_EINVAL   # dW type
-    assert f(A, A, A, A, nv.BF16, 64, 128, 128, 128, 256, 128, 128, 0, nv.BF16, None) == nv.AXN_ESHAPE  # N1 % 256
-    assert "N1 % 256 == 0" in _err()
-    b = lib.axn_swiglu_bwd_strided
-    assert b(A, A, A, A, None, nv.BF16, 8, 8, 8, 16, None) == nv.AXN_EINVAL
-    assert b(A, A, A, A, A, nv.BF16, 8, 16, 16, 8, None) == nv.AXN_EALIGN   # ld_out < N
-    assert "ld_out" in _err()
-
-
 def test_embedding_argument_errors():
     lib = nv.load()
     f, b, r = lib.axn_embedding_fwd, lib.axn_embedding_bwd, lib.axn_embedding_renorm
@@ -188,7 +171,7 @@ def test_embedding_argument_errors():
     assert "workspace" in _err()
     assert b(A, A, A, nv.F32, nv.F32, 4, 16, 8, 8, 8, -1, 0, 0, None, big, None) == nv.AXN_EINVAL
     assert r(A, None, nv.F32, 4, 16, 8, 8, 1.0, 2.0, A, big, None) == nv.AXN_EINVAL
-    assert r(A, A, nv.F16, 4, 16, 8, 8, 1.0, 2.0, A, big, None) == nv.AXN_EINVAL
+    assert r(A, A, 7, 4, 16, 8, 8, 1.0, 2.0, A, big, None) == nv.AXN_EINVAL            # unknown dtype
     assert r(A, A, nv.F32, 4, 16, 8, 8, 0.0, 2.0, A, big, None) == nv.AXN_EINVAL
     assert r(A, A, nv.F32, 4, 16, 8, 8, 1.0, -1.0, A, big, None) == nv.AXN_EINVAL
     assert r(A, A, nv.F32, 4, 16, 8, 8, 1.0, 2.0, A, 16, None) == nv.AXN_EINVAL

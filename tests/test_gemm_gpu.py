@@ -189,13 +189,20 @@ def test_unsupported_shapes_raise():
     from axonn_amd import _native as nv
     from axonn_amd import ops
 
-    X = torch.zeros(8, 12, dtype=torch.bfloat16, device="cuda")
-    W = torch.zeros(16, 12, dtype=torch.bfloat16, device="cuda")
+    X = torch.randn(8, 12, device="cuda").bfloat16()
+    W = torch.randn(16, 12, device="cuda").bfloat16()
+    Y = torch.empty(8, 16, dtype=torch.bfloat16, device="cuda")
+    # the entry points take feature counts that are multiples of 8 ...
     with pytest.raises(nv.AxnError, match="multiples of 8") as e:
-        ops.gemm_fwd(X, W)
+        nv.call("axn_gemm_fwd", nv.ptr(X), nv.ptr(W), None, nv.ptr(Y), None, 8, 16, 12, 12, 12, 16, 0,
+                nv.current_stream())
     assert e.value.code == nv.AXN_ESHAPE
     with pytest.raises(nv.AxnError, match="axn_gemm_fwd_f16: N and K must be multiples of 8"):
-        ops.gemm_fwd(X.half(), W.half())
+        nv.call("axn_gemm_fwd_f16", nv.ptr(X), nv.ptr(W), None, nv.ptr(Y), None, 8, 16, 12, 12, 12, 16, 0,
+                nv.current_stream())
+    # ... and the tensor-level wrapper pads other shapes with zeros and cuts the result back
+    y, _ = ops.gemm_fwd(X, W)
+    assert y.shape == (8, 16) and rel(np64(y), np64(X.float() @ W.float().t())) < BF16_TOL
     with pytest.raises(TypeError, match="bf16, fp16 or fp32"):
         ops.gemm_fwd(X.double(), W.double())
     with pytest.raises(TypeError):

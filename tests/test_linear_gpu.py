@@ -214,3 +214,43 @@ def test_two_layer_mlp_step_matches_cpu_path():
     for p, w in zip(model.parameters(), want["params"]):
         assert float((p.detach().cpu().reshape(-1) - w.reshape(-1)).abs().max()) < 2.1e-3
         assert rel(p.reshape(-1), w.reshape(-1)) < 1e-3
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("in_f,out_f", [(64, 10), (50, 24), (27, 13)])
+def test_feature_counts_that_are_not_multiples_of_eight(dtype, in_f, out_f):
+    """A 16-bit layer takes any shape, as the reference's does (a 10-class head, odd widths):
+    forward, input / weight / bias gradients against torch.nn.Linear in float64 on the same
+    rounded parameters, also with the weight gradient accumulated by the kernel."""
+    from axonn_amd.intra_layer import Linear, optimize_communication
+
+    torch.manual_seed(in_f * 100 + out_f)
+    layer = Linear(in_f, out_f).cuda().to(dtype)
+    with torch.no_grad():
+        layer.bias.copy_(torch.randn(out_f) * 0.1)
+    ref = torch.nn.Linear(in_f, out_f).double()
+    with torch.no_grad():
+        ref.weight.copy_(layer.weight.detach().view(out_f, in_f).double().cpu())
+        ref.bias.copy_(layer.bias.detach().double().cpu())
+    x = torch.randn(37, in_f, device="cuda").to(dtype).requires_grad_(True)
+    xr = x.detach().double().cpu().requires_grad_(True)
+    dy = (torch.randn(37, out_f, device="cuda") * 0.1).to(dtype)
+    tol = 1e-2 if dtype == torch.bfloat16 else 2e-3
+
+    def rel(a, b):
+        return float((a.double().cpu().reshape(-1) - b.reshape(-1)).norm() / b.norm())
+
+    for overlap in (False, True):
+        layer.zero_grad()
+        x.grad = None
+        xr.grad = None
+        ref.zero_grad()
+        with optimize_communication(overlap_reduce_scatter=overlap):
+            y = layer(x)
+            y.backward(dy)
+        yr = ref(xr)
+        yr.backward(dy.double().cpu())
+        assert y.shape == (37, out_f)
+        assert rel(y, yr.detach()) < tol and rel(x.grad, xr.grad) < tol
+        assert rel(layer.weight.grad, ref.weight.grad) < tol
+        assert rel(layer.bias.grad, ref.bias.grad) < tol
