@@ -21,7 +21,7 @@ AXN_ELIMIT = -5
 BF16, F16, F32 = 0, 1, 2
 EPI_NONE, EPI_BIAS, EPI_BIAS_GELU, EPI_GELU = 0, 1, 2, 3
 
-ABI_VERSION = 10
+ABI_VERSION = 11
 
 # Every symbol include/axn.h declares: name -> (restype, argtypes)
 _c = ctypes
@@ -58,8 +58,9 @@ SYMBOLS = {
     "axn_gemm_wgrad_f16": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _int, _int,
                                   _vp]),
     "axn_gemm_workspace_bytes": (_sz, [_int, _i64, _i64, _i64]),
-    "axn_gemm_fwd_ws": (_int, [_vp, _vp, _vp, _int, _i64, _i64, _i64, _i64, _i64, _i64, _vp, _sz,
-                               _vp]),
+    "axn_gemm_set_shared_tiles": (_int, [_int]),
+    "axn_gemm_fwd_ws": (_int, [_vp, _vp, _vp, _vp, _vp, _int, _i64, _i64, _i64, _i64, _i64, _i64, _int,
+                               _vp, _sz, _vp]),
     "axn_gemm_dgrad_ws": (_int, [_vp, _vp, _vp, _int, _i64, _i64, _i64, _i64, _i64, _i64, _vp, _sz,
                                  _vp]),
     "axn_gemm_wgrad_ws": (_int, [_vp, _vp, _vp, _int, _i64, _i64, _i64, _i64, _i64, _i64, _int,

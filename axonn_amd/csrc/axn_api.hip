@@ -255,13 +255,17 @@ size_t axn_gemm_workspace_bytes(int op, int64_t M, int64_t N, int64_t K) {
   // dense operands: the leading dimensions are the row lengths
   fill_gemm_args(g, op, nullptr, nullptr, nullptr, M, N, K, op == AXN_GEMM_FWD ? K : N, K,
                  op == AXN_GEMM_FWD ? N : K);
+  if (gemm_streamk_applies(kLayoutOfOp[op], g)) return gemm_streamk_workspace();
   const int s = gemm_splits(kLayoutOfOp[op], g);
   return s > 1 ? (size_t)s * (size_t)g.M * (size_t)g.N * sizeof(float) : 0;
 }
 
+int axn_gemm_set_shared_tiles(int enable) { return gemm_streamk_set_policy(enable); }
+
 static int gemm_ws(const char* name, int op, const void* a, const void* b, void* c, int dtype,
                    int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc, int beta,
-                   int out_dtype, void* workspace, size_t workspace_bytes, void* stream) {
+                   int out_dtype, void* workspace, size_t workspace_bytes, void* stream,
+                   const float* bias = nullptr, void* zsave = nullptr, int epilogue = AXN_EPI_NONE) {
   REQUIRE(dtype == AXN_BF16 || dtype == AXN_F16, AXN_EINVAL, "%s: dtype must be bf16 or fp16", name);
   const bool half = dtype == AXN_F16;
   int rc;
@@ -276,26 +280,43 @@ static int gemm_ws(const char* name, int op, const void* a, const void* b, void*
   GemmArgs g = {};
   fill_gemm_args(g, op, a, b, c, M, N, K, lda, ldb, ldc);
   g.beta = beta;
+  g.bias = bias;
+  g.Z = (uint16_t*)zsave;
   const GemmLayout layout = kLayoutOfOp[op];
-  const int splits = (workspace != nullptr) ? gemm_splits(layout, g) : 1;
+  if (workspace != nullptr && gemm_streamk_applies(layout, g)) {
+    // shares of (tile, stage) units, one workgroup per CU: no partly filled last round
+    const size_t need = gemm_streamk_workspace();
+    REQUIRE(workspace_bytes >= need, AXN_EINVAL,
+            "%s: workspace too small (%zu bytes given, %zu needed)", name, workspace_bytes, need);
+    REQUIRE(aligned16(workspace), AXN_EALIGN, "%s: workspace must be 16-byte aligned", name);
+    return launch_gemm_streamk(layout, g, half, epilogue, out_dtype == AXN_F32, workspace,
+                               (hipStream_t)stream);
+  }
+  bool wide_tiles = false;
+  const int splits =
+      (workspace != nullptr && epilogue == AXN_EPI_NONE) ? gemm_splits(layout, g, &wide_tiles) : 1;
   if (splits > 1) {
     const size_t need = (size_t)splits * (size_t)g.M * (size_t)g.N * sizeof(float);
     REQUIRE(workspace_bytes >= need, AXN_EINVAL,
             "%s: workspace too small (%zu bytes given, %zu needed)", name, workspace_bytes, need);
     REQUIRE(aligned16(workspace), AXN_EALIGN, "%s: workspace must be 16-byte aligned", name);
-    return launch_gemm_splitk(layout, g, half, out_dtype, splits, (float*)workspace,
+    return launch_gemm_splitk(layout, g, half, out_dtype, splits, wide_tiles, (float*)workspace,
                               (hipStream_t)stream);
   }
-  return half ? launch_gemm_f16(layout, g, AXN_EPI_NONE, out_dtype == AXN_F32, (hipStream_t)stream)
-              : launch_gemm_bf16(layout, g, AXN_EPI_NONE, out_dtype == AXN_F32,
-                                 (hipStream_t)stream);
+  return half ? launch_gemm_f16(layout, g, epilogue, out_dtype == AXN_F32, (hipStream_t)stream)
+              : launch_gemm_bf16(layout, g, epilogue, out_dtype == AXN_F32, (hipStream_t)stream);
 }
 
-int axn_gemm_fwd_ws(const void* X, const void* W, void* Y, int dtype, int64_t M, int64_t N,
-                    int64_t K, int64_t ldx, int64_t ldw, int64_t ldy, void* workspace,
-                    size_t workspace_bytes, void* stream) {
-  return gemm_ws("axn_gemm_fwd_ws", AXN_GEMM_FWD, X, W, Y, dtype, M, N, K, ldx, ldw, ldy, 0, dtype,
-                 workspace, workspace_bytes, stream);
+int axn_gemm_fwd_ws(const void* X, const void* W, const float* bias, void* Y, void* Zsave, int dtype,
+                    int64_t M, int64_t N, int64_t K, int64_t ldx, int64_t ldw, int64_t ldy,
+                    int epilogue, void* workspace, size_t workspace_bytes, void* stream) {
+  const char* name = "axn_gemm_fwd_ws";
+  int rc = check_epilogue(name, epilogue, bias);
+  if (rc) return rc;
+  REQUIRE(Zsave == nullptr || aligned16(Zsave), AXN_EALIGN, "%s: Zsave must be 16-byte aligned",
+          name);
+  return gemm_ws(name, AXN_GEMM_FWD, X, W, Y, dtype, M, N, K, ldx, ldw, ldy, 0, dtype, workspace,
+                 workspace_bytes, stream, bias, Zsave, epilogue);
 }
 
 int axn_gemm_dgrad_ws(const void* dY, const void* W, void* dX, int dtype, int64_t M, int64_t N,

@@ -106,6 +106,15 @@ struct GemmArgs {
   // the leading dimensions of A and B.
   const uint16_t* A2;
   int k_first;
+  // Shares of (tile, stage) units instead of whole tiles (launch_gemm_streamk): fp32
+  // partial sums of a tile that two or more workgroups share go through sk_partials (one
+  // slot of 256 x 256 floats per workgroup), handed over with one flag per wave that is
+  // set to sk_token, a value no earlier launch has used; sk_error is set if a flag does
+  // not arrive within the bounded wait.
+  float* sk_partials;
+  unsigned long long* sk_flags;
+  unsigned long long sk_token;
+  int* sk_error;
 };
 
 enum GemmLayout { GEMM_NT = 0, GEMM_NN = 1, GEMM_TN = 2 };
@@ -119,13 +128,22 @@ int launch_gemm_bf16(GemmLayout layout, const GemmArgs& args, int epilogue,
 int launch_gemm_f16(GemmLayout layout, const GemmArgs& args, int epilogue, bool out_f32,
                     hipStream_t stream);
 // Split-contraction variant for problems with few output tiles: the number of splits
-// chosen for an [M x N] output over a contraction of Kc (1 = do not split), and the
+// chosen for an [M x N] output over a contraction of Kc (1 = do not split; *wide_tiles:
+// the parts run on 256 x 128 tiles instead of 128 x 128), and the
 // launch: partial products in fp32 to `ws` (splits * M * N floats), then one pass that
 // adds them in split order, adds the old output if args.beta, and stores args.C in
 // out_dtype.  No epilogue.
-int gemm_splits(GemmLayout layout, const GemmArgs& args);
+int gemm_splits(GemmLayout layout, const GemmArgs& args, bool* wide_tiles = nullptr);
+// One workgroup per CU, each with an equal share of the problem's (256 x 256 tile, 64-deep
+// stage) units (see solo_gemm): whether a problem is run that way, the workspace it needs,
+// and the launch (epilogues as launch_gemm_bf16; ws as sized by gemm_streamk_workspace).
+bool gemm_streamk_applies(GemmLayout layout, const GemmArgs& args);
+int gemm_streamk_set_policy(int policy);   // 0: never, otherwise wherever it can run; returns the old value
+size_t gemm_streamk_workspace();
+int launch_gemm_streamk(GemmLayout layout, const GemmArgs& args, bool half, int epilogue,
+                        bool out_f32, void* ws, hipStream_t stream);
 int launch_gemm_splitk(GemmLayout layout, const GemmArgs& args, bool half, int out_dtype,
-                       int splits, float* ws, hipStream_t stream);
+                       int splits, bool wide_tiles, float* ws, hipStream_t stream);
 
 // C = silu(A B^T) * (A B2^T) in one launch (both weight matrices [N][Kc], K-major), for
 // M % 256 == 0, N % 128 == 0, Kc % 64 == 0 and operands below 2 GiB; AXN_ESHAPE otherwise.

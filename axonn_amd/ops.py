@@ -71,8 +71,9 @@ GEMM_FWD, GEMM_DGRAD, GEMM_WGRAD = 0, 1, 2
 
 
 def _split_workspace(op, M, N, K, device):
-    """Workspace for a GEMM whose contraction the library would split over workgroups
-    (few output tiles), or (None, 0)."""
+    """Workspace for a GEMM whose contraction the library would divide among workgroups
+    (few output tiles, or a tile count that leaves a partly filled last round), or
+    (None, 0)."""
     nbytes = nv.load().axn_gemm_workspace_bytes(op, M, N, K)
     if nbytes == 0:
         return None, 0
@@ -109,13 +110,13 @@ def gemm_fwd(x, w, bias=None, activation=None, save_z=False):
         x, ldx = _prep_bf16(x)
         w, ldw = _prep_bf16(w)
         y = torch.empty((M, N), dtype=x.dtype, device=x.device)
-        ws, ws_bytes = _split_workspace(GEMM_FWD, M, N, K, x.device) if epi == nv.EPI_NONE \
-            else (None, 0)
-        if ws is not None:
-            nv.call("axn_gemm_fwd_ws", nv.ptr(x), nv.ptr(w), nv.ptr(y), nv.dtype_code(x.dtype),
-                    M, N, K, ldx, ldw, N, nv.ptr(ws), ws_bytes, nv.current_stream())
-            return y, None
         z = torch.empty_like(y) if want_z else None
+        ws, ws_bytes = _split_workspace(GEMM_FWD, M, N, K, x.device)
+        if ws is not None:
+            nv.call("axn_gemm_fwd_ws", nv.ptr(x), nv.ptr(w), nv.ptr(bias), nv.ptr(y), nv.ptr(z),
+                    nv.dtype_code(x.dtype), M, N, K, ldx, ldw, N, epi, nv.ptr(ws), ws_bytes,
+                    nv.current_stream())
+            return y, z
         nv.call("axn_gemm_fwd" + _GEMM16[x.dtype], nv.ptr(x), nv.ptr(w), nv.ptr(bias), nv.ptr(y), nv.ptr(z),
                 M, N, K, ldx, ldw, N, epi, nv.current_stream())
     elif x.dtype == torch.float32:

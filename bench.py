@@ -314,8 +314,8 @@ def main():
                 S = sets[turn["i"] % len(sets)]
                 turn["i"] += 1
                 a = (nv.BF16, S.M, S.N, S.K)
-                nv.check(lib.axn_gemm_fwd_ws(S.X.data_ptr(), S.W.data_ptr(), S.Y.data_ptr(), *a,
-                                             S.K, S.K, S.N, ws.data_ptr(), ws_bytes, stream))
+                nv.check(lib.axn_gemm_fwd_ws(S.X.data_ptr(), S.W.data_ptr(), None, S.Y.data_ptr(), None, *a,
+                                             S.K, S.K, S.N, nv.EPI_NONE, ws.data_ptr(), ws_bytes, stream))
                 nv.check(lib.axn_gemm_dgrad_ws(S.dY.data_ptr(), S.W.data_ptr(), S.dX.data_ptr(), *a,
                                                S.N, S.K, S.K, ws.data_ptr(), ws_bytes, stream))
                 nv.check(lib.axn_gemm_wgrad_ws(S.dY.data_ptr(), S.X.data_ptr(), S.dW.data_ptr(), *a,

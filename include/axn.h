@@ -30,7 +30,7 @@
 extern "C" {
 #endif
 
-#define AXN_ABI_VERSION 10
+#define AXN_ABI_VERSION 11
 
 #if defined(__GNUC__)
 #define AXN_API __attribute__((visibility("default")))
@@ -129,23 +129,36 @@ AXN_API int axn_gemm_wgrad_f16(const void* dY, const void* X, void* dW, int64_t 
                        int64_t N, int64_t K, int64_t lddy, int64_t ldx, int64_t lddw,
                        int beta, int dw_dtype, void* stream);
 
-/* Variants of the three GEMMs that may split the contraction over workgroups.
- * A problem with few output tiles (a short batch, a narrow shard) leaves most of
- * the 256 CUs without work; with a workspace the library cuts the contraction
- * into 2, 4 or 8 parts, writes fp32 partial products and adds them in a fixed
- * order in a second pass (deterministic).  No reference counterpart: torch picks
- * such kernels inside its GEMM library.
- *   axn_gemm_workspace_bytes(op, M, N, K): bytes the call below would use for
- *   dense operands, 0 if it would not split.  op, M, N, K as in the call.
- *   axn_gemm_*_ws: arguments as axn_gemm_fwd (epilogue NONE) / _dgrad / _wgrad,
- *   plus dtype (AXN_BF16 or AXN_F16) of the 16-bit operands and results, and
- *   the workspace.  workspace == NULL, or a shape that does not profit: the
- *   call is the plain GEMM. */
+/* Variants of the three GEMMs that may divide the contraction among workgroups, given
+ * a workspace.  No reference counterpart: torch picks such kernels inside its GEMM library.
+ *   - A problem whose count of 256 x 256 output tiles is not a multiple of the CU count
+ *     ends in a round of tiles that leaves CUs idle.  With a workspace, problems of at
+ *     least one tile per CU run as one workgroup per CU with an equal share of the
+ *     (tile, 64-deep stage) units each; a tile shared by two workgroups has its earlier
+ *     stages' fp32 sums handed over through the workspace (flag per wave, the later
+ *     workgroup starts its accumulators from them).  Every sum has an order fixed by the
+ *     launch: results are reproducible bit for bit.  All epilogues.
+ *   - A problem with few output tiles (a short batch, a narrow shard) leaves most CUs
+ *     without work: the contraction is cut into 2, 4 or 8 parts whose fp32 partial
+ *     products a second pass adds in a fixed order (epilogue NONE only).
+ *   axn_gemm_workspace_bytes(op, M, N, K): bytes the call below would use for dense
+ *   operands, 0 if it would do neither.  op, M, N, K as in the call.
+ *   axn_gemm_*_ws: arguments as axn_gemm_fwd / _dgrad / _wgrad, plus dtype (AXN_BF16 or
+ *   AXN_F16) of the 16-bit operands and results, and the workspace (16-byte aligned, used
+ *   by this call alone until it has finished; contents need not be initialised).
+ *   workspace == NULL, or a shape that does not profit: the call is the plain GEMM.
+ *   The first scheme is OFF unless asked for (axn_gemm_set_shared_tiles(1), or
+ *   AXN_GEMM_STREAMK=always in the environment when the library is loaded): on MI355X,
+ *   which runs these kernels power-limited, it measured 0..10 % slower than whole rounds
+ *   plus a second launch for the rest; it takes problems of k x 256 + 128 tiles, k >= 0. */
 typedef enum axn_gemm_op { AXN_GEMM_FWD = 0, AXN_GEMM_DGRAD = 1, AXN_GEMM_WGRAD = 2 } axn_gemm_op;
 AXN_API size_t axn_gemm_workspace_bytes(int op, int64_t M, int64_t N, int64_t K);
-AXN_API int axn_gemm_fwd_ws(const void* X, const void* W, void* Y, int dtype, int64_t M,
-                    int64_t N, int64_t K, int64_t ldx, int64_t ldw, int64_t ldy,
-                    void* workspace, size_t workspace_bytes, void* stream);
+/* Process-wide switch of the shared-tile scheme above; returns the previous setting. */
+AXN_API int axn_gemm_set_shared_tiles(int enable);
+AXN_API int axn_gemm_fwd_ws(const void* X, const void* W, const float* bias, void* Y, void* Zsave,
+                    int dtype, int64_t M, int64_t N, int64_t K, int64_t ldx, int64_t ldw,
+                    int64_t ldy, int epilogue, void* workspace, size_t workspace_bytes,
+                    void* stream);
 AXN_API int axn_gemm_dgrad_ws(const void* dY, const void* W, void* dX, int dtype, int64_t M,
                       int64_t N, int64_t K, int64_t lddy, int64_t ldw, int64_t lddx,
                       void* workspace, size_t workspace_bytes, void* stream);

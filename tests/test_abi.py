@@ -44,9 +44,21 @@ def test_workspace_queries():
     assert lib.axn_dgelu_dbias_workspace_bytes(0, 8) == 0
     # split contraction: fp32 partial products, only for problems with few 128 x 128 tiles
     assert lib.axn_gemm_workspace_bytes(1, 512, 8192, 3584) == 4 * 512 * 3584 * 4   # dgrad, 112 tiles
-    assert lib.axn_gemm_workspace_bytes(0, 512, 8192, 3584) == 0                    # fwd, 256 tiles: no gain
-    assert lib.axn_gemm_workspace_bytes(2, 512, 8192, 3584) == 0                    # wgrad, 1792 tiles
-    assert lib.axn_gemm_workspace_bytes(0, 4096, 4096, 4096) == 0
+    assert lib.axn_gemm_workspace_bytes(0, 512, 8192, 3584) == 2 * 512 * 8192 * 4   # fwd, 128 tiles of 256 x 128, 2 parts
+    assert lib.axn_gemm_workspace_bytes(2, 512, 8192, 3584) == 0                    # wgrad, 448 large tiles
+    # tiles shared by two workgroups (k x 256 + 128 tiles): off unless switched on
+    shares = 16384 + 256 * 256 * 256 * 4    # flags + one slot of fp32 partial sums per workgroup
+    assert lib.axn_gemm_workspace_bytes(0, 4096, 6144, 4096) == 0
+    old = lib.axn_gemm_set_shared_tiles(1)
+    try:
+        assert old == 0
+        assert lib.axn_gemm_workspace_bytes(0, 4096, 14336, 4096) == shares         # 896 = 3 x 256 + 128 tiles
+        assert lib.axn_gemm_workspace_bytes(0, 4096, 6144, 4096) == shares          # 384: one round and a half
+        assert lib.axn_gemm_workspace_bytes(0, 4096, 4096, 4096) == 0               # whole rounds
+        assert lib.axn_gemm_workspace_bytes(1, 8192, 5120, 2560) == 0               # 320 tiles: not half a round
+    finally:
+        assert lib.axn_gemm_set_shared_tiles(old) == 1
+    assert lib.axn_gemm_workspace_bytes(0, 4096, 4096, 4096) == 0                   # one whole round
     assert lib.axn_gemm_workspace_bytes(0, 100, 128, 1024) == 0                     # ragged: no split
     assert lib.axn_gemm_workspace_bytes(0, 128, 128, 512) == 0                      # contraction too short
     assert lib.axn_gemm_workspace_bytes(0, 128, 128, 4096) == 8 * 128 * 128 * 4
@@ -99,7 +111,8 @@ def test_gemm_argument_errors():
               None) == nv.AXN_EALIGN
     assert ws(A, None, A, nv.BF16, 512, 8192, 3584, 8192, 3584, 3584, A, 1 << 30, None) == nv.AXN_EINVAL
     assert lib.axn_gemm_wgrad_ws(A, A, A, nv.BF16, 8, 8, 8, 8, 8, 8, 0, nv.F16, A, 64, None) == nv.AXN_EINVAL
-    assert lib.axn_gemm_fwd_ws(A, A, A, nv.F16, 8, 12, 8, 8, 8, 16, None, 0, None) == nv.AXN_ESHAPE
+    assert lib.axn_gemm_fwd_ws(A, A, None, A, None, nv.F16, 8, 12, 8, 8, 8, 16, 0, None, 0, None) == nv.AXN_ESHAPE
+    assert lib.axn_gemm_fwd_ws(A, A, None, A, None, nv.F16, 8, 16, 8, 8, 8, 16, 1, None, 0, None) == nv.AXN_EINVAL  # bias missing
     assert lib.axn_gemm_fwd_f32(A, None, None, A, None, 4, 4, 4, 0, None) == nv.AXN_EINVAL
     assert lib.axn_gemm_wgrad_f32(A, A, A, 4, 4, 4, 3, None) == nv.AXN_EINVAL
     assert lib.axn_gemm_dgrad_f32(ctypes.c_void_p(0x1002), A, A, 4, 4, 4, None) == nv.AXN_EALIGN

@@ -454,8 +454,8 @@ def test_split_contraction_output_rows_may_be_strided():
     nbytes = nv.load().axn_gemm_workspace_bytes(0, M, N, K)
     assert nbytes > 0
     ws = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
-    nv.call("axn_gemm_fwd_ws", nv.ptr(X), nv.ptr(W), nv.ptr(big), nv.BF16, M, N, K, K, K, N + 64,
-            nv.ptr(ws), nbytes, nv.current_stream())
+    nv.call("axn_gemm_fwd_ws", nv.ptr(X), nv.ptr(W), None, nv.ptr(big), None, nv.BF16, M, N, K, K, K, N + 64,
+            0, nv.ptr(ws), nbytes, nv.current_stream())
     want = (X.float() @ W.float().t())
     assert rel(np64(big[:, :N]), np64(want)) < BF16_TOL
     assert not big[:, N:].any()
