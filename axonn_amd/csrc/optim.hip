@@ -33,10 +33,7 @@ namespace {
 #define AXN_SCAN_CHUNK 65536
 #endif
 #ifndef AXN_ADAM_CHUNK
-#define AXN_ADAM_CHUNK 8192
-#endif
-#ifndef AXN_ADAM_UNROLL
-#define AXN_ADAM_UNROLL 1
+#define AXN_ADAM_CHUNK 16384
 #endif
 #ifndef AXN_ADAM_NT_G
 #define AXN_ADAM_NT_G 1
@@ -45,23 +42,22 @@ namespace {
 #define AXN_ADAM_NT_STORE 1
 #endif
 #ifndef AXN_ADAM_NT_LOAD
-#define AXN_ADAM_NT_LOAD 0
+#define AXN_ADAM_NT_LOAD 1
 #endif
 #ifndef AXN_ADAM_WGS_PER_CU
-#define AXN_ADAM_WGS_PER_CU 4096
+#define AXN_ADAM_WGS_PER_CU 65536
 #endif
 
 constexpr int MT_MAX = 64;         // tensors per launch
 constexpr int MT_THREADS = 256;    // threads per workgroup
 constexpr int MT_VEC = 8;          // elements per lane per step
 // Elements per workgroup.  The read-only scan streams best in long runs with
-// non-temporal loads; the read-modify-write update does best with short runs,
-// cached loads, high occupancy (one vector per lane in flight) and
-// non-temporal stores.  Both measured on MI355X.
+// non-temporal loads; the read-modify-write update does best in the finest grain (one
+// 4-element vector per lane, see mt_adam_kernel).  Both measured on MI355X.
 constexpr int SCAN_CHUNK = AXN_SCAN_CHUNK;
 constexpr int ADAM_CHUNK = AXN_ADAM_CHUNK;
 constexpr int SCALE_CHUNK = 16384;
-constexpr int ADAM_UNROLL = AXN_ADAM_UNROLL;  // independent vectors per lane in flight
+constexpr int ADAM_VEC = 4;                   // elements per lane of the update kernel
 
 // Memory access policies, compile-time per call site.
 template <bool NT, typename T>
@@ -386,13 +382,64 @@ __device__ __forceinline__ void adam_math(float g, float& p, float& m, float& v,
   asm volatile("" : "+v"(p));
 }
 
-// One workgroup per chunk up to a cap of AXN_ADAM_WGS_PER_CU workgroups per CU, beyond
-// which workgroups walk the chunk list with a stride of the grid size.  The cap is far
-// above what the optimizer configurations reach, on purpose: measured on MI355X (1.3e9
-// elements, 64 tensors) a grid of one workgroup per chunk, which the dispatcher hands out
-// in order so that the chip works on one compact window of every stream, updates at
-// 5.23 TB/s; 256 workgroups per CU at 5.18, 64 at 5.08, 4 to 16 at 5.05 - workgroups
-// that stay resident drift apart and the window widens.
+// 4 consecutive low-precision elements from an address aligned to their 4 (8 or 16 bytes).
+typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
+template <int DT, bool NT>
+__device__ __forceinline__ void load4(const void* base, int64_t i, typename Lowp<DT>::raw (&r)[4]) {
+  typedef typename Lowp<DT>::raw raw;
+  const raw* p = (const raw*)base + i;
+  if (sizeof(raw) == 2) {
+    const u32x2 w = ld<NT>((const u32x2*)p);
+#pragma unroll
+    for (int e = 0; e < 2; ++e) {
+      r[2 * e] = (raw)(w[e] & 0xFFFFu);
+      r[2 * e + 1] = (raw)(w[e] >> 16);
+    }
+  } else {
+    const u32x4 w = ld<NT>((const u32x4*)p);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) r[e] = (raw)w[e];
+  }
+}
+template <int DT, bool NT>
+__device__ __forceinline__ void store4(void* base, int64_t i, const typename Lowp<DT>::raw (&r)[4]) {
+  typedef typename Lowp<DT>::raw raw;
+  raw* p = (raw*)base + i;
+  if (sizeof(raw) == 2) {
+    u32x2 w;
+#pragma unroll
+    for (int e = 0; e < 2; ++e) w[e] = (uint32_t)r[2 * e] | ((uint32_t)r[2 * e + 1] << 16);
+    st<NT>(w, (u32x2*)p);
+  } else {
+    u32x4 w;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) w[e] = (uint32_t)r[e];
+    st<NT>(w, (u32x4*)p);
+  }
+}
+
+// The chunk's tensor without a chain of dependent loads: lane i compares chunk_start[i + 1]
+// with the chunk index, and the number of tensors that end at or before it is the answer.
+__device__ __forceinline__ int find_tensor_by_vote(const MtTable& t, int block) {
+  const int lane = threadIdx.x & 63;
+  const bool before = lane < t.n && t.chunk_start[lane + 1] <= block;
+  // the same in every lane and wave: as a scalar, so that the tensor's fields are scalar loads
+  return __builtin_amdgcn_readfirstlane(__builtin_popcountll(__ballot(before)));
+}
+
+// What the update's rate hangs on, measured on MI355X in a stand-alone harness with this
+// access pattern (1.3e9 elements, 64 tensors): one 4-element vector per lane and trip (16
+// bytes of each fp32 stream, 8 of each 16-bit one) with every access non-temporal gives
+// 5.69 TB/s - 8 elements per lane 5.36, and 4.94 with cached loads of the state; and one
+// workgroup per chunk, handed out by the dispatcher in order so that the chip works on one
+// compact window of every stream - workgroups that stay resident and stride over the chunks
+// give 5.26 at 1024 per CU and 5.02 at 256.  128, 512 or 1024 lanes per workgroup: 5.29 to
+// 5.57.  The chunk size is free (1 K to 32 K elements, within 1 %); 16 K keeps the launch
+// of a step that is skipped on overflow at 80 K workgroups that return at once.  Where the
+// five streams lie relative to one another matters as much as the kernel: the same code
+// object measures 5.2 to 5.7 TB/s from one process and machine to the next.  Beyond
+// AXN_ADAM_WGS_PER_CU workgroups per CU (far above what the optimizer configurations
+// reach) a workgroup takes several chunks.
 template <int GDT, int PDT, bool HAS_PLOW>
 __global__ void __launch_bounds__(MT_THREADS)
     mt_adam_kernel(const MtTable tab, const AdamScalars s,
@@ -405,9 +452,8 @@ __global__ void __launch_bounds__(MT_THREADS)
     gmul = scan->clip_coef;
   }
   const int tid = threadIdx.x;
-  int t = find_tensor(tab, blockIdx.x);
   for (int b = blockIdx.x; b < total_chunks; b += gridDim.x) {
-    while (tab.chunk_start[t + 1] <= b) ++t;  // uniform: chunk ids only grow
+    const int t = find_tensor_by_vote(tab, b);
     const int c = b - tab.chunk_start[t];
     const Range rg = chunk_range(tab, t, c);
     const void* g = tab.g[t];
@@ -427,57 +473,30 @@ __global__ void __launch_bounds__(MT_THREADS)
 
     if (tab.vec_ok[t]) {
       if (c == 0 && tid < tab.head[t]) one(tid);
-      const int64_t nvec = (rg.end - rg.begin) / MT_VEC;
-      int64_t i = tid;
-      // Main body: ADAM_UNROLL independent vectors per lane in flight.
-      for (; i + (ADAM_UNROLL - 1) * MT_THREADS < nvec; i += ADAM_UNROLL * MT_THREADS) {
-        graw gr[ADAM_UNROLL][8];
-        float pp[ADAM_UNROLL][8], mm[ADAM_UNROLL][8], vv[ADAM_UNROLL][8];
+      const int nvec = (int)((rg.end - rg.begin) / ADAM_VEC);
+      for (int i = tid; i < nvec; i += MT_THREADS) {
+        const int64_t e0 = rg.begin + (int64_t)i * ADAM_VEC;
+        graw gr[4];
+        praw pl[4];
+        load4<GDT, AXN_ADAM_NT_G != 0>(g, e0, gr);
+        f32x4 pp = ld<AXN_ADAM_NT_LOAD != 0>((const f32x4*)(p + e0));
+        f32x4 mm = ld<AXN_ADAM_NT_LOAD != 0>((const f32x4*)(m + e0));
+        f32x4 vv = ld<AXN_ADAM_NT_LOAD != 0>((const f32x4*)(v + e0));
 #pragma unroll
-        for (int u = 0; u < ADAM_UNROLL; ++u) {
-          const int64_t e0 = rg.begin + (i + u * MT_THREADS) * MT_VEC;
-          load8<GDT, AXN_ADAM_NT_G != 0>(g, e0, gr[u]);
-          loadf8<AXN_ADAM_NT_LOAD != 0>(p + e0, pp[u]);
-          loadf8<AXN_ADAM_NT_LOAD != 0>(m + e0, mm[u]);
-          loadf8<AXN_ADAM_NT_LOAD != 0>(v + e0, vv[u]);
+        for (int e = 0; e < 4; ++e) {
+          float pe = pp[e], me = mm[e], ve = vv[e];
+          adam_math(Lowp<GDT>::to_float(gr[e]), pe, me, ve, s, gmul);
+          pp[e] = pe;
+          mm[e] = me;
+          vv[e] = ve;
+          if (HAS_PLOW) pl[e] = Lowp<PDT>::from_float(pe);
         }
-#pragma unroll
-        for (int u = 0; u < ADAM_UNROLL; ++u) {
-          const int64_t e0 = rg.begin + (i + u * MT_THREADS) * MT_VEC;
-          praw pl[8];
-#pragma unroll
-          for (int e = 0; e < 8; ++e) {
-            adam_math(Lowp<GDT>::to_float(gr[u][e]), pp[u][e], mm[u][e], vv[u][e], s, gmul);
-            if (HAS_PLOW) pl[e] = Lowp<PDT>::from_float(pp[u][e]);
-          }
-          storef8<AXN_ADAM_NT_STORE != 0>(p + e0, pp[u]);
-          storef8<AXN_ADAM_NT_STORE != 0>(m + e0, mm[u]);
-          storef8<AXN_ADAM_NT_STORE != 0>(v + e0, vv[u]);
-          if (HAS_PLOW) store8<PDT, AXN_ADAM_NT_STORE != 0>(plow, e0, pl);
-        }
+        st<AXN_ADAM_NT_STORE != 0>(pp, (f32x4*)(p + e0));
+        st<AXN_ADAM_NT_STORE != 0>(mm, (f32x4*)(m + e0));
+        st<AXN_ADAM_NT_STORE != 0>(vv, (f32x4*)(v + e0));
+        if (HAS_PLOW) store4<PDT, AXN_ADAM_NT_STORE != 0>(plow, e0, pl);
       }
-      if (ADAM_UNROLL > 1) {
-        for (; i < nvec; i += MT_THREADS) {
-          const int64_t e0 = rg.begin + i * MT_VEC;
-          graw gr[8];
-          float pp[8], mm[8], vv[8];
-          praw pl[8];
-          load8<GDT, AXN_ADAM_NT_G != 0>(g, e0, gr);
-          loadf8<AXN_ADAM_NT_LOAD != 0>(p + e0, pp);
-          loadf8<AXN_ADAM_NT_LOAD != 0>(m + e0, mm);
-          loadf8<AXN_ADAM_NT_LOAD != 0>(v + e0, vv);
-#pragma unroll
-          for (int e = 0; e < 8; ++e) {
-            adam_math(Lowp<GDT>::to_float(gr[e]), pp[e], mm[e], vv[e], s, gmul);
-            if (HAS_PLOW) pl[e] = Lowp<PDT>::from_float(pp[e]);
-          }
-          storef8<AXN_ADAM_NT_STORE != 0>(p + e0, pp);
-          storef8<AXN_ADAM_NT_STORE != 0>(m + e0, mm);
-          storef8<AXN_ADAM_NT_STORE != 0>(v + e0, vv);
-          if (HAS_PLOW) store8<PDT, AXN_ADAM_NT_STORE != 0>(plow, e0, pl);
-        }
-      }
-      const int64_t tail = rg.begin + nvec * MT_VEC;
+      const int64_t tail = rg.begin + (int64_t)nvec * ADAM_VEC;
       if (tail + tid < rg.end) one(tail + tid);
     } else {
       const int64_t b0 = (c == 0) ? 0 : rg.begin;
@@ -523,30 +542,28 @@ __global__ void __launch_bounds__(MT_THREADS)
 }
 
 // ------------------------------------------------------------- probes ------
-// Plain streaming kernels in the optimizer's access pattern (16-byte vectors, grid-stride,
-// non-temporal stores): what the memory system gives a read, a fill and a copy on this
-// GPU, measured beside the optimizer step by benchmarks.
+// Plain streaming kernels in the pattern that measured fastest for a copy on MI355X (one
+// 16-byte vector per lane, one workgroup per 4 KiB, non-temporal loads and stores: 6.6 TB/s
+// against 5.6..5.8 with four vectors per lane and 4.7..5.2 with resident workgroups that
+// stride): what the memory system gives a read, a fill and a copy on this GPU, measured
+// beside the optimizer step by benchmarks.
 __global__ void __launch_bounds__(MT_THREADS)
     probe_read_kernel(const f32x4* __restrict__ src, int64_t nvec, float* sink) {
-  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-  for (int64_t i = (int64_t)blockIdx.x * MT_THREADS + threadIdx.x; i < nvec;
-       i += (int64_t)gridDim.x * MT_THREADS)
-    acc += ld<true>(src + i);
-  // never true for finite data: keeps the loads alive without a store per lane
-  if (acc[0] + acc[1] + acc[2] + acc[3] == 1.2345678e38f) *sink = acc[0];
+  const int64_t i = (int64_t)blockIdx.x * MT_THREADS + threadIdx.x;
+  if (i >= nvec) return;
+  const f32x4 x = ld<true>(src + i);
+  // never true for finite data: keeps the load alive without a store per lane
+  if (x[0] + x[1] + x[2] + x[3] == 1.2345678e38f) *sink = x[0];
 }
 __global__ void __launch_bounds__(MT_THREADS)
     probe_fill_kernel(f32x4* __restrict__ dst, int64_t nvec) {
-  const f32x4 x = {0.f, 0.f, 0.f, 0.f};
-  for (int64_t i = (int64_t)blockIdx.x * MT_THREADS + threadIdx.x; i < nvec;
-       i += (int64_t)gridDim.x * MT_THREADS)
-    st<true>(x, dst + i);
+  const int64_t i = (int64_t)blockIdx.x * MT_THREADS + threadIdx.x;
+  if (i < nvec) dst[i] = f32x4{0.f, 0.f, 0.f, 0.f};
 }
 __global__ void __launch_bounds__(MT_THREADS)
     probe_copy_kernel(const f32x4* src, f32x4* dst, int64_t nvec) {
-  for (int64_t i = (int64_t)blockIdx.x * MT_THREADS + threadIdx.x; i < nvec;
-       i += (int64_t)gridDim.x * MT_THREADS)
-    st<true>(ld<false>(src + i), dst + i);
+  const int64_t i = (int64_t)blockIdx.x * MT_THREADS + threadIdx.x;
+  if (i < nvec) st<true>(ld<true>(src + i), dst + i);
 }
 
 // ------------------------------------------------------------- host side ----
@@ -852,10 +869,11 @@ int launch_mt_adam(const void* const* h_g, void* const* h_p, void* const* h_m,
 int launch_stream_probe(int kind, const void* src, void* dst, size_t bytes, hipStream_t stream) {
   const int64_t nvec = (int64_t)(bytes / 16);
   if (nvec == 0) return AXN_OK;
-  // enough workgroups to keep every CU's memory pipeline full, few enough to stay resident
-  long long blocks = (nvec + MT_THREADS - 1) / MT_THREADS;
-  const long long cap = (long long)cu_count() * 32;
-  if (blocks > cap) blocks = cap;
+  const long long blocks = (nvec + MT_THREADS - 1) / MT_THREADS;
+  if (blocks > 0x7fffffffLL) {
+    set_error("axn_stream_probe: at most %lld bytes per call", 0x7fffffffLL * MT_THREADS * 16);
+    return AXN_ELIMIT;
+  }
   const dim3 grid((unsigned)blocks), block(MT_THREADS);
   switch (kind) {
     case AXN_PROBE_READ:
