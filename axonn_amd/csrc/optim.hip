@@ -11,13 +11,14 @@
 //
 // Addressing.  The tensors of one launch (at most MT_MAX) travel in the kernel
 // argument block: pointers, sizes and a prefix sum of per-tensor chunk counts.
-// Workgroup b finds its tensor by binary search in that prefix sum (scalar
-// loads from the argument block) and owns one chunk of consecutive elements of it.
+// Workgroup b finds its tensor in that prefix sum with scalar loads from the argument
+// block (binary search; the update kernel's two-step search is described there) and owns
+// one chunk of consecutive elements of it.
 // Tensors are views into flat buffers at arbitrary element offsets
 // (axonn/utils.py:11-30), so each tensor starts with a scalar "head" of up to 63
 // elements after which every pointer of the tensor is 16-byte aligned (and on a
-// cache line when the buffers allow it); the
-// body is then moved as 16-byte vectors, 8 elements per lane per step.  A
+// cache line when the buffers allow it); the body is then moved as 16-byte vectors
+// (8-byte ones for 16-bit streams of the update kernel).  A
 // tensor whose pointers cannot be aligned by one common head is processed with
 // scalar accesses.
 #include "axn_internal.h"
@@ -32,8 +33,14 @@ namespace {
 #ifndef AXN_SCAN_CHUNK
 #define AXN_SCAN_CHUNK 65536
 #endif
+#ifndef AXN_ADAM_THREADS
+#define AXN_ADAM_THREADS 64
+#endif
 #ifndef AXN_ADAM_CHUNK
-#define AXN_ADAM_CHUNK 16384
+#define AXN_ADAM_CHUNK (AXN_ADAM_THREADS * 4)
+#endif
+#ifndef AXN_ADAM_LDS
+#define AXN_ADAM_LDS 16384
 #endif
 #ifndef AXN_ADAM_NT_G
 #define AXN_ADAM_NT_G 1
@@ -43,9 +50,6 @@ namespace {
 #endif
 #ifndef AXN_ADAM_NT_LOAD
 #define AXN_ADAM_NT_LOAD 1
-#endif
-#ifndef AXN_ADAM_WGS_PER_CU
-#define AXN_ADAM_WGS_PER_CU 65536
 #endif
 
 constexpr int MT_MAX = 64;         // tensors per launch
@@ -58,6 +62,10 @@ constexpr int SCAN_CHUNK = AXN_SCAN_CHUNK;
 constexpr int ADAM_CHUNK = AXN_ADAM_CHUNK;
 constexpr int SCALE_CHUNK = 16384;
 constexpr int ADAM_VEC = 4;                   // elements per lane of the update kernel
+constexpr int ADAM_THREADS = AXN_ADAM_THREADS;  // lanes per workgroup of the update kernel
+// LDS the update kernel reserves per workgroup and never touches: it bounds the
+// workgroups that are resident on a CU (160 KB per CU), see mt_adam_kernel.
+constexpr int ADAM_LDS = AXN_ADAM_LDS;
 
 // Memory access policies, compile-time per call site.
 template <bool NT, typename T>
@@ -83,8 +91,8 @@ struct MtTable {
   void* plow[MT_MAX];
   int64_t size[MT_MAX];
   int32_t chunk_start[MT_MAX + 1];  // prefix sum of chunks per tensor
-  uint8_t head[MT_MAX];             // scalar elements before the aligned body
-  uint8_t vec_ok[MT_MAX];           // 0: scalar accesses only
+  int32_t meta[MT_MAX];             // bits 0-7: scalar elements before the aligned body;
+                                    // bit 8: vector accesses allowed
   int32_t n;
   int32_t chunk;                    // elements per workgroup (multiple of MT_VEC)
 };
@@ -95,6 +103,9 @@ struct ScanPartial {
   int32_t nonfinite;
   int32_t pad;
 };
+
+__device__ __forceinline__ int head_of(const MtTable& t, int i) { return t.meta[i] & 0xff; }
+__device__ __forceinline__ bool vec_ok_of(const MtTable& t, int i) { return (t.meta[i] & 0x100) != 0; }
 
 __device__ __forceinline__ int find_tensor(const MtTable& t, int block) {
   int lo = 0, hi = t.n;  // chunk_start[lo] <= block < chunk_start[hi]
@@ -199,7 +210,7 @@ struct Range {
   int64_t begin, end;
 };
 __device__ __forceinline__ Range chunk_range(const MtTable& tab, int t, int c) {
-  const int64_t head = tab.head[t];
+  const int64_t head = head_of(tab, t);
   Range r;
   r.begin = head + (int64_t)c * tab.chunk;
   r.end = r.begin + tab.chunk;
@@ -252,8 +263,8 @@ __global__ void __launch_bounds__(MT_THREADS)
     sm += f;
     sq += norm_term<MODE>(f * inv_scale, norm_type);
   };
-  if (tab.vec_ok[t]) {
-    if (c == 0 && tid < tab.head[t]) one(((const raw*)g)[tid]);
+  if (vec_ok_of(tab, t)) {
+    if (c == 0 && tid < head_of(tab, t)) one(((const raw*)g)[tid]);
     const int64_t nvec = (rg.end - rg.begin) / MT_VEC;
     for (int64_t i = tid; i < nvec; i += MT_THREADS) {
       raw r[8];
@@ -418,90 +429,134 @@ __device__ __forceinline__ void store4(void* base, int64_t i, const typename Low
   }
 }
 
-// The chunk's tensor without a chain of dependent loads: lane i compares chunk_start[i + 1]
-// with the chunk index, and the number of tensors that end at or before it is the answer.
-__device__ __forceinline__ int find_tensor_by_vote(const MtTable& t, int block) {
-  const int lane = threadIdx.x & 63;
-  const bool before = lane < t.n && t.chunk_start[lane + 1] <= block;
-  // the same in every lane and wave: as a scalar, so that the tensor's fields are scalar loads
-  return __builtin_amdgcn_readfirstlane(__builtin_popcountll(__ballot(before)));
+// One tensor's row of the table, in scalar registers.
+struct TensorRow {
+  const void* g;
+  float* p;
+  float* m;
+  float* v;
+  void* plow;
+  int64_t size;
+  int first_chunk;
+  int meta;
+};
+
+// The row of the tensor that owns chunk `block`, through the scalar cache only: three
+// pivots pick a quarter of the table, fifteen scalar compares on that quarter's starts pick
+// the tensor, its row follows - three rounds of scalar loads from the argument block,
+// which every wave of the launch repeats and the scalar cache holds.  Rows past the last
+// tensor start at 2^31 - 1, which no chunk index reaches.  (Fetching row i in lane i with
+// vector loads and voting is one round only, but those loads queue behind the streaming
+// loads of the CU's other waves: 5.9 against 6.3 TB/s for the update.)
+__device__ __forceinline__ TensorRow row_by_scalar_search(const MtTable& tab, int block) {
+  static_assert(MT_MAX == 64, "four quarters of sixteen rows");
+  // start <= block as the sign bit of start - block - 1 (both in [0, 2^31)): scalar adds only
+  auto at_or_before = [block](int start) -> int { return (int)((uint32_t)(start - block - 1) >> 31); };
+  const int q = at_or_before(tab.chunk_start[16]) + at_or_before(tab.chunk_start[32]) +
+                at_or_before(tab.chunk_start[48]);
+  const int base = q * 16;
+  int t = base;
+#pragma unroll
+  for (int j = 1; j < 16; ++j) t += at_or_before(tab.chunk_start[base + j]);
+  TensorRow r;
+  r.g = tab.g[t];
+  r.p = (float*)tab.p[t];
+  r.m = (float*)tab.m[t];
+  r.v = (float*)tab.v[t];
+  r.plow = tab.plow[t];
+  r.size = tab.size[t];
+  r.first_chunk = tab.chunk_start[t];
+  r.meta = tab.meta[t];
+  return r;
 }
 
-// What the update's rate hangs on, measured on MI355X in a stand-alone harness with this
-// access pattern (1.3e9 elements, 64 tensors): one 4-element vector per lane and trip (16
-// bytes of each fp32 stream, 8 of each 16-bit one) with every access non-temporal gives
-// 5.69 TB/s - 8 elements per lane 5.36, and 4.94 with cached loads of the state; and one
-// workgroup per chunk, handed out by the dispatcher in order so that the chip works on one
-// compact window of every stream - workgroups that stay resident and stride over the chunks
-// give 5.26 at 1024 per CU and 5.02 at 256.  128, 512 or 1024 lanes per workgroup: 5.29 to
-// 5.57.  The chunk size is free (1 K to 32 K elements, within 1 %); 16 K keeps the launch
-// of a step that is skipped on overflow at 80 K workgroups that return at once.  Where the
-// five streams lie relative to one another matters as much as the kernel: the same code
-// object measures 5.2 to 5.7 TB/s from one process and machine to the next.  Beyond
-// AXN_ADAM_WGS_PER_CU workgroups per CU (far above what the optimizer configurations
-// reach) a workgroup takes several chunks.
-template <int GDT, int PDT, bool HAS_PLOW>
-__global__ void __launch_bounds__(MT_THREADS)
-    mt_adam_kernel(const MtTable tab, const AdamScalars s,
-                   const axn_scan_result* scan, int total_chunks) {
+// What the update's rate hangs on, measured on MI355X (1.3e9 elements, 64 tensors, 28 bytes
+// per element):
+//  - one 4-element vector per lane (16 bytes of each fp32 stream, 8 of each 16-bit one),
+//    every access non-temporal, and a wave that ends after its one vector: a wave that
+//    loops waits for its own stores before its next loads return (the memory counter is
+//    in order; 16 vectors per wave lose 6 %), 8 elements per lane lose 6 %, cached loads
+//    of the state 13 %;
+//  - one chunk per workgroup, handed out by the dispatcher in order, so that the chip
+//    works on one compact window of every stream; resident workgroups that stride over
+//    the chunks lose 8 to 12 %;
+//  - FEWER waves in flight than the registers allow: with all 32 one-wave workgroups of a
+//    CU resident the five streams thrash one another in the memory system (5.7 TB/s),
+//    with about ten the same kernel moves 6.3 TB/s.  The launch reserves ADAM_LDS bytes of
+//    LDS per workgroup, which the kernel never touches, to hold the count there (14 to
+//    20 KB measure the same within 1 %; 12 KB and 22 KB lose 3 %);
+//  - a short way from the wave's start to its loads, because with few waves nothing hides
+//    it: the table lookup stays on the scalar path, and the scan result is loaded beside
+//    it, not in front of it.
+template <int GDT, int PDT, bool HAS_PLOW, bool HAS_SCAN>
+__global__ void __launch_bounds__(ADAM_THREADS)
+    mt_adam_kernel(const MtTable tab, const AdamScalars s, const axn_scan_result* scan) {
   typedef typename Lowp<GDT>::raw graw;
   typedef typename Lowp<PDT>::raw praw;
+  const int tid = threadIdx.x;
+  const int b = blockIdx.x;
+  const TensorRow row = row_by_scalar_search(tab, b);
+  int found_inf = 0;
   float gmul = 1.0f;
-  if (scan != nullptr) {
-    if (scan->found_inf != 0) return;  // overflow: the whole step is skipped
+  if (HAS_SCAN) {
+    found_inf = scan->found_inf;
     gmul = scan->clip_coef;
   }
-  const int tid = threadIdx.x;
-  for (int b = blockIdx.x; b < total_chunks; b += gridDim.x) {
-    const int t = find_tensor_by_vote(tab, b);
-    const int c = b - tab.chunk_start[t];
-    const Range rg = chunk_range(tab, t, c);
-    const void* g = tab.g[t];
-    float* p = (float*)tab.p[t];
-    float* m = (float*)tab.m[t];
-    float* v = (float*)tab.v[t];
-    void* plow = tab.plow[t];
+  const int c = b - row.first_chunk;
+  // Overflow: the whole step is skipped.  As an empty range rather than an early return,
+  // so that the scan result's load runs beside the table's and not in front of it.
+  const int head = found_inf != 0 ? 0 : row.meta & 0xff;
+  const int64_t size = found_inf != 0 ? 0 : row.size;
+  Range rg;
+  rg.begin = head + (int64_t)c * ADAM_CHUNK;
+  rg.end = rg.begin + ADAM_CHUNK;
+  if (rg.end > size) rg.end = size;
+  if (rg.begin > rg.end) rg.begin = rg.end;
+  const void* g = row.g;
+  float* p = row.p;
+  float* m = row.m;
+  float* v = row.v;
+  void* plow = row.plow;
 
-    auto one = [&](int64_t i) {
-      float pp = p[i], mm = m[i], vv = v[i];
-      adam_math(Lowp<GDT>::to_float(((const graw*)g)[i]), pp, mm, vv, s, gmul);
-      p[i] = pp;
-      m[i] = mm;
-      v[i] = vv;
-      if (HAS_PLOW) ((praw*)plow)[i] = Lowp<PDT>::from_float(pp);
-    };
+  auto one = [&](int64_t i) {
+    float pp = p[i], mm = m[i], vv = v[i];
+    adam_math(Lowp<GDT>::to_float(((const graw*)g)[i]), pp, mm, vv, s, gmul);
+    p[i] = pp;
+    m[i] = mm;
+    v[i] = vv;
+    if (HAS_PLOW) ((praw*)plow)[i] = Lowp<PDT>::from_float(pp);
+  };
 
-    if (tab.vec_ok[t]) {
-      if (c == 0 && tid < tab.head[t]) one(tid);
-      const int nvec = (int)((rg.end - rg.begin) / ADAM_VEC);
-      for (int i = tid; i < nvec; i += MT_THREADS) {
-        const int64_t e0 = rg.begin + (int64_t)i * ADAM_VEC;
-        graw gr[4];
-        praw pl[4];
-        load4<GDT, AXN_ADAM_NT_G != 0>(g, e0, gr);
-        f32x4 pp = ld<AXN_ADAM_NT_LOAD != 0>((const f32x4*)(p + e0));
-        f32x4 mm = ld<AXN_ADAM_NT_LOAD != 0>((const f32x4*)(m + e0));
-        f32x4 vv = ld<AXN_ADAM_NT_LOAD != 0>((const f32x4*)(v + e0));
+  if (row.meta & 0x100) {
+    if (c == 0 && tid < head) one(tid);
+    const int nvec = (int)((rg.end - rg.begin) / ADAM_VEC);
+    for (int i = tid; i < nvec; i += ADAM_THREADS) {  // one trip: ADAM_CHUNK = 4 per lane
+      const int64_t e0 = rg.begin + (int64_t)i * ADAM_VEC;
+      graw gr[4];
+      praw pl[4];
+      load4<GDT, AXN_ADAM_NT_G != 0>(g, e0, gr);
+      f32x4 pp = ld<AXN_ADAM_NT_LOAD != 0>((const f32x4*)(p + e0));
+      f32x4 mm = ld<AXN_ADAM_NT_LOAD != 0>((const f32x4*)(m + e0));
+      f32x4 vv = ld<AXN_ADAM_NT_LOAD != 0>((const f32x4*)(v + e0));
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          float pe = pp[e], me = mm[e], ve = vv[e];
-          adam_math(Lowp<GDT>::to_float(gr[e]), pe, me, ve, s, gmul);
-          pp[e] = pe;
-          mm[e] = me;
-          vv[e] = ve;
-          if (HAS_PLOW) pl[e] = Lowp<PDT>::from_float(pe);
-        }
-        st<AXN_ADAM_NT_STORE != 0>(pp, (f32x4*)(p + e0));
-        st<AXN_ADAM_NT_STORE != 0>(mm, (f32x4*)(m + e0));
-        st<AXN_ADAM_NT_STORE != 0>(vv, (f32x4*)(v + e0));
-        if (HAS_PLOW) store4<PDT, AXN_ADAM_NT_STORE != 0>(plow, e0, pl);
+      for (int e = 0; e < 4; ++e) {
+        float pe = pp[e], me = mm[e], ve = vv[e];
+        adam_math(Lowp<GDT>::to_float(gr[e]), pe, me, ve, s, gmul);
+        pp[e] = pe;
+        mm[e] = me;
+        vv[e] = ve;
+        if (HAS_PLOW) pl[e] = Lowp<PDT>::from_float(pe);
       }
-      const int64_t tail = rg.begin + (int64_t)nvec * ADAM_VEC;
-      if (tail + tid < rg.end) one(tail + tid);
-    } else {
-      const int64_t b0 = (c == 0) ? 0 : rg.begin;
-      for (int64_t i = b0 + tid; i < rg.end; i += MT_THREADS) one(i);
+      st<AXN_ADAM_NT_STORE != 0>(pp, (f32x4*)(p + e0));
+      st<AXN_ADAM_NT_STORE != 0>(mm, (f32x4*)(m + e0));
+      st<AXN_ADAM_NT_STORE != 0>(vv, (f32x4*)(v + e0));
+      if (HAS_PLOW) store4<PDT, AXN_ADAM_NT_STORE != 0>(plow, e0, pl);
     }
+    const int64_t tail = rg.begin + (int64_t)nvec * ADAM_VEC;
+    if (tail + tid < rg.end) one(tail + tid);
+  } else {
+    const int64_t b0 = (c == 0) ? 0 : rg.begin;
+    for (int64_t i = b0 + tid; i < rg.end; i += ADAM_THREADS) one(i);
   }
 }
 
@@ -523,8 +578,8 @@ __global__ void __launch_bounds__(MT_THREADS)
     if (use_clip) y = Lowp<DT>::from_float(Lowp<DT>::to_float(y) * coef);
     return y;
   };
-  if (tab.vec_ok[t]) {
-    if (c == 0 && tid < tab.head[t]) ((raw*)g)[tid] = f(((raw*)g)[tid]);
+  if (vec_ok_of(tab, t)) {
+    if (c == 0 && tid < head_of(tab, t)) ((raw*)g)[tid] = f(((raw*)g)[tid]);
     const int64_t nvec = (rg.end - rg.begin) / MT_VEC;
     for (int64_t i = tid; i < nvec; i += MT_THREADS) {
       raw r[8];
@@ -621,7 +676,9 @@ int for_each_group(const void* const* const* ptr_sets, const int* elem_sizes, in
     if (k == 0) return AXN_OK;
     cur.tab.n = k;
     cur.tab.chunk = chunk;
-    cur.tab.chunk_start[k] = cur.blocks;
+    // past the last tensor: a start no workgroup index reaches, so that a lookup need
+    // not know the count
+    for (int j = k; j <= MT_MAX; ++j) cur.tab.chunk_start[j] = j == k ? cur.blocks : 0x7fffffff;
     const int rc = emit(cur);
     cur.tab = MtTable();
     cur.blocks = 0;
@@ -656,8 +713,7 @@ int for_each_group(const void* const* const* ptr_sets, const int* elem_sizes, in
     cur.tab.plow[k] = const_cast<void*>(ptrs[4]);
     cur.tab.size[k] = sz;
     cur.tab.chunk_start[k] = cur.blocks;
-    cur.tab.head[k] = (uint8_t)head;
-    cur.tab.vec_ok[k] = vec_ok ? 1 : 0;
+    cur.tab.meta[k] = head | (vec_ok ? 0x100 : 0);
     cur.blocks += (int)chunks;
     ++k;
   }
@@ -825,23 +881,28 @@ int launch_mt_scan_noalloc(const void* const* h_g, const int64_t* h_sizes, int64
 }
 
 namespace {
-template <int GDT>
-int adam_dispatch(const Group& gr, const AdamScalars& s, int plow_dtype,
-                  bool has_plow, const axn_scan_result* scan, hipStream_t stream) {
-  const long long cap = (long long)cu_count() * AXN_ADAM_WGS_PER_CU;
-  const dim3 grid((unsigned)(gr.blocks < cap ? gr.blocks : cap)), block(MT_THREADS);
+template <int GDT, bool HAS_SCAN>
+int adam_launch(const Group& gr, const AdamScalars& s, int plow_dtype, bool has_plow,
+                const axn_scan_result* scan, hipStream_t stream) {
+  const dim3 grid((unsigned)gr.blocks), block(ADAM_THREADS);
   if (!has_plow) {
-    hipLaunchKernelGGL((mt_adam_kernel<GDT, AXN_BF16, false>), grid, block, 0,
-                       stream, gr.tab, s, scan, gr.blocks);
+    hipLaunchKernelGGL((mt_adam_kernel<GDT, AXN_BF16, false, HAS_SCAN>), grid, block, ADAM_LDS,
+                       stream, gr.tab, s, scan);
   } else if (plow_dtype == AXN_BF16) {
-    hipLaunchKernelGGL((mt_adam_kernel<GDT, AXN_BF16, true>), grid, block, 0,
-                       stream, gr.tab, s, scan, gr.blocks);
+    hipLaunchKernelGGL((mt_adam_kernel<GDT, AXN_BF16, true, HAS_SCAN>), grid, block, ADAM_LDS,
+                       stream, gr.tab, s, scan);
   } else {
-    hipLaunchKernelGGL((mt_adam_kernel<GDT, AXN_F16, true>), grid, block, 0,
-                       stream, gr.tab, s, scan, gr.blocks);
+    hipLaunchKernelGGL((mt_adam_kernel<GDT, AXN_F16, true, HAS_SCAN>), grid, block, ADAM_LDS,
+                       stream, gr.tab, s, scan);
   }
   AXN_HIP_TRY(hipGetLastError());
   return AXN_OK;
+}
+template <int GDT>
+int adam_dispatch(const Group& gr, const AdamScalars& s, int plow_dtype,
+                  bool has_plow, const axn_scan_result* scan, hipStream_t stream) {
+  return scan != nullptr ? adam_launch<GDT, true>(gr, s, plow_dtype, has_plow, scan, stream)
+                         : adam_launch<GDT, false>(gr, s, plow_dtype, has_plow, scan, stream);
 }
 }  // namespace
 
