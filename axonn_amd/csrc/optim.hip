@@ -40,7 +40,7 @@ namespace {
 #define AXN_ADAM_CHUNK (AXN_ADAM_THREADS * 4)
 #endif
 #ifndef AXN_ADAM_LDS
-#define AXN_ADAM_LDS 16384
+#define AXN_ADAM_LDS 14336
 #endif
 #ifndef AXN_ADAM_NT_G
 #define AXN_ADAM_NT_G 1
