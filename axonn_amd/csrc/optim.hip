@@ -36,11 +36,12 @@ namespace {
 #ifndef AXN_ADAM_THREADS
 #define AXN_ADAM_THREADS 64
 #endif
-#ifndef AXN_ADAM_CHUNK
-#define AXN_ADAM_CHUNK (AXN_ADAM_THREADS * 4)
+#ifndef AXN_ADAM_VECS
+#define AXN_ADAM_VECS 4
 #endif
+#define AXN_ADAM_CHUNK (AXN_ADAM_THREADS * 4 * AXN_ADAM_VECS)
 #ifndef AXN_ADAM_LDS
-#define AXN_ADAM_LDS 14336
+#define AXN_ADAM_LDS 27136
 #endif
 #ifndef AXN_ADAM_NT_G
 #define AXN_ADAM_NT_G 1
@@ -63,6 +64,7 @@ constexpr int ADAM_CHUNK = AXN_ADAM_CHUNK;
 constexpr int SCALE_CHUNK = 16384;
 constexpr int ADAM_VEC = 4;                   // elements per lane of the update kernel
 constexpr int ADAM_THREADS = AXN_ADAM_THREADS;  // lanes per workgroup of the update kernel
+constexpr int ADAM_VECS = AXN_ADAM_VECS;        // vectors per lane
 // LDS the update kernel reserves per workgroup and never touches: it bounds the
 // workgroups that are resident on a CU (160 KB per CU), see mt_adam_kernel.
 constexpr int ADAM_LDS = AXN_ADAM_LDS;
@@ -472,19 +474,21 @@ __device__ __forceinline__ TensorRow row_by_scalar_search(const MtTable& tab, in
 
 // What the update's rate hangs on, measured on MI355X (1.3e9 elements, 64 tensors, 28 bytes
 // per element):
-//  - one 4-element vector per lane (16 bytes of each fp32 stream, 8 of each 16-bit one),
-//    every access non-temporal, and a wave that ends after its one vector: a wave that
-//    loops waits for its own stores before its next loads return (the memory counter is
-//    in order; 16 vectors per wave lose 6 %), 8 elements per lane lose 6 %, cached loads
-//    of the state 13 %;
+//  - every access a wave makes covers consecutive bytes (one 4-element vector per lane:
+//    16 bytes of each fp32 stream, 8 of each 16-bit one) and is non-temporal; 8 elements
+//    per lane in one access lose 6 %, cached loads of the state 13 %;
+//  - all loads of a wave in front of its first store, and a wave that ends after its
+//    stores: a wave that loops waits for its own stores before its next loads return
+//    (the memory counter is in order; 16 trips per wave lose 6 %);
 //  - one chunk per workgroup, handed out by the dispatcher in order, so that the chip
 //    works on one compact window of every stream; resident workgroups that stride over
 //    the chunks lose 8 to 12 %;
 //  - FEWER waves in flight than the registers allow: with all 32 one-wave workgroups of a
-//    CU resident the five streams thrash one another in the memory system (5.7 TB/s),
-//    with about ten the same kernel moves 6.3 TB/s.  The launch reserves ADAM_LDS bytes of
-//    LDS per workgroup, which the kernel never touches, to hold the count there (14 to
-//    20 KB measure the same within 1 %; 12 KB and 22 KB lose 3 %);
+//    CU resident the five streams thrash one another in the memory system (5.7 TB/s);
+//    six waves of four vectors per lane, or ten of one, move 6.2 to 6.3 TB/s.  The launch
+//    reserves ADAM_LDS bytes of LDS per workgroup, which the kernel never touches, to hold
+//    the count there (four vectors per lane: 24 to 40 KB measure within 1.5 % of the best,
+//    20 KB loses 5 %; four vectors instead of one halve the cost of a skipped step);
 //  - a short way from the wave's start to its loads, because with few waves nothing hides
 //    it: the table lookup stays on the scalar path, and the scan result is loaded beside
 //    it, not in front of it.
@@ -530,27 +534,46 @@ __global__ void __launch_bounds__(ADAM_THREADS)
   if (row.meta & 0x100) {
     if (c == 0 && tid < head) one(tid);
     const int nvec = (int)((rg.end - rg.begin) / ADAM_VEC);
-    for (int i = tid; i < nvec; i += ADAM_THREADS) {  // one trip: ADAM_CHUNK = 4 per lane
-      const int64_t e0 = rg.begin + (int64_t)i * ADAM_VEC;
-      graw gr[4];
+    // ADAM_VECS vectors per lane, ADAM_THREADS vectors apart (every access of the wave
+    // covers consecutive bytes), all loads in front of the first store.
+    graw gr[ADAM_VECS][4];
+    f32x4 pp[ADAM_VECS], mm[ADAM_VECS], vv[ADAM_VECS];
+    auto fetch = [&](int k) {
+      const int64_t e0 = rg.begin + (int64_t)(tid + k * ADAM_THREADS) * ADAM_VEC;
+      load4<GDT, AXN_ADAM_NT_G != 0>(g, e0, gr[k]);
+      pp[k] = ld<AXN_ADAM_NT_LOAD != 0>((const f32x4*)(p + e0));
+      mm[k] = ld<AXN_ADAM_NT_LOAD != 0>((const f32x4*)(m + e0));
+      vv[k] = ld<AXN_ADAM_NT_LOAD != 0>((const f32x4*)(v + e0));
+    };
+    auto update = [&](int k) {
+      const int64_t e0 = rg.begin + (int64_t)(tid + k * ADAM_THREADS) * ADAM_VEC;
       praw pl[4];
-      load4<GDT, AXN_ADAM_NT_G != 0>(g, e0, gr);
-      f32x4 pp = ld<AXN_ADAM_NT_LOAD != 0>((const f32x4*)(p + e0));
-      f32x4 mm = ld<AXN_ADAM_NT_LOAD != 0>((const f32x4*)(m + e0));
-      f32x4 vv = ld<AXN_ADAM_NT_LOAD != 0>((const f32x4*)(v + e0));
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        float pe = pp[e], me = mm[e], ve = vv[e];
-        adam_math(Lowp<GDT>::to_float(gr[e]), pe, me, ve, s, gmul);
-        pp[e] = pe;
-        mm[e] = me;
-        vv[e] = ve;
+        float pe = pp[k][e], me = mm[k][e], ve = vv[k][e];
+        adam_math(Lowp<GDT>::to_float(gr[k][e]), pe, me, ve, s, gmul);
+        pp[k][e] = pe;
+        mm[k][e] = me;
+        vv[k][e] = ve;
         if (HAS_PLOW) pl[e] = Lowp<PDT>::from_float(pe);
       }
-      st<AXN_ADAM_NT_STORE != 0>(pp, (f32x4*)(p + e0));
-      st<AXN_ADAM_NT_STORE != 0>(mm, (f32x4*)(m + e0));
-      st<AXN_ADAM_NT_STORE != 0>(vv, (f32x4*)(v + e0));
+      st<AXN_ADAM_NT_STORE != 0>(pp[k], (f32x4*)(p + e0));
+      st<AXN_ADAM_NT_STORE != 0>(mm[k], (f32x4*)(m + e0));
+      st<AXN_ADAM_NT_STORE != 0>(vv[k], (f32x4*)(v + e0));
       if (HAS_PLOW) store4<PDT, AXN_ADAM_NT_STORE != 0>(plow, e0, pl);
+    };
+    if (nvec == ADAM_VECS * ADAM_THREADS) {  // a whole chunk: nothing to guard
+#pragma unroll
+      for (int k = 0; k < ADAM_VECS; ++k) fetch(k);
+#pragma unroll
+      for (int k = 0; k < ADAM_VECS; ++k) update(k);
+    } else {
+#pragma unroll
+      for (int k = 0; k < ADAM_VECS; ++k)
+        if (tid + k * ADAM_THREADS < nvec) fetch(k);
+#pragma unroll
+      for (int k = 0; k < ADAM_VECS; ++k)
+        if (tid + k * ADAM_THREADS < nvec) update(k);
     }
     const int64_t tail = rg.begin + (int64_t)nvec * ADAM_VEC;
     if (tail + tid < rg.end) one(tail + tid);
