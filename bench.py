@@ -42,8 +42,9 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 # file, scaled by what the same counters read for the 1 GiB copy below
 # (profiles/gemm_adam_llama_set_pmc.txt has the runs and the arithmetic).  The
 # counters sit between L2 and the fabric, so hits in the memory-side cache are included.
-TRAFFIC_BYTES_PER_LAUNCH = {"fwd": 634638544, "dgrad": 587542396, "wgrad": 664855104}
-ADAM_TRAFFIC_BYTES_PER_STEP = 39286797387   # scan + update, 1.3e9 elements
+TRAFFIC_BYTES_PER_LAUNCH = {"fwd": 634663897, "dgrad": 587559040, "wgrad": 664873790}
+ADAM_TRAFFIC_BYTES_PER_STEP = 39000439559   # scan + update, 1.3e9 elements: 1.000 x 30 B/element
+TRAFFIC_SOURCE = "profiles/gemm_adam_llama_set_pmc.txt"
 
 LLAMA_SET = [  # (name, M, N, K), gate and up are two layers of one shape
     ("qkv", 4096, 6144, 4096),
@@ -208,6 +209,7 @@ def main():
             "launches_timed": kinds[dom]["launches"],  # those of every EVENT_EVERY-th timed step
             "flops_per_launch": kinds[dom]["tflops"] * 1e12 * kinds[dom]["avg_us"] * 1e-6,
             "traffic": TRAFFIC_BYTES_PER_LAUNCH.get(dom),
+            "traffic_source": TRAFFIC_SOURCE,
             "traffic_counts": "bytes between the 8 XCD-private L2s and the fabric (FETCH_SIZE + WRITE_SIZE), "
                               "reads served by the 256 MB memory-side cache included: each L2 pulls its own "
                               "copy of a shared operand panel, so this bounds HBM bytes from above",
@@ -598,7 +600,8 @@ def bench_adam(args, torch, nv, lib, stream, time_loop):
         "roofline": {"bound": "hbm", "kernel": "mt_adam_kernel + mt_scan_kernel",
                      "achieved": round(30.0 * total / t_full / 1e9, 1), "peak": PEAK_HBM_GBS,
                      "unit": "GB/s", "frac": round(30.0 * total / t_full / 1e9 / PEAK_HBM_GBS, 4),
-                     "traffic": ADAM_TRAFFIC_BYTES_PER_STEP if total == 1300000000 else None},
+                     "traffic": ADAM_TRAFFIC_BYTES_PER_STEP if total == 1300000000 else None,
+                     "traffic_source": TRAFFIC_SOURCE},
         "scan_ms": round(t_scan * 1e3, 4), "scan_gbs": round(2.0 * total / t_scan / 1e9, 1),
         "update_ms": round(t_upd * 1e3, 4), "update_gbs": round(28.0 * total / t_upd / 1e9, 1),
         "found_inf": found,

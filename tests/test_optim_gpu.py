@@ -88,6 +88,20 @@ def test_step_matches_oracle_ragged_layouts(sizes, start):
         assert torch.equal(out[0][:start].cpu(), P[:start])
 
 
+@pytest.mark.parametrize("count", [2, 15, 16, 17, 31, 32, 33, 47, 48, 49, 63, 64, 65, 130])
+def test_every_row_of_the_tensor_table_is_found(count):
+    """The update kernel finds a chunk's tensor in two steps (a quarter of the 64-row table,
+    then a row of it): tensor counts on both sides of every quarter, tensors of less than
+    one chunk, of exactly one (1024 elements), and of several with a ragged end, and more
+    tensors than one launch holds."""
+    rng = np.random.default_rng(count)
+    sizes = [int(rng.choice([1, 5, 255, 256, 1023, 1024, 1025, 2048, 4097, 5000])) for _ in range(count)]
+    P, G, M, V = make_state(sizes, seed=100 + count)
+    res = run_oracle(P, G, M, V, sizes, 0, 2, 65536.0, 1.0, "bf16")
+    out = run_hip(P, G, M, V, sizes, 0, 2, 65536.0, 1.0)
+    check_against_oracle(res, *out, sizes, 0)
+
+
 @pytest.mark.parametrize("g_dtype,name", [(torch.float16, "f16"), (torch.float32, "f32")])
 def test_step_other_gradient_dtypes(g_dtype, name):
     sizes = [5001, 17, 40000]
