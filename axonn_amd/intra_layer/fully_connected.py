@@ -100,29 +100,34 @@ class AsyncLinear(Function):
         weight = weight.reshape(local_weight_shape)
         dt = _compute_dtype(input_, weight)
         x = input_.reshape(-1, input_.shape[-1]).to(dt)
-        ctx.save_for_backward(x, original_weight)
+        w = weight.to(dt)
+        # A weight cast for this step (fp32 parameter under autocast) is kept for the
+        # backward pass, as torch's autocast keeps its casts of parameters: one cast per
+        # step, not one in forward and one more in backward.
+        ctx.save_for_backward(x, original_weight, w if w.dtype != weight.dtype else None)
         ctx.backward_all_reduce_group = backward_all_reduce_group
         ctx.depth_parallel_group = depth_parallel_group
         ctx.shape = local_weight_shape
         ctx.input_shape = input_.shape
         ctx.compute_dtype = dt
         get_world_size(forward_all_reduce_group)  # one rank: the all-reduce is the identity
-        output, _ = ops.gemm_fwd(x, weight.to(dt))
+        output, _ = ops.gemm_fwd(x, w)
         return output.reshape(*input_.shape[:-1], local_weight_shape[0])
 
     @staticmethod
     @torch.amp.custom_bwd(device_type="cuda")
     def backward(ctx, grad_output):
-        x, original_weight = ctx.saved_tensors
+        x, original_weight, w_cast = ctx.saved_tensors
         weight = _gather(original_weight, dim=0, process_group=ctx.depth_parallel_group,
                          cache=False)
         weight = weight.reshape(ctx.shape)
         dt = ctx.compute_dtype
+        w = w_cast if w_cast is not None else weight.to(dt)
         g = grad_output.reshape(-1, grad_output.shape[-1]).to(dt)
         grad_input, grad_weight = None, None
         get_world_size(ctx.backward_all_reduce_group)
         if ctx.needs_input_grad[0]:
-            grad_input = ops.gemm_dgrad(g, weight.to(dt)).reshape(ctx.input_shape)
+            grad_input = ops.gemm_dgrad(g, w).reshape(ctx.input_shape)
         if ctx.needs_input_grad[1]:
             grad_weight = _weight_grad(g, x, original_weight)
         return grad_input, grad_weight, None, None, None, None, None
@@ -142,9 +147,10 @@ class FusedLinear(Function):
         dt = _compute_dtype(input_, weight)
         x = input_.reshape(-1, input_.shape[-1]).to(dt)
         needs_grad = any(ctx.needs_input_grad[:3])
-        output, z = ops.gemm_fwd(x, weight.to(dt), bias=bias, activation=activation,
-                                 save_z=needs_grad)
-        ctx.save_for_backward(x, original_weight, z)
+        w = weight.to(dt)
+        output, z = ops.gemm_fwd(x, w, bias=bias, activation=activation, save_z=needs_grad)
+        # the step's cast of an fp32 weight is kept for the backward pass (see AsyncLinear)
+        ctx.save_for_backward(x, original_weight, z, w if w.dtype != weight.dtype else None)
         ctx.shape = local_weight_shape
         ctx.input_shape = input_.shape
         ctx.compute_dtype = dt
@@ -154,9 +160,10 @@ class FusedLinear(Function):
     @staticmethod
     @torch.amp.custom_bwd(device_type="cuda")
     def backward(ctx, grad_output):
-        x, original_weight, z = ctx.saved_tensors
+        x, original_weight, z, w_cast = ctx.saved_tensors
         weight = original_weight.reshape(ctx.shape)
         dt = ctx.compute_dtype
+        w = w_cast if w_cast is not None else weight.to(dt)
         g = grad_output.reshape(-1, grad_output.shape[-1]).to(dt)
         want_dbias = ctx.has_bias and ctx.needs_input_grad[2]
         grad_bias = None
@@ -164,7 +171,7 @@ class FusedLinear(Function):
             g, grad_bias = ops.dgelu_dbias(g, z, want_dbias=want_dbias)
         grad_input, grad_weight = None, None
         if ctx.needs_input_grad[0]:
-            grad_input = ops.gemm_dgrad(g, weight.to(dt)).reshape(ctx.input_shape)
+            grad_input = ops.gemm_dgrad(g, w).reshape(ctx.input_shape)
         if ctx.needs_input_grad[1]:
             grad_weight = _weight_grad(g, x, original_weight)
         return grad_input, grad_weight, grad_bias, None, None
