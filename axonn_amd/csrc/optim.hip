@@ -36,20 +36,18 @@ namespace {
 #define AXN_ADAM_THREADS 64
 #endif
 #ifndef AXN_ADAM_VECS
-#define AXN_ADAM_VECS 4
+#define AXN_ADAM_VECS 1
 #endif
 #define AXN_ADAM_CHUNK (AXN_ADAM_THREADS * 4 * AXN_ADAM_VECS)
 #ifndef AXN_ADAM_LDS
-#define AXN_ADAM_LDS 27136
+#define AXN_ADAM_LDS 15360
 #endif
-#ifndef AXN_ADAM_NT_G
-#define AXN_ADAM_NT_G 1
+// Cache policy bits of the update kernel's buffer accesses (1 sc0, 2 nt, 16 sc1).
+#ifndef AXN_ADAM_LOAD_POLICY
+#define AXN_ADAM_LOAD_POLICY 2
 #endif
-#ifndef AXN_ADAM_NT_STORE
-#define AXN_ADAM_NT_STORE 1
-#endif
-#ifndef AXN_ADAM_NT_LOAD
-#define AXN_ADAM_NT_LOAD 1
+#ifndef AXN_ADAM_STORE_POLICY
+#define AXN_ADAM_STORE_POLICY 18
 #endif
 
 constexpr int MT_MAX = 64;         // tensors per launch
@@ -57,7 +55,7 @@ constexpr int MT_THREADS = 256;    // threads per workgroup
 constexpr int MT_VEC = 8;          // elements per lane per step
 // Elements per workgroup.  The read-only scan streams best in long runs with
 // non-temporal loads; the read-modify-write update does best with one-wave workgroups
-// that make one trip (ADAM_VECS 4-element vectors per lane, see mt_adam_kernel).  Both
+// that make one trip of ADAM_VECS 4-element vectors per lane (see mt_adam_kernel).  Both
 // measured on MI355X.
 constexpr int SCAN_CHUNK = AXN_SCAN_CHUNK;
 constexpr int ADAM_CHUNK = AXN_ADAM_CHUNK;
@@ -68,6 +66,9 @@ constexpr int ADAM_VECS = AXN_ADAM_VECS;        // vectors per lane
 // LDS the update kernel reserves per workgroup and never touches: it bounds the
 // workgroups that are resident on a CU (160 KB per CU), see mt_adam_kernel.
 constexpr int ADAM_LDS = AXN_ADAM_LDS;
+// Loads non-temporal; stores non-temporal and written through (nt + sc1): 1 to 2 % over
+// nt alone, 10 % over plain stores, measured on MI355X.
+constexpr int ADAM_LOAD_POLICY = AXN_ADAM_LOAD_POLICY, ADAM_STORE_POLICY = AXN_ADAM_STORE_POLICY;
 static_assert(ADAM_THREADS >= 64 && ADAM_THREADS % 64 == 0, "a tensor's scalar head (up to 63 elements) is one element per lane");
 static_assert(ADAM_CHUNK % MT_VEC == 0, "chunks keep the 16-byte alignment of the tensor's body");
 static_assert(ADAM_LDS <= 65536, "dynamic LDS a launch may ask for without a function attribute");
@@ -398,41 +399,7 @@ __device__ __forceinline__ void adam_math(float g, float& p, float& m, float& v,
   asm volatile("" : "+v"(p));
 }
 
-// 4 consecutive low-precision elements from an address aligned to their 4 (8 or 16 bytes).
 typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
-template <int DT, bool NT>
-__device__ __forceinline__ void load4(const void* base, int64_t i, typename Lowp<DT>::raw (&r)[4]) {
-  typedef typename Lowp<DT>::raw raw;
-  const raw* p = (const raw*)base + i;
-  if (sizeof(raw) == 2) {
-    const u32x2 w = ld<NT>((const u32x2*)p);
-#pragma unroll
-    for (int e = 0; e < 2; ++e) {
-      r[2 * e] = (raw)(w[e] & 0xFFFFu);
-      r[2 * e + 1] = (raw)(w[e] >> 16);
-    }
-  } else {
-    const u32x4 w = ld<NT>((const u32x4*)p);
-#pragma unroll
-    for (int e = 0; e < 4; ++e) r[e] = (raw)w[e];
-  }
-}
-template <int DT, bool NT>
-__device__ __forceinline__ void store4(void* base, int64_t i, const typename Lowp<DT>::raw (&r)[4]) {
-  typedef typename Lowp<DT>::raw raw;
-  raw* p = (raw*)base + i;
-  if (sizeof(raw) == 2) {
-    u32x2 w;
-#pragma unroll
-    for (int e = 0; e < 2; ++e) w[e] = (uint32_t)r[2 * e] | ((uint32_t)r[2 * e + 1] << 16);
-    st<NT>(w, (u32x2*)p);
-  } else {
-    u32x4 w;
-#pragma unroll
-    for (int e = 0; e < 4; ++e) w[e] = (uint32_t)r[e];
-    st<NT>(w, (u32x4*)p);
-  }
-}
 
 // One tensor's row of the table, in scalar registers.
 struct TensorRow {
@@ -476,10 +443,11 @@ __device__ __forceinline__ TensorRow row_by_scalar_search(const MtTable& tab, in
 }
 
 // What the update's rate hangs on, measured on MI355X (1.3e9 elements, 64 tensors, 28 bytes
-// per element):
+// per element; 6.5 to 6.6 TB/s as it stands):
 //  - every access a wave makes covers consecutive bytes (one 4-element vector per lane:
-//    16 bytes of each fp32 stream, 8 of each 16-bit one) and is non-temporal; 8 elements
-//    per lane in one access lose 6 %, cached loads of the state 13 %;
+//    16 bytes of each fp32 stream, 8 of each 16-bit one); loads non-temporal, stores
+//    non-temporal and written through (nt + sc1: 1 to 2 % over nt alone, 10 % over plain
+//    stores); 8 elements per lane in one access lose 6 %, cached loads of the state 13 %;
 //  - all loads of a wave in front of its first store, and a wave that ends after its
 //    stores: a wave that loops waits for its own stores before its next loads return
 //    (the memory counter is in order; 16 trips per wave lose 6 %);
@@ -488,13 +456,16 @@ __device__ __forceinline__ TensorRow row_by_scalar_search(const MtTable& tab, in
 //    the chunks lose 8 to 12 %;
 //  - FEWER waves in flight than the registers allow: with all 32 one-wave workgroups of a
 //    CU resident the five streams thrash one another in the memory system (5.7 TB/s);
-//    six waves of four vectors per lane, or ten of one, move 6.2 to 6.3 TB/s.  The launch
-//    reserves ADAM_LDS bytes of LDS per workgroup, which the kernel never touches, to hold
-//    the count there (four vectors per lane: 24 to 40 KB measure within 1.5 % of the best,
-//    20 KB loses 5 %; four vectors instead of one halve the cost of a skipped step);
+//    ten or eleven waves of one vector per lane are the best found (14 to 16 KB reserved
+//    per workgroup: within 0.5 %; 12 KB: -2 %, 18 KB: -2.5 %).  The launch reserves ADAM_LDS
+//    bytes of LDS per workgroup, which the kernel never touches, to hold the count there.
+//    Several vectors per lane (ADAM_VECS) need fewer waves and make a skipped step cheaper
+//    (1.27 M instead of 5.1 M workgroups that leave at once), but move 6 % less;
 //  - a short way from the wave's start to its loads, because with few waves nothing hides
-//    it: the table lookup stays on the scalar path, and the scan result is loaded beside
-//    it, not in front of it.
+//    it: the table lookup stays on the scalar path, the scan result is loaded beside it,
+//    not in front of it, and the accesses are buffer accesses (one descriptor per stream
+//    in scalar registers, one 32-bit offset per lane: +3 to 4 % over 64-bit addresses
+//    computed per lane).
 template <int GDT, int PDT, bool HAS_PLOW, bool HAS_SCAN>
 __global__ void __launch_bounds__(ADAM_THREADS)
     mt_adam_kernel(const MtTable tab, const AdamScalars s, const axn_scan_result* scan) {
@@ -541,17 +512,42 @@ __global__ void __launch_bounds__(ADAM_THREADS)
     // covers consecutive bytes), all loads in front of the first store.  Vector by vector
     // (g p m v, g p m v, ...); stream by stream (p p p p, m m m m, ...) measured the same on
     // constant data and 2 % slower on random data.
+    // Each stream of the chunk is a buffer of exactly the bytes of its nvec vectors: the
+    // hardware drops the accesses of the lanes behind the end (loads return zero, stores
+    // do nothing), so a ragged last chunk runs the same code, and a lane needs one 32-bit
+    // offset per access instead of a 64-bit address.
+    constexpr int GSZ = (int)sizeof(graw), PSZ = (int)sizeof(praw);
+    auto stream = [&](const void* base, int elem) {
+      return __builtin_amdgcn_make_buffer_rsrc((void*)((const char*)base + rg.begin * elem), 0,
+                                               nvec * ADAM_VEC * elem, 0x00020000);
+    };
+    if (nvec > 0) {   // (a skipped step's waves leave here)
+    const __amdgpu_buffer_rsrc_t bg = stream(g, GSZ), bp = stream(p, 4), bm = stream(m, 4),
+                                 bv = stream(v, 4), bl = stream(HAS_PLOW ? plow : p, PSZ);
     graw gr[ADAM_VECS][4];
     f32x4 pp[ADAM_VECS], mm[ADAM_VECS], vv[ADAM_VECS];
-    auto fetch = [&](int k) {
-      const int64_t e0 = rg.begin + (int64_t)(tid + k * ADAM_THREADS) * ADAM_VEC;
-      load4<GDT, AXN_ADAM_NT_G != 0>(g, e0, gr[k]);
-      pp[k] = ld<AXN_ADAM_NT_LOAD != 0>((const f32x4*)(p + e0));
-      mm[k] = ld<AXN_ADAM_NT_LOAD != 0>((const f32x4*)(m + e0));
-      vv[k] = ld<AXN_ADAM_NT_LOAD != 0>((const f32x4*)(v + e0));
-    };
-    auto update = [&](int k) {
-      const int64_t e0 = rg.begin + (int64_t)(tid + k * ADAM_THREADS) * ADAM_VEC;
+#pragma unroll
+    for (int k = 0; k < ADAM_VECS; ++k) {
+      const int e0 = (tid + k * ADAM_THREADS) * ADAM_VEC;
+      if (GSZ == 2) {
+        const u32x2 w = __builtin_bit_cast(u32x2, __builtin_amdgcn_raw_buffer_load_b64(bg, e0 * 2, 0, ADAM_LOAD_POLICY));
+        gr[k][0] = (graw)(w[0] & 0xFFFFu);
+        gr[k][1] = (graw)(w[0] >> 16);
+        gr[k][2] = (graw)(w[1] & 0xFFFFu);
+        gr[k][3] = (graw)(w[1] >> 16);
+      } else {
+        const u32x4 w = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(bg, e0 * 4, 0, ADAM_LOAD_POLICY));
+#pragma unroll
+        for (int e = 0; e < 4; ++e) gr[k][e] = (graw)w[e];
+      }
+      pp[k] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(bp, e0 * 4, 0, ADAM_LOAD_POLICY));
+      mm[k] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(bm, e0 * 4, 0, ADAM_LOAD_POLICY));
+      vv[k] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(bv, e0 * 4, 0, ADAM_LOAD_POLICY));
+    }
+    __builtin_amdgcn_sched_barrier(0);   // every load is issued before the arithmetic of the first vector
+#pragma unroll
+    for (int k = 0; k < ADAM_VECS; ++k) {
+      const int e0 = (tid + k * ADAM_THREADS) * ADAM_VEC;
       praw pl[4];
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
@@ -562,23 +558,23 @@ __global__ void __launch_bounds__(ADAM_THREADS)
         vv[k][e] = ve;
         if (HAS_PLOW) pl[e] = Lowp<PDT>::from_float(pe);
       }
-      st<AXN_ADAM_NT_STORE != 0>(pp[k], (f32x4*)(p + e0));
-      st<AXN_ADAM_NT_STORE != 0>(mm[k], (f32x4*)(m + e0));
-      st<AXN_ADAM_NT_STORE != 0>(vv[k], (f32x4*)(v + e0));
-      if (HAS_PLOW) store4<PDT, AXN_ADAM_NT_STORE != 0>(plow, e0, pl);
-    };
-    if (nvec == ADAM_VECS * ADAM_THREADS) {  // a whole chunk: nothing to guard
+      __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, pp[k]), bp, e0 * 4, 0, ADAM_STORE_POLICY);
+      __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, mm[k]), bm, e0 * 4, 0, ADAM_STORE_POLICY);
+      __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, vv[k]), bv, e0 * 4, 0, ADAM_STORE_POLICY);
+      if (HAS_PLOW) {
+        if (PSZ == 2) {
+          u32x2 w;
+          w[0] = (uint32_t)pl[0] | ((uint32_t)pl[1] << 16);
+          w[1] = (uint32_t)pl[2] | ((uint32_t)pl[3] << 16);
+          __builtin_amdgcn_raw_buffer_store_b64(w, bl, e0 * 2, 0, ADAM_STORE_POLICY);
+        } else {
+          u32x4 w;
 #pragma unroll
-      for (int k = 0; k < ADAM_VECS; ++k) fetch(k);
-#pragma unroll
-      for (int k = 0; k < ADAM_VECS; ++k) update(k);
-    } else {
-#pragma unroll
-      for (int k = 0; k < ADAM_VECS; ++k)
-        if (tid + k * ADAM_THREADS < nvec) fetch(k);
-#pragma unroll
-      for (int k = 0; k < ADAM_VECS; ++k)
-        if (tid + k * ADAM_THREADS < nvec) update(k);
+          for (int e = 0; e < 4; ++e) w[e] = (uint32_t)pl[e];
+          __builtin_amdgcn_raw_buffer_store_b128(w, bl, e0 * 4, 0, ADAM_STORE_POLICY);
+        }
+      }
+    }
     }
     const int64_t tail = rg.begin + (int64_t)nvec * ADAM_VEC;
     if (tail + tid < rg.end) one(tail + tid);
