@@ -621,11 +621,19 @@ __global__ void __launch_bounds__(MT_THREADS)
 }
 
 // ------------------------------------------------------------- probes ------
-// Plain streaming kernels in the pattern that measured fastest for a copy on MI355X (one
-// 16-byte vector per lane, one workgroup per 4 KiB, non-temporal loads and stores: 6.6 TB/s
-// against 5.6..5.8 with four vectors per lane and 4.7..5.2 with resident workgroups that
-// stride): what the memory system gives a read, a fill and a copy on this GPU, measured
-// beside the optimizer step by benchmarks.
+// Plain streaming kernels, each in the pattern that measured fastest for it on MI355X: what
+// the memory system gives a read, a fill and a copy on this GPU, measured beside the
+// optimizer step by benchmarks.  One 16-byte vector per lane and a wave that ends behind it
+// in all three (four vectors per lane: 5.6 to 5.8 TB/s for a copy, resident workgroups that
+// stride: 4.7 to 5.2); stores non-temporal and written through like the update kernel's.
+//   read  256-lane workgroups, every wave the registers allow resident: 7.1 TB/s
+//   fill  256-lane workgroups, 24 waves per CU (26.5 KB of LDS reserved per workgroup):
+//         7.3 TB/s (7.0 with plain non-temporal stores, 6.8 with 32 waves)
+//   copy  one-wave workgroups, all resident: 6.8 TB/s (256-lane workgroups 6.5 to 6.7)
+constexpr int PROBE_FILL_LDS = 27136;
+__device__ __forceinline__ void store_through(f32x4 x, f32x4* p) {
+  asm volatile("global_store_dwordx4 %0, %1, off sc1 nt" ::"v"(p), "v"(x) : "memory");
+}
 __global__ void __launch_bounds__(MT_THREADS)
     probe_read_kernel(const f32x4* __restrict__ src, int64_t nvec, float* sink) {
   const int64_t i = (int64_t)blockIdx.x * MT_THREADS + threadIdx.x;
@@ -637,12 +645,12 @@ __global__ void __launch_bounds__(MT_THREADS)
 __global__ void __launch_bounds__(MT_THREADS)
     probe_fill_kernel(f32x4* __restrict__ dst, int64_t nvec) {
   const int64_t i = (int64_t)blockIdx.x * MT_THREADS + threadIdx.x;
-  if (i < nvec) dst[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+  if (i < nvec) store_through(f32x4{0.f, 0.f, 0.f, 0.f}, dst + i);
 }
-__global__ void __launch_bounds__(MT_THREADS)
+__global__ void __launch_bounds__(64)
     probe_copy_kernel(const f32x4* src, f32x4* dst, int64_t nvec) {
-  const int64_t i = (int64_t)blockIdx.x * MT_THREADS + threadIdx.x;
-  if (i < nvec) st<true>(ld<true>(src + i), dst + i);
+  const int64_t i = (int64_t)blockIdx.x * 64 + threadIdx.x;
+  if (i < nvec) store_through(ld<true>(src + i), dst + i);
 }
 
 // ------------------------------------------------------------- host side ----
@@ -940,19 +948,20 @@ int launch_mt_adam(const void* const* h_g, void* const* h_p, void* const* h_m,
 int launch_stream_probe(int kind, const void* src, void* dst, size_t bytes, hipStream_t stream) {
   const int64_t nvec = (int64_t)(bytes / 16);
   if (nvec == 0) return AXN_OK;
-  const long long blocks = (nvec + MT_THREADS - 1) / MT_THREADS;
+  const int lanes = kind == AXN_PROBE_COPY ? 64 : MT_THREADS;
+  const long long blocks = (nvec + lanes - 1) / lanes;
   if (blocks > 0x7fffffffLL) {
-    set_error("axn_stream_probe: at most %lld bytes per call", 0x7fffffffLL * MT_THREADS * 16);
+    set_error("axn_stream_probe: at most %lld bytes per call", 0x7fffffffLL * lanes * 16);
     return AXN_ELIMIT;
   }
-  const dim3 grid((unsigned)blocks), block(MT_THREADS);
+  const dim3 grid((unsigned)blocks), block(lanes);
   switch (kind) {
     case AXN_PROBE_READ:
       hipLaunchKernelGGL(probe_read_kernel, grid, block, 0, stream, (const f32x4*)src, nvec,
                          (float*)dst);
       break;
     case AXN_PROBE_FILL:
-      hipLaunchKernelGGL(probe_fill_kernel, grid, block, 0, stream, (f32x4*)dst, nvec);
+      hipLaunchKernelGGL(probe_fill_kernel, grid, block, PROBE_FILL_LDS, stream, (f32x4*)dst, nvec);
       break;
     default:
       hipLaunchKernelGGL(probe_copy_kernel, grid, block, 0, stream, (const f32x4*)src, (f32x4*)dst,

@@ -393,9 +393,9 @@ AXN_API int axn_mt_scale(void* const* h_g, const int64_t* h_sizes, int64_t n,
 
 /* ------------------------------------------------------------------------
  * Measurement aid, no counterpart in the reference: plain streaming kernels (one 16-byte
- * vector per lane, one workgroup per 4 KiB, non-temporal accesses - the pattern that
- * measured fastest for a copy), so that a benchmark can put the optimizer step's rate
- * beside what the memory system of the same GPU gives a plain read, fill or copy.
+ * vector per lane, non-temporal accesses, each in the launch shape that measured fastest
+ * for it), so that a benchmark can put the optimizer step's rate beside what the memory
+ * system of the same GPU gives a plain read, fill or copy.
  *   AXN_PROBE_READ: reads `bytes` from src (dst: 4 writable bytes, never written for
  *                   finite data); AXN_PROBE_FILL: writes `bytes` of zeros to dst;
  *   AXN_PROBE_COPY: copies `bytes` from src to dst (src == dst: in place).

@@ -636,3 +636,30 @@ def test_order_zero_counts_gradients_with_a_nonzero_element():
     assert float(get_total_norm(gs, 0.0)) == 2.0
     want = torch.norm(torch.stack([torch.norm(g, 0.0) for g in gs]), 0.0)
     assert float(want) == 2.0
+
+
+def test_stream_probes_read_fill_copy():
+    """The yardstick kernels of the benchmarks do what they are timed for: a copy equals its
+    source (also in place, also over a ragged number of 16-byte vectors), a fill writes zeros
+    and nothing behind the given bytes, a read writes nothing."""
+    import ctypes
+
+    from axonn_amd import _native as nv
+
+    lib = nv.load()
+    stream = nv.current_stream()
+    for n in (4, 1000, 64 * 4 * 1000 + 12, 1 << 22):   # floats
+        g = torch.Generator(device="cuda").manual_seed(n)
+        src = torch.randn(n + 8, generator=g, device="cuda")
+        dst = torch.full((n + 8,), 7.0, device="cuda")
+        nbytes = n * 4
+        nv.check(lib.axn_stream_probe(2, src.data_ptr(), dst.data_ptr(), nbytes, stream))
+        assert torch.equal(dst[:n], src[:n]) and bool((dst[n:] == 7.0).all())
+        keep = src.clone()
+        nv.check(lib.axn_stream_probe(2, src.data_ptr(), src.data_ptr(), nbytes, stream))
+        assert torch.equal(src, keep)
+        sink = torch.full((4,), 3.0, device="cuda")
+        nv.check(lib.axn_stream_probe(0, src.data_ptr(), sink.data_ptr(), nbytes, stream))
+        assert torch.equal(src, keep) and bool((sink == 3.0).all())
+        nv.check(lib.axn_stream_probe(1, None, dst.data_ptr(), nbytes, stream))
+        assert bool((dst[:n] == 0.0).all()) and bool((dst[n:] == 7.0).all())
