@@ -41,7 +41,9 @@ constexpr int EW_BAND = AXN_EW_BAND;  // rows per workgroup (dGELU + dbias: colu
 // SwiGLU has no sums to carry down the rows: one row piece per wave, the workgroups handed
 // out in row-major order, so that the chip reads and writes one compact window of every
 // operand (4096 x 14336 bf16 from HBM: forward 76 -> 59 us, backward 131 -> 98 us against
-// 128-row bands, measured on MI355X).
+// 128-row bands, measured on MI355X).  Stores written through (nt + sc1), which gain 1 to
+// 2 % in the optimizer's update kernel, change nothing in the forward and lose 6 % in the
+// backward (two outputs): plain stores.
 constexpr int SWIGLU_BAND = AXN_SWIGLU_BAND;
 
 // 8 consecutive columns as floats, for bf16 / fp16 (16 bytes) and fp32 (32 bytes) rows.
