@@ -632,7 +632,9 @@ __global__ void __launch_bounds__(MT_THREADS)
 //   copy  one-wave workgroups, all resident: 6.8 TB/s (256-lane workgroups 6.5 to 6.7)
 constexpr int PROBE_FILL_LDS = 27136;
 __device__ __forceinline__ void store_through(f32x4 x, f32x4* p) {
-  asm volatile("global_store_dwordx4 %0, %1, off sc1 nt" ::"v"(p), "v"(x) : "memory");
+  // s_nop: the wait states a store of more than 8 bytes needs before its data registers
+  // may be written again, which the compiler inserts for its own stores only
+  asm volatile("global_store_dwordx4 %0, %1, off sc1 nt\n\ts_nop 1" ::"v"(p), "v"(x) : "memory");
 }
 __global__ void __launch_bounds__(MT_THREADS)
     probe_read_kernel(const f32x4* __restrict__ src, int64_t nvec, float* sink) {

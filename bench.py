@@ -281,6 +281,7 @@ def main():
     del layers
     torch.cuda.empty_cache()
     if not args.no_extra_shapes:
+        P = lambda t: t.data_ptr()  # noqa: E731
         if want("mlp_shard"):
             # 12B-style MLP shard: bias + GELU fused, dW accumulated over 4 micro-batches
             L = Layer("mlp_shard", 8192, 5120, 2560, 10, torch, bias=True)
@@ -348,7 +349,6 @@ def main():
             dact, dgt, dup = (torch.empty(Mt, I, **bf) for _ in range(3))
             y, dx1, dx2 = (torch.empty(Mt, H, **bf) for _ in range(3))
             dwg, dwu, dwd = torch.empty(I, H, **bf), torch.empty(I, H, **bf), torch.empty(H, I, **bf)
-            P = lambda t: t.data_ptr()  # noqa: E731
 
             def gate_up_three_calls():
                 chk = nv.check
