@@ -79,3 +79,55 @@ def test_main_loop_mfma_operands_have_fixed_register_classes(gemm_asm):
                 ops = [o.strip() for o in s.split(None, 1)[1].split(",")]
                 assert ops[0].startswith("a[") and ops[3].startswith("a[") and ops[0] == ops[3], (name, s)
                 assert ops[1].startswith("v[") and ops[2].startswith("v["), (name, s)
+
+
+def _device_asm(tmp_path_factory, name):
+    if not os.path.exists(HIPCC):
+        pytest.skip("hipcc not available")
+    out = tmp_path_factory.mktemp("asm") / (name + ".s")
+    src = os.path.join(ROOT, "axonn_amd", "csrc", name + ".hip")
+    cmd = [HIPCC, "--offload-arch=gfx950", "-O3", "-std=c++17", "-Xclang", "-target-feature", "-Xclang",
+           "-packed-fp32-ops", "-I" + os.path.join(ROOT, "include"), "-I" + os.path.dirname(src),
+           "--cuda-device-only", "-S", src, "-o", str(out)]
+    subprocess.run(cmd, check=True, capture_output=True, timeout=900)
+    text = out.read_text()
+    kernels = {}
+    for m in re.finditer(r"^(_ZN3axn\S+):\s", text, re.M):
+        end = text.find(".end_amdhsa_kernel", m.end())
+        if end > 0 and ".amdhsa_kernel" in text[m.end():end]:
+            kernels[m.group(1)] = text[m.end():end]
+    return kernels
+
+
+@pytest.mark.parametrize("source", ["optim", "embedding"])
+def test_hand_written_stores_are_followed_by_their_wait_states(tmp_path_factory, source):
+    """A store of more than 8 bytes needs wait states before its data registers are written
+    again.  The compiler inserts them for its own stores, not for a store inside an asm
+    statement: each of those carries its own s_nop."""
+    kernels = _device_asm(tmp_path_factory, source)
+    seen = 0
+    for name, body in kernels.items():
+        ins = _instructions(body)
+        for i, s_ in enumerate(ins):
+            if s_.startswith("global_store_dwordx4") and "sc1 nt" in s_:
+                # (only the asm statements write "sc1 nt"; the compiler prints "nt sc1")
+                seen += 1
+                assert ins[i + 1].startswith("s_nop"), (name, s_, ins[i + 1])
+    assert seen > 0, source
+
+
+def test_update_kernel_streams_through_buffer_accesses_without_scratch(tmp_path_factory):
+    """The optimizer's update kernel: no spills, every streaming access a buffer access with
+    its cache policy (loads nt, stores nt sc1), all loads of the vector path ahead of the
+    first store."""
+    kernels = {k: v for k, v in _device_asm(tmp_path_factory, "optim").items() if "mt_adam_kernel" in k}
+    assert len(kernels) == 18, sorted(kernels)   # 3 gradient types x (no copy, bf16, fp16) x with/without scan result
+    for name, body in kernels.items():
+        assert re.search(r"\.amdhsa_private_segment_fixed_size 0\b", body), name
+        ins = _instructions(body)
+        loads = [i for i, s_ in enumerate(ins) if s_.startswith("buffer_load_dwordx")]
+        stores = [i for i, s_ in enumerate(ins) if s_.startswith("buffer_store_dwordx")]
+        assert len(loads) == 4 and len(stores) in (3, 4), (name, len(loads), len(stores))
+        assert max(loads) < min(stores), name
+        assert all(ins[i].endswith(" nt") for i in loads), name
+        assert all(ins[i].endswith(" nt sc1") for i in stores), name
