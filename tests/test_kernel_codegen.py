@@ -81,7 +81,12 @@ def test_main_loop_mfma_operands_have_fixed_register_classes(gemm_asm):
                 assert ops[1].startswith("v[") and ops[2].startswith("v["), (name, s)
 
 
+_ASM_CACHE = {}
+
+
 def _device_asm(tmp_path_factory, name):
+    if name in _ASM_CACHE:
+        return _ASM_CACHE[name]
     if not os.path.exists(HIPCC):
         pytest.skip("hipcc not available")
     out = tmp_path_factory.mktemp("asm") / (name + ".s")
@@ -96,6 +101,7 @@ def _device_asm(tmp_path_factory, name):
         end = text.find(".end_amdhsa_kernel", m.end())
         if end > 0 and ".amdhsa_kernel" in text[m.end():end]:
             kernels[m.group(1)] = text[m.end():end]
+    _ASM_CACHE[name] = kernels
     return kernels
 
 
