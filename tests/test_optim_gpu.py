@@ -92,7 +92,7 @@ def test_step_matches_oracle_ragged_layouts(sizes, start):
 def test_every_row_of_the_tensor_table_is_found(count):
     """The update kernel finds a chunk's tensor in two steps (a quarter of the 64-row table,
     then a row of it): tensor counts on both sides of every quarter, tensors of less than
-    one chunk, of exactly one (1024 elements), and of several with a ragged end, and more
+    one chunk, of exactly one (256 elements), and of several with a ragged end, and more
     tensors than one launch holds."""
     rng = np.random.default_rng(count)
     sizes = [int(rng.choice([1, 5, 255, 256, 1023, 1024, 1025, 2048, 4097, 5000])) for _ in range(count)]
