@@ -21,7 +21,7 @@ AXN_ELIMIT = -5
 BF16, F16, F32 = 0, 1, 2
 EPI_NONE, EPI_BIAS, EPI_BIAS_GELU, EPI_GELU = 0, 1, 2, 3
 
-ABI_VERSION = 11
+ABI_VERSION = 12
 
 # Every symbol include/axn.h declares: name -> (restype, argtypes)
 _c = ctypes
@@ -54,11 +54,12 @@ SYMBOLS = {
     "axn_gemm_wgrad": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _int, _int, _vp]),
     "axn_gemm_fwd_f16": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _int,
                                 _vp]),
+    "axn_gemm_fwd_f32out": (_int, [_vp, _vp, _vp, _vp, _vp, _int, _i64, _i64, _i64, _i64, _i64, _i64,
+                                   _int, _vp]),
     "axn_gemm_dgrad_f16": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _vp]),
     "axn_gemm_wgrad_f16": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _int, _int,
                                   _vp]),
     "axn_gemm_workspace_bytes": (_sz, [_int, _i64, _i64, _i64]),
-    "axn_gemm_set_shared_tiles": (_int, [_int]),
     "axn_gemm_fwd_ws": (_int, [_vp, _vp, _vp, _vp, _vp, _int, _i64, _i64, _i64, _i64, _i64, _i64, _int,
                                _vp, _sz, _vp]),
     "axn_gemm_dgrad_ws": (_int, [_vp, _vp, _vp, _int, _i64, _i64, _i64, _i64, _i64, _i64, _vp, _sz,
@@ -87,10 +88,10 @@ SYMBOLS = {
     "axn_mt_adam": (_int, [_pp, _pp, _pp, _pp, _pp, _pi64, _i64, _int, _int, _f32, _vp,
                            _c.POINTER(AdamHParams), _vp]),
     "axn_mt_scale": (_int, [_pp, _pi64, _i64, _int, _f32, _vp, _int, _vp]),
-    "axn_stream_probe": (_int, [_int, _vp, _vp, _sz, _vp]),
 }
 
 _lib = None
+_probe_lib = None
 _lock = threading.Lock()
 
 
@@ -138,6 +139,22 @@ def load():
             )
         _lib = lib
     return _lib
+
+
+def load_probe():
+    """The benchmark-only library of streaming yardsticks (include/axn_probe.h)."""
+    global _probe_lib
+    if _probe_lib is None:
+        path = os.path.join(os.path.dirname(_LIB_PATH), "libaxn_probe_gfx950.so")
+        if not os.path.exists(path):
+            raise ImportError("libaxn_probe_gfx950.so is not built (expected at %s); run "
+                              "`python -m axonn_amd.csrc.build`" % path)
+        load()  # binds the HIP runtime torch uses first
+        lib = ctypes.CDLL(path)
+        lib.axn_probe_stream.restype = _int
+        lib.axn_probe_stream.argtypes = [_int, _vp, _vp, _sz, _vp]
+        _probe_lib = lib
+    return _probe_lib
 
 
 def check(rc):

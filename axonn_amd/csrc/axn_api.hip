@@ -119,11 +119,15 @@ const char* axn_last_error(void) { return g_err; }
 // The 16-bit GEMM entry points: `half` selects IEEE half instead of bfloat16.
 static int gemm_fwd_16(const char* name, bool half, const void* X, const void* W,
                        const float* bias, void* Y, void* Zsave, int64_t M, int64_t N, int64_t K,
-                       int64_t ldx, int64_t ldw, int64_t ldy, int epilogue, void* stream) {
+                       int64_t ldx, int64_t ldw, int64_t ldy, int epilogue, void* stream,
+                       bool y_f32 = false) {
   int rc = check_gemm(name, X, W, Y, M, N, K, ldx, ldw, ldy, K, K, N);
   if (rc) return rc;
   rc = check_epilogue(name, epilogue, bias);
   if (rc) return rc;
+  REQUIRE(!y_f32 || epilogue == AXN_EPI_BIAS || epilogue == AXN_EPI_BIAS_GELU, AXN_EINVAL,
+          "%s: an fp32 result is the promotion of an fp32 bias: epilogue must be BIAS or BIAS_GELU",
+          name);
   REQUIRE(Zsave == nullptr || aligned16(Zsave), AXN_EALIGN, "%s: Zsave must be 16-byte aligned",
           name);
   GemmArgs g = {};
@@ -139,8 +143,8 @@ static int gemm_fwd_16(const char* name, bool half, const void* X, const void* W
   g.ldb = ldw;
   g.ldc = ldy;
   g.beta = 0;
-  return half ? launch_gemm_f16(GEMM_NT, g, epilogue, false, (hipStream_t)stream)
-              : launch_gemm_bf16(GEMM_NT, g, epilogue, false, (hipStream_t)stream);
+  return half ? launch_gemm_f16(GEMM_NT, g, epilogue, y_f32, (hipStream_t)stream)
+              : launch_gemm_bf16(GEMM_NT, g, epilogue, y_f32, (hipStream_t)stream);
 }
 
 static int gemm_dgrad_16(const char* name, bool half, const void* dY, const void* W, void* dX,
@@ -193,6 +197,15 @@ int axn_gemm_fwd(const void* X, const void* W, const float* bias, void* Y,
                  int64_t ldw, int64_t ldy, int epilogue, void* stream) {
   return gemm_fwd_16("axn_gemm_fwd", false, X, W, bias, Y, Zsave, M, N, K, ldx, ldw, ldy,
                      epilogue, stream);
+}
+
+int axn_gemm_fwd_f32out(const void* X, const void* W, const float* bias, float* Y, void* Zsave,
+                        int dtype, int64_t M, int64_t N, int64_t K, int64_t ldx, int64_t ldw,
+                        int64_t ldy, int epilogue, void* stream) {
+  const char* name = "axn_gemm_fwd_f32out";
+  REQUIRE(dtype == AXN_BF16 || dtype == AXN_F16, AXN_EINVAL, "%s: dtype must be bf16 or fp16", name);
+  return gemm_fwd_16(name, dtype == AXN_F16, X, W, bias, Y, Zsave, M, N, K, ldx, ldw, ldy, epilogue,
+                     stream, true);
 }
 
 int axn_gemm_dgrad(const void* dY, const void* W, void* dX, int64_t M, int64_t N,
@@ -255,12 +268,9 @@ size_t axn_gemm_workspace_bytes(int op, int64_t M, int64_t N, int64_t K) {
   // dense operands: the leading dimensions are the row lengths
   fill_gemm_args(g, op, nullptr, nullptr, nullptr, M, N, K, op == AXN_GEMM_FWD ? K : N, K,
                  op == AXN_GEMM_FWD ? N : K);
-  if (gemm_streamk_applies(kLayoutOfOp[op], g)) return gemm_streamk_workspace();
   const int s = gemm_splits(kLayoutOfOp[op], g);
   return s > 1 ? (size_t)s * (size_t)g.M * (size_t)g.N * sizeof(float) : 0;
 }
-
-int axn_gemm_set_shared_tiles(int enable) { return gemm_streamk_set_policy(enable); }
 
 static int gemm_ws(const char* name, int op, const void* a, const void* b, void* c, int dtype,
                    int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc, int beta,
@@ -283,15 +293,6 @@ static int gemm_ws(const char* name, int op, const void* a, const void* b, void*
   g.bias = bias;
   g.Z = (uint16_t*)zsave;
   const GemmLayout layout = kLayoutOfOp[op];
-  if (workspace != nullptr && gemm_streamk_applies(layout, g)) {
-    // shares of (tile, stage) units, one workgroup per CU: no partly filled last round
-    const size_t need = gemm_streamk_workspace();
-    REQUIRE(workspace_bytes >= need, AXN_EINVAL,
-            "%s: workspace too small (%zu bytes given, %zu needed)", name, workspace_bytes, need);
-    REQUIRE(aligned16(workspace), AXN_EALIGN, "%s: workspace must be 16-byte aligned", name);
-    return launch_gemm_streamk(layout, g, half, epilogue, out_dtype == AXN_F32, workspace,
-                               (hipStream_t)stream);
-  }
   bool wide_tiles = false;
   const int splits =
       (workspace != nullptr && epilogue == AXN_EPI_NONE) ? gemm_splits(layout, g, &wide_tiles) : 1;
@@ -575,8 +576,7 @@ int check_scan_args(const char* name, const void* const* h_g, const int64_t* h_s
   REQUIRE(n == 0 || h_g != nullptr, AXN_EINVAL, "%s: null pointer array", name);
   REQUIRE(result != nullptr, AXN_EINVAL, "%s: result is null", name);
   REQUIRE(((uintptr_t)result & 7u) == 0, AXN_EALIGN, "%s: result must be 8-byte aligned", name);
-  REQUIRE(std::isfinite(norm_type), AXN_EINVAL,
-          "%s: the norm's order must be finite (got %g)", name, (double)norm_type);
+  REQUIRE(norm_type == norm_type, AXN_EINVAL, "%s: the norm's order is NaN", name);
   rc = check_list(name, h_g, "g", h_sizes, n, g_dtype == AXN_F32 ? 4 : 2);
   if (rc) return rc;
   REQUIRE(accumulate == 0 || accumulate == 1, AXN_EINVAL, "%s: accumulate must be 0 or 1", name);
@@ -614,17 +614,6 @@ int axn_mt_scan_noalloc(const void* const* h_g, const int64_t* h_sizes, int64_t 
   if (rc) return rc;
   return launch_mt_scan_noalloc(h_g, h_sizes, n, g_dtype, inv_scale, max_norm, 2.0f, accumulate,
                                 result, (hipStream_t)stream);
-}
-
-int axn_stream_probe(int kind, const void* src, void* dst, size_t bytes, void* stream) {
-  const char* name = "axn_stream_probe";
-  REQUIRE(kind == AXN_PROBE_READ || kind == AXN_PROBE_FILL || kind == AXN_PROBE_COPY, AXN_EINVAL,
-          "%s: unknown kind %d", name, kind);
-  REQUIRE(dst != nullptr, AXN_EINVAL, "%s: dst is null", name);
-  REQUIRE(kind == AXN_PROBE_FILL || src != nullptr, AXN_EINVAL, "%s: src is null", name);
-  REQUIRE(((uintptr_t)src & 15u) == 0 && ((uintptr_t)dst & (kind == AXN_PROBE_READ ? 3u : 15u)) == 0,
-          AXN_EALIGN, "%s: pointers must be 16-byte aligned", name);
-  return launch_stream_probe(kind, src, dst, bytes, (hipStream_t)stream);
 }
 
 int axn_mt_adam(const void* const* h_g, void* const* h_p, void* const* h_m,

@@ -106,15 +106,6 @@ struct GemmArgs {
   // the leading dimensions of A and B.
   const uint16_t* A2;
   int k_first;
-  // Shares of (tile, stage) units instead of whole tiles (launch_gemm_streamk): fp32
-  // partial sums of a tile that two or more workgroups share go through sk_partials (one
-  // slot of 256 x 256 floats per workgroup), handed over with one flag per wave that is
-  // set to sk_token, a value no earlier launch has used; sk_error is set if a flag does
-  // not arrive within the bounded wait.
-  float* sk_partials;
-  unsigned long long* sk_flags;
-  unsigned long long sk_token;
-  int* sk_error;
 };
 
 enum GemmLayout { GEMM_NT = 0, GEMM_NN = 1, GEMM_TN = 2 };
@@ -134,14 +125,6 @@ int launch_gemm_f16(GemmLayout layout, const GemmArgs& args, int epilogue, bool 
 // adds them in split order, adds the old output if args.beta, and stores args.C in
 // out_dtype.  No epilogue.
 int gemm_splits(GemmLayout layout, const GemmArgs& args, bool* wide_tiles = nullptr);
-// One workgroup per CU, each with an equal share of the problem's (256 x 256 tile, 64-deep
-// stage) units (see solo_gemm): whether a problem is run that way, the workspace it needs,
-// and the launch (epilogues as launch_gemm_bf16; ws as sized by gemm_streamk_workspace).
-bool gemm_streamk_applies(GemmLayout layout, const GemmArgs& args);
-int gemm_streamk_set_policy(int policy);   // 0: never, otherwise wherever it can run; returns the old value
-size_t gemm_streamk_workspace();
-int launch_gemm_streamk(GemmLayout layout, const GemmArgs& args, bool half, int epilogue,
-                        bool out_f32, void* ws, hipStream_t stream);
 int launch_gemm_splitk(GemmLayout layout, const GemmArgs& args, bool half, int out_dtype,
                        int splits, bool wide_tiles, float* ws, hipStream_t stream);
 
@@ -206,7 +189,5 @@ int launch_mt_scale(void* const* h_g, const int64_t* h_sizes, int64_t n,
                     int g_dtype, float inv_scale, const axn_scan_result* scan,
                     int use_clip, hipStream_t stream);
 
-// Streaming yardsticks (axn_stream_probe).
-int launch_stream_probe(int kind, const void* src, void* dst, size_t bytes, hipStream_t stream);
 
 }  // namespace axn

@@ -1,4 +1,5 @@
-"""Builds libaxn_gfx950.so from the HIP sources in this directory.
+"""Builds libaxn_gfx950.so (the product library) and libaxn_probe_gfx950.so (streaming
+yardsticks for benchmarks, include/axn_probe.h) from the HIP sources in this directory.
 
     python -m axonn_amd.csrc.build
 
@@ -16,9 +17,11 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(os.path.dirname(HERE))
 LIB_DIR = os.path.join(os.path.dirname(HERE), "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libaxn_gfx950.so")
+PROBE_LIB_PATH = os.path.join(LIB_DIR, "libaxn_probe_gfx950.so")
 OBJ_DIR = os.path.join(HERE, "build")
 
 SOURCES = ["axn_api.hip", "gemm_bf16.hip", "gemm_f32.hip", "elementwise.hip", "embedding.hip", "optim.hip"]
+PROBE_SOURCES = ["stream_probe.hip"]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 
@@ -61,11 +64,13 @@ def build_library(verbose=False, extra_flags=()):
             print(out)
         return obj
 
-    with ThreadPoolExecutor(max_workers=min(len(SOURCES), os.cpu_count() or 1)) as pool:
-        objs = list(pool.map(compile_one, SOURCES))
-    out = _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", *objs, "-o", LIB_PATH])
-    if verbose and out.strip():
-        print(out)
+    every = SOURCES + PROBE_SOURCES
+    with ThreadPoolExecutor(max_workers=min(len(every), os.cpu_count() or 1)) as pool:
+        objs = list(pool.map(compile_one, every))
+    for path, part in ((LIB_PATH, objs[:len(SOURCES)]), (PROBE_LIB_PATH, objs[len(SOURCES):])):
+        out = _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", *part, "-o", path])
+        if verbose and out.strip():
+            print(out)
     return LIB_PATH
 
 

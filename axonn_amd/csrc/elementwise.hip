@@ -25,26 +25,18 @@ typedef __attribute__((ext_vector_type(4))) float f32x4;
 constexpr int EW_TX = 64;          // lanes along columns (8 columns each)
 constexpr int EW_TY = 4;           // row phases per workgroup
 constexpr int EW_COLS = EW_TX * 8; // 512 columns per workgroup
-#ifndef AXN_EW_BAND
-#define AXN_EW_BAND 128
-#endif
+constexpr int EW_BAND = 128;       // rows per workgroup (dGELU + dbias: column sums per band)
 // Non-temporal loads of dY and Z: 12 % faster when the operands come from HBM (62 -> 55 us),
 // 12 % slower when the memory-side cache holds them, which is the case in a training step
 // (dY was written by the layer behind a moment ago): off.
-#ifndef AXN_DGELU_NT
-#define AXN_DGELU_NT 0
-#endif
-constexpr int EW_BAND = AXN_EW_BAND;  // rows per workgroup (dGELU + dbias: column sums per band)
-#ifndef AXN_SWIGLU_BAND
-#define AXN_SWIGLU_BAND 4
-#endif
+constexpr bool DGELU_NT = false;
 // SwiGLU has no sums to carry down the rows: one row piece per wave, the workgroups handed
 // out in row-major order, so that the chip reads and writes one compact window of every
 // operand (4096 x 14336 bf16 from HBM: forward 76 -> 59 us, backward 131 -> 98 us against
 // 128-row bands, measured on MI355X).  Stores written through (nt + sc1), which gain 1 to
 // 2 % in the optimizer's update kernel, change nothing in the forward and lose 6 % in the
 // backward (two outputs): plain stores.
-constexpr int SWIGLU_BAND = AXN_SWIGLU_BAND;
+constexpr int SWIGLU_BAND = 4;
 
 // 8 consecutive columns as floats, for bf16 / fp16 (16 bytes) and fp32 (32 bytes) rows.
 // NT: non-temporal loads, for operands read once.  They are worth 15 % on the SwiGLU
@@ -107,7 +99,7 @@ template <> struct Raw8<_Float16> { typedef f16x8 type; };
 template <> struct Raw8<float> { struct type { f32x4 lo, hi; }; };
 template <typename T>
 __device__ __forceinline__ typename Raw8<T>::type load_raw8(const T* p) {
-  if constexpr (AXN_DGELU_NT != 0 && sizeof(T) == 2) {
+  if constexpr (DGELU_NT && sizeof(T) == 2) {
     return __builtin_nontemporal_load((const typename Raw8<T>::type*)p);
   } else {
     return *(const typename Raw8<T>::type*)p;

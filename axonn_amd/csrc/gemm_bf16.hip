@@ -37,10 +37,6 @@
 // bounds checks, one barrier per step, epilogue transposed through LDS; ragged shapes,
 // contractions that are not multiples of 64, operands of 2 GiB and more.
 #include <atomic>
-#include <chrono>
-#include <cstdlib>
-#include <cstring>
-#include <random>
 #include <utility>
 
 #include "axn_internal.h"
@@ -66,14 +62,6 @@ constexpr int EPI_SWIGLU = 100;
 // Internal: no epilogue, but the contraction runs through two operand pairs one after the
 // other (C = A B + A2 B2).
 constexpr int EPI_PAIR = 101;
-// Written to the workspace's error word (byte 16320) by a workgroup whose bounded wait for
-// another's partial sums ran out; nothing else ever writes that word.
-constexpr int SK_TIMED_OUT = (int)0xBAD0BAD0u;
-// Cache policy of the partial sums' stores and loads (sc0 | sc1: system scope - write
-// through to memory, read from memory), so that handing them from one XCD to another needs
-// neither a write-back nor an invalidation of an L2.
-constexpr int SK_PAST_CACHES = 1 | 16;
-
 #define LDS_PTR(T, p) ((__attribute__((address_space(3))) T*)(p))
 
 template <int... I, class F>
@@ -502,21 +490,7 @@ __device__ __forceinline__ void wait_vmcnt() {
 // rounds of 256 x 256 tiles: a rest of r <= 128 large tiles makes 2 r <= 256 of these,
 // one per CU, and needs 3/4 of the global -> LDS bytes per MFMA of the 128 x 128 tile.
 // Its ring has five slots of the larger (A) tile's size.
-// STREAMK: the launch is one workgroup per CU for a problem of k whole rounds of tiles and
-// half a round more.  A workgroup walks its tile of every whole round like the plain
-// kernel's workgroups do (the tiles in flight at any time are neighbours: they share
-// operand panels in their XCD's L2), and the tiles of the half round are each shared by two
-// workgroups, so that the problem ends without a half-empty round.  The first workgroup of
-// a pair (on an XCD 0..3) computes the tile's first stages before anything else (fp32
-// partial sums to its slot of the workspace, a flag per wave released behind them); the
-// second (same index on the XCD four further) computes the other stages after its whole
-// tiles, with accumulators that start from those partial sums instead of zero, and runs
-// the epilogue - the same additions in the same order as one workgroup would make.  A
-// workgroup only ever waits for the workgroup four indices below it, which the dispatcher
-// starts before it and which computes what is waited for first: no wait can be circular,
-// and nothing depends on timing.
-template <int BM, int BN, bool A_KMAJOR, bool B_KMAJOR, int EPI, bool OUT_F32, bool HALF,
-          bool STREAMK = false>
+template <int BM, int BN, bool A_KMAJOR, bool B_KMAJOR, int EPI, bool OUT_F32, bool HALF>
 __device__ __forceinline__ void solo_gemm(const GemmArgs& g) {
   constexpr int WTM = BM / 2, WTN = BN / 2, FRM = BM / 32, FRN = BN / 32;
   constexpr int PK = 64, NSLOT = 5;
@@ -543,9 +517,6 @@ __device__ __forceinline__ void solo_gemm(const GemmArgs& g) {
   static_assert(!PAIR || (A_KMAJOR && !B_KMAJOR), "the two-term product is the dgrad layout");
   static_assert(!SWIGLU || (BM == 256 && BN == 256 && A_KMAJOR && B_KMAJOR && !OUT_F32),
                 "the gate/up forward runs on the 256 x 256 tile with contraction-contiguous operands");
-  static_assert(!STREAMK || (!SWIGLU && !PAIR), "shares of stages: plain products only");
-  constexpr int CHUNKS = FRM * (FRN / 2);          // 8-column pieces of a lane's part of the tile
-  constexpr int SLOT_FLOATS = BM * BN;             // one workgroup's partial sums
 
   extern __shared__ __attribute__((aligned(16))) char lds[];
 
@@ -692,261 +663,104 @@ __device__ __forceinline__ void solo_gemm(const GemmArgs& g) {
   using T = std::true_type;
   using F = std::false_type;
 
-  // ---- what this workgroup computes -------------------------------------------------
-  // A segment: KP stages of tile (tm, tn) from stage s0 on.
-  enum SegMode { SEG_FULL = 0, SEG_PRODUCE = 1, SEG_OWN = 2 };
-  int tm = 0, tn = 0, s0 = 0, KP = 0, mode = SEG_FULL, split = 0;
-  // STREAMK: the XCD's first tile, its whole rounds (workgroup l of the XCD's sk_wpx takes
-  // tile r * sk_wpx + l of round r) and the rest of sk_rem = sk_wpx / 2 tiles behind them.
-  // The 2 sk_rem rest tiles of the XCDs x < 4 and x + 4 are shared by the workgroups l of
-  // those two XCDs: x's computes the stages [0, KT / 2) first of all (partial sums to the
-  // workspace), x + 4's the other stages last of all, from those sums on.  All workgroups
-  // of an XCD thus stay in step with each other (the tiles they work on share operand
-  // panels in the XCD's L2 only while they walk the contraction together); the XCDs 0..3
-  // run half a tile ahead of 4..7.
-  int sk_tile0 = 0, sk_wpx = 1, sk_l = 0, sk_xcd = 0, sk_phase = 0, sk_round = 0, sk_rounds = 0, sk_rem = 0;
-  const int KT = g.Kc / PK;   // stages of a whole tile
-  if constexpr (STREAMK) {
-    sk_xcd = blockIdx.x % NUM_XCD;
-    sk_l = blockIdx.x / NUM_XCD;
-    sk_wpx = gridDim.x / NUM_XCD;
-    const int mine = g.tiles_m * g.tiles_n / NUM_XCD;   // the launch sees to it: a multiple of NUM_XCD
-    sk_tile0 = sk_xcd * mine;
-    sk_rounds = mine / sk_wpx;
-    sk_rem = mine - sk_rounds * sk_wpx;                  // 0 or sk_wpx / 2
+  // This workgroup's tile and, for a split contraction, its part: KP stages from stage s0 on.
+  int tm, tn, split = 0;
+  {
+    int pid = blockIdx.x;
+    if (g.splits > 1) {
+      split = pid / (g.tiles_m * g.tiles_n);
+      pid -= split * (g.tiles_m * g.tiles_n);
+    }
+    tile_of_workgroup(pid, g.tiles_m, g.tiles_n, tm, tn);
   }
-  // tile t of the band order -> (tm, tn)
-  auto tile_coords = [&](int t) {
-    constexpr int GROUP_M = 8;
-    const int in_group = GROUP_M * g.tiles_n;
-    const int group = t / in_group;
-    const int first_m = group * GROUP_M;
-    const int gsz = (g.tiles_m - first_m < GROUP_M) ? g.tiles_m - first_m : GROUP_M;
-    const int r = t - group * in_group;
-    tm = first_m + r % gsz;
-    tn = r / gsz;
-  };
-  auto next_segment = [&]() -> bool {
-    if constexpr (!STREAMK) {
-      if (sk_phase++ != 0) return false;
-      int pid = blockIdx.x;
-      if (g.splits > 1) {
-        split = pid / (g.tiles_m * g.tiles_n);
-        pid -= split * (g.tiles_m * g.tiles_n);
-      }
-      tile_of_workgroup(pid, g.tiles_m, g.tiles_n, tm, tn);
-      KP = (g.splits > 1 ? g.k_split : g.Kc) / PK;
-      s0 = split * KP;
-      mode = SEG_FULL;
-      return true;
-    } else {
-      const bool shares = sk_rem > 0;
-      const bool producer = shares && sk_xcd < NUM_XCD / 2;
-      // the shared tile of workgroup l of the XCDs x and x + 4: tile l of x's half round for
-      // l < sk_rem, tile l - sk_rem of x + 4's otherwise
-      const int sk_shared = ((sk_xcd & (NUM_XCD / 2 - 1)) + (sk_l < sk_rem ? 0 : NUM_XCD / 2)) *
-                                (sk_rounds * sk_wpx + sk_rem) + sk_rounds * sk_wpx +
-                            (sk_l < sk_rem ? sk_l : sk_l - sk_rem);
-      if (sk_phase == 0) {
-        sk_phase = 1;
-        if (producer) {   // the earlier stages of the shared tile, before anything else
-          tile_coords(sk_shared);
-          s0 = 0;
-          KP = KT / 2;
-          mode = SEG_PRODUCE;
-          return true;
-        }
-      }
-      if (sk_round < sk_rounds) {
-        tile_coords(sk_tile0 + sk_round * sk_wpx + sk_l);
-        ++sk_round;
-        s0 = 0;
-        KP = KT;
-        mode = SEG_FULL;
-        return true;
-      }
-      if (sk_phase == 1) {
-        sk_phase = 2;
-        if (shares && !producer) {   // the later stages, last: the partial sums are long there
-          tile_coords(sk_shared);
-          s0 = KT / 2;
-          KP = KT - s0;
-          mode = SEG_OWN;
-          return true;
-        }
-      }
-      return false;
-    }
-  };
+  const int KP = (g.splits > 1 ? g.k_split : g.Kc) / PK;
+  const int s0 = split * KP;
+  const int m0 = tm * BM, n0 = tn * (SWIGLU ? BN / 2 : BN);
+  va = OA::dma_offset(g.lda, m0, wave, lane, a_is);
+  vb = OB::dma_offset(g.ldb, n0, wave, lane, b_is);
+  ka = (uint32_t)s0 * a_step;
+  kb = (uint32_t)s0 * b_step;
 
-  bool first_segment = true;
-  while (next_segment()) {
-    const int m0 = tm * BM, n0 = tn * (SWIGLU ? BN / 2 : BN);
-    if constexpr (STREAMK) {
-      // every wave has read its last fragments of the previous segment before the ring is
-      // filled again
-      if (!first_segment) {
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the previous segment's stores have left
-        __builtin_amdgcn_s_barrier();
-      }
-      first_segment = false;
-    }
-    va = OA::dma_offset(g.lda, m0, wave, lane, a_is);
-    vb = OB::dma_offset(g.ldb, n0, wave, lane, b_is);
-    ka = (uint32_t)s0 * a_step;
-    kb = (uint32_t)s0 * b_step;
-    wslot = 0;
-    sa = 0;
-    sb = SLOT;
-
-    if constexpr (STREAMK) if (mode == SEG_OWN) {
-      // The tile's earlier stages are in the slot of the workgroup before this one: wait
-      // for this wave's flag (a bounded wait: a flag that never comes is reported and the
-      // kernel still ends) and let the accumulators start from those sums, requested ahead
-      // of the first operand tiles.
-      const int slot = (sk_xcd - NUM_XCD / 2) * sk_wpx + sk_l;
-      const unsigned long long* flag = g.sk_flags + slot * 4 + wave;
-      int spins = 0;
-      while (__hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != g.sk_token) {
-        __builtin_amdgcn_s_sleep(8);
-        if (++spins > (1 << 24)) {
-          if (lane == 0) *g.sk_error = SK_TIMED_OUT;
-          break;
-        }
-      }
-      // The partial sums were stored past the caches (below) and are loaded past them: no
-      // cache of this XCD, which its other workgroups' operand panels live in, is
-      // invalidated.  The statement keeps the loads behind the wait.
-      asm volatile("" ::: "memory");
-      // (compiler-visible loads: it places the waits before whatever it does with the
-      // registers; buffer addressing keeps the address arithmetic out of the registers)
-      const __amdgpu_buffer_rsrc_t prs = __builtin_amdgcn_make_buffer_rsrc(
-          (void*)(g.sk_partials + (int64_t)slot * SLOT_FLOATS + wave * (CHUNKS * 64 * 8)), 0,
-          CHUNKS * 64 * 8 * 4, 0x00020000);
-      const int lofs = lane * 32;
-#pragma unroll
-      for (int i = 0; i < FRM; ++i)
-#pragma unroll
-        for (int j = 0; j < FRN; ++j) {
-          // the piece as stored: 8 columns = blocks 2 t and 2 t + 1 of row block i
-          const int so = (i * (FRN / 2) + j / 2) * (64 * 8 * 4);
-          acc[i][j] = __builtin_bit_cast(
-              f32x4, __builtin_amdgcn_raw_buffer_load_b128(prs, lofs + (j % 2) * 16, so, SK_PAST_CACHES));
-        }
-    }
-    // A0 B0 (A1 B1) up front.
+  // A0 B0 (A1 B1) up front.
+  static_for<NCA>(copy_a); a_done();
+  static_for<NCB>(copy_b); b_done();
+  if (KP > 1) {
     static_for<NCA>(copy_a); a_done();
     static_for<NCB>(copy_b); b_done();
-    if (KP > 1) {
-      static_for<NCA>(copy_a); a_done();
-      static_for<NCB>(copy_b); b_done();
-    }
-    // The accumulators are cleared here, while the first tiles are on their way: left
-    // to itself the compiler clears them where they are first used, behind the wait.
-    if (!(STREAMK && mode == SEG_OWN)) {
+  }
+  // The accumulators are cleared here, while the first tiles are on their way: left
+  // to itself the compiler clears them where they are first used, behind the wait.
 #pragma unroll
-      for (int i = 0; i < FRM; ++i)
+  for (int i = 0; i < FRM; ++i)
 #pragma unroll
-        for (int j = 0; j < FRN; ++j) acc[i][j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-    }
+    for (int j = 0; j < FRN; ++j) acc[i][j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-    for (int i = 0; i < FRM; ++i) settle_accumulators(acc[i]);
-    if (KP > 1) {
-      wait_vmcnt<NCA + NCB>();
-    } else {
-      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    }
-    __builtin_amdgcn_s_barrier();
+  for (int i = 0; i < FRM; ++i) settle_accumulators(acc[i]);
+  if (KP > 1) {
+    wait_vmcnt<NCA + NCB>();
+  } else {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  }
+  __builtin_amdgcn_s_barrier();
 
-    static_for<NFRAG>([&](auto f_) { read(std::integral_constant<int, 0>{}, f_, sa, sb); });
+  static_for<NFRAG>([&](auto f_) { read(std::integral_constant<int, 0>{}, f_, sa, sb); });
 
-    if constexpr (PAIR) {
-      const int kp1 = g.k_first / PK;  // >= 2: the stages copied up front are of the first pair
-      const uint32_t b2_bytes = (uint32_t)((int64_t)(g.Kc - g.k_first) * g.ldb * 2);
-      for (int p = 0; p < KP - 2; ++p) {
-        if (p == kp1 - 2) {  // this stage copies the tiles of stage kp1, the second pair's first
-          ra_cur = __builtin_amdgcn_make_buffer_rsrc((void*)g.A2, 0, (int)a_bytes, 0x00020000);
-          rb_cur = __builtin_amdgcn_make_buffer_rsrc((void*)g.B2, 0, (int)b2_bytes, 0x00020000);
-          ka = 0;
-          kb = 0;
-        }
-        stage(T{}, F{});
+  if constexpr (PAIR) {
+    const int kp1 = g.k_first / PK;  // >= 2: the stages copied up front are of the first pair
+    const uint32_t b2_bytes = (uint32_t)((int64_t)(g.Kc - g.k_first) * g.ldb * 2);
+    for (int p = 0; p < KP - 2; ++p) {
+      if (p == kp1 - 2) {  // this stage copies the tiles of stage kp1, the second pair's first
+        ra_cur = __builtin_amdgcn_make_buffer_rsrc((void*)g.A2, 0, (int)a_bytes, 0x00020000);
+        rb_cur = __builtin_amdgcn_make_buffer_rsrc((void*)g.B2, 0, (int)b2_bytes, 0x00020000);
+        ka = 0;
+        kb = 0;
       }
-    } else {
-      for (int p = 0; p < KP - 2; ++p) stage(T{}, F{});
+      stage(T{}, F{});
     }
-    if (KP > 1) stage(F{}, F{});
-    stage(F{}, T{});
-    // The compiler does not know that the statements above are MFMAs: left alone it
-    // copies an accumulator out of its AGPRs right behind the MFMA that writes it,
-    // before the result has left the pipeline.  Every accumulator is therefore
-    // passed through a statement that follows the last MFMA by more than its
-    // latency; the epilogue can only read the values these statements return.
-    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+  } else {
+    for (int p = 0; p < KP - 2; ++p) stage(T{}, F{});
+  }
+  if (KP > 1) stage(F{}, F{});
+  stage(F{}, T{});
+  // The compiler does not know that the statements above are MFMAs: left alone it
+  // copies an accumulator out of its AGPRs right behind the MFMA that writes it,
+  // before the result has left the pipeline.  Every accumulator is therefore
+  // passed through a statement that follows the last MFMA by more than its
+  // latency; the epilogue can only read the values these statements return.
+  asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
 #pragma unroll
-    for (int i = 0; i < FRM; ++i) settle_accumulators(acc[i]);
-    // With the permuted column fragments a lane owns, per block row i and block
-    // pair t, the 8 consecutive columns 32 t + 8 (l / 16) .. + 7 of row 16 i + l % 16:
-    // they go out straight from the registers, 64 contiguous bytes per row and
-    // instruction.
-    const int orow = m0 + wm * WTM + (lane & 15);
-    const int ocol = n0 + wn * WTN + 8 * (lane >> 4);
-    if constexpr (SWIGLU) {
-      // blocks 0..3 of a lane's row hold 64 gate columns, blocks 4..7 the up values of the
-      // same columns
-      const int hcol = n0 + wn * (WTN / 2) + 8 * (lane >> 4);
+  for (int i = 0; i < FRM; ++i) settle_accumulators(acc[i]);
+  // With the permuted column fragments a lane owns, per block row i and block
+  // pair t, the 8 consecutive columns 32 t + 8 (l / 16) .. + 7 of row 16 i + l % 16:
+  // they go out straight from the registers, 64 contiguous bytes per row and
+  // instruction.
+  const int orow = m0 + wm * WTM + (lane & 15);
+  const int ocol = n0 + wn * WTN + 8 * (lane >> 4);
+  if constexpr (SWIGLU) {
+    // blocks 0..3 of a lane's row hold 64 gate columns, blocks 4..7 the up values of the
+    // same columns
+    const int hcol = n0 + wn * (WTN / 2) + 8 * (lane >> 4);
 #pragma unroll
-      for (int i = 0; i < FRM; ++i)
+    for (int i = 0; i < FRM; ++i)
 #pragma unroll
-        for (int t = 0; t < FRN / 4; ++t) {
-          const f32x4 gl = acc[i][2 * t], gh = acc[i][2 * t + 1];
-          const f32x4 ul = acc[i][2 * t + FRN / 2], uh = acc[i][2 * t + 1 + FRN / 2];
-          const float vg[8] = {gl[0], gl[1], gl[2], gl[3], gh[0], gh[1], gh[2], gh[3]};
-          const float vu[8] = {ul[0], ul[1], ul[2], ul[3], uh[0], uh[1], uh[2], uh[3]};
-          store_swiglu8<HALF>(vg, vu, g, orow + 16 * i, hcol + 32 * t);
-        }
-    } else if (STREAMK && mode == SEG_PRODUCE) {
-      // partial sums to this workgroup's slot, in the order a lane holds them (32 bytes per
-      // lane and piece, a wave writes 2 KiB in a row), then this wave's flag
-      // (buffer addressing: one descriptor per wave, the lane's offset in one register, the
-      // piece in the instruction's scalar offset - no 64-bit address per piece to keep)
-      const int slot = sk_xcd * sk_wpx + sk_l;
-      const __amdgpu_buffer_rsrc_t prs = __builtin_amdgcn_make_buffer_rsrc(
-          (void*)(g.sk_partials + (int64_t)slot * SLOT_FLOATS + wave * (CHUNKS * 64 * 8)), 0,
-          CHUNKS * 64 * 8 * 4, 0x00020000);
-      const int lofs = lane * 32;
-#pragma unroll
-      for (int i = 0; i < FRM; ++i) {
-#pragma unroll
-        for (int t = 0; t < FRN / 2; ++t) {
-          constexpr int PIECE = 64 * 8 * 4;
-          const int c = i * (FRN / 2) + t;
-          __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, acc[i][2 * t]), prs, lofs,
-                                                 c * PIECE, SK_PAST_CACHES);
-          __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, acc[i][2 * t + 1]), prs, lofs + 16,
-                                                 c * PIECE, SK_PAST_CACHES);
-        }
-        __builtin_amdgcn_sched_barrier(0);   // row block by row block: few registers in flight
+      for (int t = 0; t < FRN / 4; ++t) {
+        const f32x4 gl = acc[i][2 * t], gh = acc[i][2 * t + 1];
+        const f32x4 ul = acc[i][2 * t + FRN / 2], uh = acc[i][2 * t + 1 + FRN / 2];
+        const float vg[8] = {gl[0], gl[1], gl[2], gl[3], gh[0], gh[1], gh[2], gh[3]};
+        const float vu[8] = {ul[0], ul[1], ul[2], ul[3], uh[0], uh[1], uh[2], uh[3]};
+        store_swiglu8<HALF>(vg, vu, g, orow + 16 * i, hcol + 32 * t);
       }
-      // the flag becomes visible after the sums: the stores go through to memory (no
-      // write-back of this XCD's L2 is needed to publish them), the wave waits until all
-      // of its lanes' stores are acknowledged, then lane 0 sets the flag
-      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-      if (lane == 0)
-        __hip_atomic_store(g.sk_flags + slot * 4 + wave, g.sk_token, __ATOMIC_RELAXED,
-                           __HIP_MEMORY_SCOPE_AGENT);
-    } else {
-      GemmArgs go = g;  // a split writes its own fp32 partial product
-      if (OUT_F32 && !STREAMK && g.splits > 1) go.C = (float*)g.C + (int64_t)split * g.M * g.ldc;
+  } else {
+    GemmArgs go = g;  // a split writes its own fp32 partial product
+    if (OUT_F32 && g.splits > 1) go.C = (float*)g.C + (int64_t)split * g.M * g.ldc;
 #pragma unroll
-      for (int i = 0; i < FRM; ++i)
+    for (int i = 0; i < FRM; ++i)
 #pragma unroll
-        for (int t = 0; t < FRN / 2; ++t) {
-          const f32x4 lo = acc[i][2 * t], hi = acc[i][2 * t + 1];
-          float v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-          store_row8<(PAIR ? (int)AXN_EPI_NONE : EPI), OUT_F32, HALF>(v, go, orow + 16 * i, ocol + 32 * t);
-        }
-    }
+      for (int t = 0; t < FRN / 2; ++t) {
+        const f32x4 lo = acc[i][2 * t], hi = acc[i][2 * t + 1];
+        float v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        store_row8<(PAIR ? (int)AXN_EPI_NONE : EPI), OUT_F32, HALF>(v, go, orow + 16 * i, ocol + 32 * t);
+      }
   }
 }
 
@@ -957,15 +771,6 @@ __global__ void __launch_bounds__(256) gemm_bf16_solo_kernel(const GemmArgs g) {
 template <int TILE, bool A_KMAJOR, bool B_KMAJOR, int EPI, bool OUT_F32>
 __global__ void __launch_bounds__(256) gemm_f16_solo_kernel(const GemmArgs g) {
   solo_gemm<TILE, TILE, A_KMAJOR, B_KMAJOR, EPI, OUT_F32, true>(g);
-}
-// 256 x 256 tiles, one workgroup per CU with an equal share of the (tile, stage) units.
-template <bool A_KMAJOR, bool B_KMAJOR, int EPI, bool OUT_F32>
-__global__ void __launch_bounds__(256) gemm_bf16_streamk_kernel(const GemmArgs g) {
-  solo_gemm<256, 256, A_KMAJOR, B_KMAJOR, EPI, OUT_F32, false, true>(g);
-}
-template <bool A_KMAJOR, bool B_KMAJOR, int EPI, bool OUT_F32>
-__global__ void __launch_bounds__(256) gemm_f16_streamk_kernel(const GemmArgs g) {
-  solo_gemm<256, 256, A_KMAJOR, B_KMAJOR, EPI, OUT_F32, true, true>(g);
 }
 // The 256 x 128 tile of the launches that finish a problem.
 template <bool A_KMAJOR, bool B_KMAJOR, int EPI, bool OUT_F32>
@@ -1325,7 +1130,12 @@ int launch_layout(GemmLayout layout, const GemmArgs& g, int epilogue, bool out_f
                   hipStream_t stream) {
   switch (layout) {
     case GEMM_NT:
-      if (out_f32) break;
+      if (out_f32) {  // 16-bit product + fp32 bias promoted to fp32, as `x + bias` promotes it
+        if (epilogue == AXN_EPI_BIAS) return launch_shape<true, true, AXN_EPI_BIAS, true, HALF>(g, stream);
+        if (epilogue == AXN_EPI_BIAS_GELU)
+          return launch_shape<true, true, AXN_EPI_BIAS_GELU, true, HALF>(g, stream);
+        break;
+      }
       switch (epilogue) {
         case AXN_EPI_NONE:
           return launch_shape<true, true, AXN_EPI_NONE, false, HALF>(g, stream);
@@ -1390,117 +1200,6 @@ int launch_gemm_swiglu(const GemmArgs& in, bool half, hipStream_t stream) {
                      stream, g);
   AXN_HIP_TRY(hipGetLastError());
   return AXN_OK;
-}
-
-// ---- shares of stages --------------------------------------------------------------
-namespace {
-constexpr int SK_WGS = 256;                          // one per CU of the part
-constexpr size_t SK_HEADER = 16384;                  // flags (256 x 4 x 8 bytes) and the error word
-constexpr size_t SK_SLOT = 256 * 256 * sizeof(float);
-
-// 0: never (the default: measured on MI355X the scheme is 0..10 % slower than whole rounds
-// plus a launch for the rest on every shape of the benchmark sets - the part runs these
-// kernels power-limited, and the half-empty round it removes was paid back as clock), 1: on
-// every problem the kernel can run.  AXN_GEMM_STREAMK in the environment sets the start
-// value, gemm_streamk_set_policy changes it.
-std::atomic<int>& streamk_policy_ref() {
-  static std::atomic<int> policy{[] {
-    const char* e = getenv("AXN_GEMM_STREAMK");
-    return (e != nullptr && (!strcmp(e, "always") || !strcmp(e, "1"))) ? 1 : 0;
-  }()};
-  return policy;
-}
-int streamk_policy() { return streamk_policy_ref().load(std::memory_order_relaxed); }
-
-// A value no launch of this or an earlier process has handed out: a random 64-bit start
-// (so that flags left in recycled device memory cannot match) plus a counter.
-unsigned long long next_token() {
-  static std::atomic<unsigned long long> counter{[] {
-    std::random_device rd;
-    unsigned long long v = ((unsigned long long)rd() << 32) ^ rd();
-    v ^= (unsigned long long)std::chrono::steady_clock::now().time_since_epoch().count() * 0x9E3779B97F4A7C15ull;
-    return v | 1ull;
-  }()};
-  return counter.fetch_add(1, std::memory_order_relaxed);
-}
-
-template <bool AK, bool BKM, int EPI, bool OUT_F32, bool HALF>
-int launch_streamk(const GemmArgs& in, void* ws, hipStream_t stream) {
-  GemmArgs g = in;
-  g.tiles_m = g.M / 256;
-  g.tiles_n = g.N / 256;
-  g.splits = 0;
-  g.sk_flags = (unsigned long long*)ws;
-  g.sk_error = (int*)((char*)ws + SK_HEADER - 64);
-  g.sk_partials = (float*)((char*)ws + SK_HEADER);
-  g.sk_token = next_token();
-  constexpr size_t lds = 5 * 256 * 64 * 2;
-  void (*kern)(const GemmArgs) = gemm_bf16_streamk_kernel<AK, BKM, EPI, OUT_F32>;
-  if constexpr (HALF) kern = gemm_f16_streamk_kernel<AK, BKM, EPI, OUT_F32>;
-  {
-    static std::atomic<unsigned long long> lds_allowed{0};   // per template instance
-    const int rc = allow_lds((const void*)kern, lds, lds_allowed);
-    if (rc != AXN_OK) return rc;
-  }
-  hipLaunchKernelGGL(kern, dim3(SK_WGS), dim3(256), lds, stream, g);
-  AXN_HIP_TRY(hipGetLastError());
-  return AXN_OK;
-}
-
-template <bool HALF>
-int launch_streamk_layout(GemmLayout layout, const GemmArgs& g, int epilogue, bool out_f32, void* ws,
-                          hipStream_t stream) {
-  switch (layout) {
-    case GEMM_NT:
-      if (out_f32) break;
-      switch (epilogue) {
-        case AXN_EPI_NONE: return launch_streamk<true, true, AXN_EPI_NONE, false, HALF>(g, ws, stream);
-        case AXN_EPI_BIAS: return launch_streamk<true, true, AXN_EPI_BIAS, false, HALF>(g, ws, stream);
-        case AXN_EPI_BIAS_GELU:
-          return launch_streamk<true, true, AXN_EPI_BIAS_GELU, false, HALF>(g, ws, stream);
-        case AXN_EPI_GELU: return launch_streamk<true, true, AXN_EPI_GELU, false, HALF>(g, ws, stream);
-      }
-      break;
-    case GEMM_NN:
-      if (out_f32 || epilogue != AXN_EPI_NONE) break;
-      return launch_streamk<true, false, AXN_EPI_NONE, false, HALF>(g, ws, stream);
-    case GEMM_TN:
-      if (epilogue != AXN_EPI_NONE) break;
-      return out_f32 ? launch_streamk<false, false, AXN_EPI_NONE, true, HALF>(g, ws, stream)
-                     : launch_streamk<false, false, AXN_EPI_NONE, false, HALF>(g, ws, stream);
-  }
-  set_error("gemm: unsupported layout/epilogue/output combination");
-  return AXN_EINVAL;
-}
-}  // namespace
-
-size_t gemm_streamk_workspace() { return SK_HEADER + (size_t)SK_WGS * SK_SLOT; }
-
-int gemm_streamk_set_policy(int policy) {
-  return streamk_policy_ref().exchange(policy != 0 ? 1 : 0, std::memory_order_relaxed);
-}
-
-bool gemm_streamk_applies(GemmLayout layout, const GemmArgs& g) {
-  const int policy = streamk_policy();
-  if (policy == 0) return false;
-  if (g.M % 256 || g.N % 256 || g.Kc % 64) return false;
-  const bool ak = layout != GEMM_TN, bkm = layout == GEMM_NT;
-  const int64_t a_span = (int64_t)(ak ? g.M : g.Kc) * g.lda * 2;
-  const int64_t b_span = (int64_t)(bkm ? g.N : g.Kc) * g.ldb * 2;
-  if (a_span >= (1LL << 31) || b_span >= (1LL << 31)) return false;
-  const long long tiles = (long long)(g.M / 256) * (g.N / 256);
-  // The kernel takes whole rounds of tiles plus a rest of exactly half a round on every
-  // XCD (each of those tiles goes to a pair of workgroups), contractions of two stages or more.
-  if (tiles > (1 << 24) || tiles % NUM_XCD != 0 || g.Kc < 128) return false;
-  const long long mine = tiles / NUM_XCD, wpx = SK_WGS / NUM_XCD;
-  if (mine % wpx != wpx / 2) return false;
-  return true;
-}
-
-int launch_gemm_streamk(GemmLayout layout, const GemmArgs& g, bool half, int epilogue, bool out_f32,
-                        void* ws, hipStream_t stream) {
-  return half ? launch_streamk_layout<true>(layout, g, epilogue, out_f32, ws, stream)
-              : launch_streamk_layout<false>(layout, g, epilogue, out_f32, ws, stream);
 }
 
 int launch_gemm_bf16(GemmLayout layout, const GemmArgs& g, int epilogue,

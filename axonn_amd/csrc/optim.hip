@@ -29,27 +29,6 @@
 namespace axn {
 namespace {
 
-#ifndef AXN_SCAN_CHUNK
-#define AXN_SCAN_CHUNK 65536
-#endif
-#ifndef AXN_ADAM_THREADS
-#define AXN_ADAM_THREADS 64
-#endif
-#ifndef AXN_ADAM_VECS
-#define AXN_ADAM_VECS 1
-#endif
-#define AXN_ADAM_CHUNK (AXN_ADAM_THREADS * 4 * AXN_ADAM_VECS)
-#ifndef AXN_ADAM_LDS
-#define AXN_ADAM_LDS 15360
-#endif
-// Cache policy bits of the update kernel's buffer accesses (1 sc0, 2 nt, 16 sc1).
-#ifndef AXN_ADAM_LOAD_POLICY
-#define AXN_ADAM_LOAD_POLICY 2
-#endif
-#ifndef AXN_ADAM_STORE_POLICY
-#define AXN_ADAM_STORE_POLICY 18
-#endif
-
 constexpr int MT_MAX = 64;         // tensors per launch
 constexpr int MT_THREADS = 256;    // threads per workgroup
 constexpr int MT_VEC = 8;          // elements per lane per step
@@ -57,18 +36,19 @@ constexpr int MT_VEC = 8;          // elements per lane per step
 // non-temporal loads; the read-modify-write update does best with one-wave workgroups
 // that make one trip of ADAM_VECS 4-element vectors per lane (see mt_adam_kernel).  Both
 // measured on MI355X.
-constexpr int SCAN_CHUNK = AXN_SCAN_CHUNK;
-constexpr int ADAM_CHUNK = AXN_ADAM_CHUNK;
+constexpr int SCAN_CHUNK = 65536;
 constexpr int SCALE_CHUNK = 16384;
 constexpr int ADAM_VEC = 4;                     // elements per vector of the update kernel
-constexpr int ADAM_THREADS = AXN_ADAM_THREADS;  // lanes per workgroup of the update kernel
-constexpr int ADAM_VECS = AXN_ADAM_VECS;        // vectors per lane
+constexpr int ADAM_THREADS = 64;                // lanes per workgroup of the update kernel
+constexpr int ADAM_VECS = 1;                    // vectors per lane
+constexpr int ADAM_CHUNK = ADAM_THREADS * ADAM_VEC * ADAM_VECS;
 // LDS the update kernel reserves per workgroup and never touches: it bounds the
 // workgroups that are resident on a CU (160 KB per CU), see mt_adam_kernel.
-constexpr int ADAM_LDS = AXN_ADAM_LDS;
-// Loads non-temporal; stores non-temporal and written through (nt + sc1): 1 to 2 % over
-// nt alone, 10 % over plain stores, measured on MI355X.
-constexpr int ADAM_LOAD_POLICY = AXN_ADAM_LOAD_POLICY, ADAM_STORE_POLICY = AXN_ADAM_STORE_POLICY;
+constexpr int ADAM_LDS = 15360;
+// Cache policy bits of the update kernel's buffer accesses (1 sc0, 2 nt, 16 sc1).  Loads
+// non-temporal; stores non-temporal and written through (nt + sc1): 1 to 2 % over nt
+// alone, 10 % over plain stores, measured on MI355X.
+constexpr int ADAM_LOAD_POLICY = 2, ADAM_STORE_POLICY = 2 | 16;
 static_assert(ADAM_THREADS >= 64 && ADAM_THREADS % 64 == 0, "a tensor's scalar head (up to 63 elements) is one element per lane");
 static_assert(ADAM_CHUNK % MT_VEC == 0, "chunks keep the 16-byte alignment of the tensor's body");
 static_assert(ADAM_LDS <= 65536, "dynamic LDS a launch may ask for without a function attribute");
@@ -241,13 +221,26 @@ __device__ __forceinline__ int wave_or(int x) {
 // instructions, order 0 counts the non-zero elements (torch.norm's meaning of p = 0),
 // any other order goes through exp2(p log2 |u|) (|0|^p is 0 for p > 0 and +inf for p < 0,
 // as in torch).
-enum NormMode { NORM_2 = 0, NORM_1 = 1, NORM_0 = 2, NORM_P = 3 };
+// Orders +inf and -inf are the largest and the smallest |u|: their terms are combined by
+// max / min instead of a sum, a NaN staying a NaN as in torch.
+enum NormMode { NORM_2 = 0, NORM_1 = 1, NORM_0 = 2, NORM_P = 3, NORM_MAX = 4, NORM_MIN = 5 };
 template <int MODE>
 __device__ __forceinline__ float norm_term(float u, float p) {
   if (MODE == NORM_2) return u * u;
-  if (MODE == NORM_1) return fabsf(u);
+  if (MODE == NORM_1 || MODE == NORM_MAX || MODE == NORM_MIN) return fabsf(u);
   if (MODE == NORM_0) return u != 0.0f ? 1.0f : 0.0f;
   return powf(fabsf(u), p);
+}
+// How two partial results of a mode meet, and the value that changes nothing.
+template <int MODE, typename T>
+__device__ __forceinline__ T norm_join(T a, T b) {
+  if (MODE == NORM_MAX) return (a >= b || a != a) ? a : b;
+  if (MODE == NORM_MIN) return (a <= b || a != a) ? a : b;
+  return a + b;
+}
+template <int MODE>
+__device__ __forceinline__ float norm_identity() {
+  return MODE == NORM_MIN ? __builtin_inff() : 0.0f;
 }
 
 template <int DT, int MODE>
@@ -261,13 +254,13 @@ __global__ void __launch_bounds__(MT_THREADS)
   const void* g = tab.g[t];
   const int tid = threadIdx.x;
 
-  float sq = 0.f, sm = 0.f;
+  float sq = norm_identity<MODE>(), sm = 0.f;
   int bad = 0;
   auto one = [&](raw x) {
     bad |= Lowp<DT>::nonfinite(x) ? 1 : 0;
     const float f = Lowp<DT>::to_float(x);
     sm += f;
-    sq += norm_term<MODE>(f * inv_scale, norm_type);
+    sq = norm_join<MODE>(sq, norm_term<MODE>(f * inv_scale, norm_type));
   };
   if (vec_ok_of(tab, t)) {
     if (c == 0 && tid < head_of(tab, t)) one(((const raw*)g)[tid]);
@@ -287,7 +280,8 @@ __global__ void __launch_bounds__(MT_THREADS)
 
   __shared__ float s_sq[MT_THREADS / 64], s_sm[MT_THREADS / 64];
   __shared__ int s_bad[MT_THREADS / 64];
-  sq = wave_sum(sq);
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) sq = norm_join<MODE>(sq, __shfl_xor(sq, o, 64));
   sm = wave_sum(sm);
   bad = wave_or(bad);
   if ((tid & 63) == 0) {
@@ -298,12 +292,12 @@ __global__ void __launch_bounds__(MT_THREADS)
   __syncthreads();
   if (tid == 0) {
     ScanPartial p;
-    p.sumsq = 0.f;
+    p.sumsq = norm_identity<MODE>();
     p.sum = 0.f;
     p.nonfinite = 0;
 #pragma unroll
     for (int w = 0; w < MT_THREADS / 64; ++w) {  // fixed order: deterministic
-      p.sumsq += s_sq[w];
+      p.sumsq = norm_join<MODE>(p.sumsq, s_sq[w]);
       p.sum += s_sm[w];
       p.nonfinite |= s_bad[w];
     }
@@ -321,6 +315,7 @@ __device__ __forceinline__ double wave_sum_d(double x) {
 // One workgroup of 1024 threads reduces the partials of one launch group in a
 // fixed order: wave w takes tensors w, w + 16, ...; lanes stride over that
 // tensor's chunks.  `first` initialises the result, later groups accumulate.
+template <int MODE>
 __global__ void __launch_bounds__(1024)
     mt_scan_finalize_kernel(const MtTable tab, const ScanPartial* partial,
                             int block_base, double sum_limit, float max_norm,
@@ -328,26 +323,27 @@ __global__ void __launch_bounds__(1024)
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   __shared__ double s_sq[16];
   __shared__ int s_bad[16];
-  double sq = 0.0;
+  double sq = (double)norm_identity<MODE>();
   int bad = 0;
   for (int t = wave; t < tab.n; t += 16) {
-    double tsq = 0.0, tsm = 0.0;
+    double tsq = (double)norm_identity<MODE>(), tsm = 0.0;
     int tbad = 0;
     for (int b = tab.chunk_start[t] + lane; b < tab.chunk_start[t + 1]; b += 64) {
       const ScanPartial p = partial[block_base + b];
-      tsq += (double)p.sumsq;
+      tsq = norm_join<MODE>(tsq, (double)p.sumsq);
       tsm += (double)p.sum;
       tbad |= p.nonfinite;
     }
-    tsq = wave_sum_d(tsq);
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) tsq = norm_join<MODE>(tsq, __shfl_xor(tsq, o, 64));
     tsm = wave_sum_d(tsm);
     tbad = wave_or(tbad);
     // The tensor's sum, rounded to the gradient dtype, is non-finite.
     if (!(fabs(tsm) < sum_limit)) tbad = 1;
     // order 0: the norm over the stacked per-tensor norms counts the tensors whose own
     // count of non-zero elements is not zero
-    if (norm_type == 0.0f) tsq = tsq != 0.0 ? 1.0 : 0.0;
-    sq += tsq;
+    if (MODE == NORM_0) tsq = tsq != 0.0 ? 1.0 : 0.0;
+    sq = norm_join<MODE>(sq, tsq);
     bad |= tbad;
   }
   if (lane == 0) {
@@ -356,15 +352,15 @@ __global__ void __launch_bounds__(1024)
   }
   __syncthreads();
   if (threadIdx.x == 0) {
-    double total = first ? 0.0 : out->sumsq;
+    double total = first ? (double)norm_identity<MODE>() : out->sumsq;
     int flag = first ? 0 : out->found_inf;
     for (int w = 0; w < 16; ++w) {
-      total += s_sq[w];
+      total = norm_join<MODE>(total, s_sq[w]);
       flag |= s_bad[w];
     }
-    const float norm = norm_type == 2.0f ? (float)sqrt(total)
-                       : norm_type == 1.0f || norm_type == 0.0f ? (float)total
-                       : (float)pow(total, 1.0 / (double)norm_type);
+    const float norm = MODE == NORM_2 ? (float)sqrt(total)
+                       : MODE == NORM_P ? (float)pow(total, 1.0 / (double)norm_type)
+                                        : (float)total;
     float coef = 1.0f;
     if (max_norm > 0.0f) {
       coef = max_norm / (norm + 1e-6f);
@@ -620,41 +616,6 @@ __global__ void __launch_bounds__(MT_THREADS)
   }
 }
 
-// ------------------------------------------------------------- probes ------
-// Plain streaming kernels, each in the pattern that measured fastest for it on MI355X: what
-// the memory system gives a read, a fill and a copy on this GPU, measured beside the
-// optimizer step by benchmarks.  One 16-byte vector per lane and a wave that ends behind it
-// in all three (four vectors per lane: 5.6 to 5.8 TB/s for a copy, resident workgroups that
-// stride: 4.7 to 5.2); stores non-temporal and written through like the update kernel's.
-//   read  256-lane workgroups, every wave the registers allow resident: 7.1 TB/s
-//   fill  256-lane workgroups, 24 waves per CU (26.5 KB of LDS reserved per workgroup):
-//         7.3 TB/s (7.0 with plain non-temporal stores, 6.8 with 32 waves)
-//   copy  one-wave workgroups, all resident: 6.8 TB/s (256-lane workgroups 6.5 to 6.7)
-constexpr int PROBE_FILL_LDS = 27136;
-__device__ __forceinline__ void store_through(f32x4 x, f32x4* p) {
-  // s_nop: the wait states a store of more than 8 bytes needs before its data registers
-  // may be written again, which the compiler inserts for its own stores only
-  asm volatile("global_store_dwordx4 %0, %1, off sc1 nt\n\ts_nop 1" ::"v"(p), "v"(x) : "memory");
-}
-__global__ void __launch_bounds__(MT_THREADS)
-    probe_read_kernel(const f32x4* __restrict__ src, int64_t nvec, float* sink) {
-  const int64_t i = (int64_t)blockIdx.x * MT_THREADS + threadIdx.x;
-  if (i >= nvec) return;
-  const f32x4 x = ld<true>(src + i);
-  // never true for finite data: keeps the load alive without a store per lane
-  if (x[0] + x[1] + x[2] + x[3] == 1.2345678e38f) *sink = x[0];
-}
-__global__ void __launch_bounds__(MT_THREADS)
-    probe_fill_kernel(f32x4* __restrict__ dst, int64_t nvec) {
-  const int64_t i = (int64_t)blockIdx.x * MT_THREADS + threadIdx.x;
-  if (i < nvec) store_through(f32x4{0.f, 0.f, 0.f, 0.f}, dst + i);
-}
-__global__ void __launch_bounds__(64)
-    probe_copy_kernel(const f32x4* src, f32x4* dst, int64_t nvec) {
-  const int64_t i = (int64_t)blockIdx.x * 64 + threadIdx.x;
-  if (i < nvec) store_through(ld<true>(src + i), dst + i);
-}
-
 // ------------------------------------------------------------- host side ----
 int dtype_size(int dt) { return dt == AXN_F32 ? 4 : 2; }
 
@@ -763,22 +724,50 @@ double sum_limit_of(int dt) {
   }
 }
 
+int norm_mode_host(float p) {
+  return p == 2.0f ? NORM_2 : p == 1.0f ? NORM_1 : p == 0.0f ? NORM_0
+         : p == INFINITY ? NORM_MAX : p == -INFINITY ? NORM_MIN : NORM_P;
+}
+
 template <int DT>
 void scan_dispatch(const Group& gr, float inv_scale, float norm_type, ScanPartial* partial,
                    int base, hipStream_t stream) {
   const dim3 grid(gr.blocks), block(MT_THREADS);
-  if (norm_type == 2.0f)
-    hipLaunchKernelGGL((mt_scan_kernel<DT, NORM_2>), grid, block, 0, stream, gr.tab, inv_scale,
-                       norm_type, partial, base);
-  else if (norm_type == 1.0f)
-    hipLaunchKernelGGL((mt_scan_kernel<DT, NORM_1>), grid, block, 0, stream, gr.tab, inv_scale,
-                       norm_type, partial, base);
-  else if (norm_type == 0.0f)
-    hipLaunchKernelGGL((mt_scan_kernel<DT, NORM_0>), grid, block, 0, stream, gr.tab, inv_scale,
-                       norm_type, partial, base);
-  else
-    hipLaunchKernelGGL((mt_scan_kernel<DT, NORM_P>), grid, block, 0, stream, gr.tab, inv_scale,
-                       norm_type, partial, base);
+  switch (norm_mode_host(norm_type)) {
+#define AXN_SCAN_CASE(MODE)                                                                     \
+  case MODE:                                                                                    \
+    hipLaunchKernelGGL((mt_scan_kernel<DT, MODE>), grid, block, 0, stream, gr.tab, inv_scale,   \
+                       norm_type, partial, base);                                               \
+    break;
+    AXN_SCAN_CASE(NORM_2)
+    AXN_SCAN_CASE(NORM_1)
+    AXN_SCAN_CASE(NORM_0)
+    AXN_SCAN_CASE(NORM_MAX)
+    AXN_SCAN_CASE(NORM_MIN)
+    default:
+    AXN_SCAN_CASE(NORM_P)
+#undef AXN_SCAN_CASE
+  }
+}
+
+void finalize_dispatch(const MtTable& tab, const ScanPartial* partial, int base, double sum_limit,
+                       float max_norm, float norm_type, int first, axn_scan_result* result,
+                       hipStream_t stream) {
+  switch (norm_mode_host(norm_type)) {
+#define AXN_FIN_CASE(MODE)                                                                       \
+  case MODE:                                                                                     \
+    hipLaunchKernelGGL(mt_scan_finalize_kernel<MODE>, dim3(1), dim3(1024), 0, stream, tab,       \
+                       partial, base, sum_limit, max_norm, norm_type, first, result);            \
+    break;
+    AXN_FIN_CASE(NORM_2)
+    AXN_FIN_CASE(NORM_1)
+    AXN_FIN_CASE(NORM_0)
+    AXN_FIN_CASE(NORM_MAX)
+    AXN_FIN_CASE(NORM_MIN)
+    default:
+    AXN_FIN_CASE(NORM_P)
+#undef AXN_FIN_CASE
+  }
 }
 
 }  // namespace
@@ -849,9 +838,9 @@ int launch_mt_scan(const void* const* h_g, const int64_t* h_sizes, int64_t n,
     MtTable empty = MtTable();
     empty.n = 0;
     empty.chunk = SCAN_CHUNK;
-    hipLaunchKernelGGL(mt_scan_finalize_kernel, dim3(1), dim3(1024), 0, stream,
-                       empty, partial, 0, sum_limit_of(g_dtype), max_norm, norm_type,
-                       accumulate ? 0 : 1, result);
+    // (nothing scanned and nothing to add to: every order's norm is 0)
+    finalize_dispatch(empty, partial, 0, sum_limit_of(g_dtype), max_norm, accumulate ? norm_type : 2.0f,
+                      accumulate ? 0 : 1, result, stream);
     AXN_HIP_TRY(hipGetLastError());
     return AXN_OK;
   }
@@ -864,9 +853,8 @@ int launch_mt_scan(const void* const* h_g, const int64_t* h_sizes, int64_t n,
       default: scan_dispatch<AXN_F32>(gr, inv_scale, norm_type, partial, base, stream); break;
     }
     AXN_HIP_TRY(hipGetLastError());
-    hipLaunchKernelGGL(mt_scan_finalize_kernel, dim3(1), dim3(1024), 0, stream,
-                       gr.tab, partial, base, sum_limit_of(g_dtype), max_norm, norm_type,
-                       first ? 1 : 0, result);
+    finalize_dispatch(gr.tab, partial, base, sum_limit_of(g_dtype), max_norm, norm_type, first ? 1 : 0,
+                      result, stream);
     AXN_HIP_TRY(hipGetLastError());
     base += gr.blocks;
     first = false;
@@ -945,33 +933,6 @@ int launch_mt_adam(const void* const* h_g, void* const* h_p, void* const* h_m,
       default: return adam_dispatch<AXN_F32>(gr, s, plow_dtype, has_plow, scan, stream);
     }
   });
-}
-
-int launch_stream_probe(int kind, const void* src, void* dst, size_t bytes, hipStream_t stream) {
-  const int64_t nvec = (int64_t)(bytes / 16);
-  if (nvec == 0) return AXN_OK;
-  const int lanes = kind == AXN_PROBE_COPY ? 64 : MT_THREADS;
-  const long long blocks = (nvec + lanes - 1) / lanes;
-  if (blocks > 0x7fffffffLL) {
-    set_error("axn_stream_probe: at most %lld bytes per call", 0x7fffffffLL * lanes * 16);
-    return AXN_ELIMIT;
-  }
-  const dim3 grid((unsigned)blocks), block(lanes);
-  switch (kind) {
-    case AXN_PROBE_READ:
-      hipLaunchKernelGGL(probe_read_kernel, grid, block, 0, stream, (const f32x4*)src, nvec,
-                         (float*)dst);
-      break;
-    case AXN_PROBE_FILL:
-      hipLaunchKernelGGL(probe_fill_kernel, grid, block, PROBE_FILL_LDS, stream, (f32x4*)dst, nvec);
-      break;
-    default:
-      hipLaunchKernelGGL(probe_copy_kernel, grid, block, 0, stream, (const f32x4*)src, (f32x4*)dst,
-                         nvec);
-      break;
-  }
-  AXN_HIP_TRY(hipGetLastError());
-  return AXN_OK;
 }
 
 int launch_mt_scale(void* const* h_g, const int64_t* h_sizes, int64_t n,

@@ -148,7 +148,11 @@ class FusedLinear(Function):
         x = input_.reshape(-1, input_.shape[-1]).to(dt)
         needs_grad = any(ctx.needs_input_grad[:3])
         w = weight.to(dt)
-        output, z = ops.gemm_fwd(x, w, bias=bias, activation=activation, save_z=needs_grad)
+        # An fp32 bias on a 16-bit product (fp32 parameters under autocast) makes the
+        # reference's `x + bias` an fp32 tensor by type promotion (:348): so it is here.
+        out_f32 = bias is not None and bias.dtype == torch.float32 and dt != torch.float32
+        output, z = ops.gemm_fwd(x, w, bias=bias, activation=activation, save_z=needs_grad,
+                                 out_f32=out_f32)
         # the step's cast of an fp32 weight is kept for the backward pass (see AsyncLinear)
         ctx.save_for_backward(x, original_weight, z, w if w.dtype != weight.dtype else None)
         ctx.shape = local_weight_shape

@@ -72,18 +72,19 @@ GEMM_FWD, GEMM_DGRAD, GEMM_WGRAD = 0, 1, 2
 
 def _split_workspace(op, M, N, K, device):
     """Workspace for a GEMM whose contraction the library would divide among workgroups
-    (few output tiles, or a tile count that leaves a partly filled last round), or
-    (None, 0)."""
+    (few output tiles), or (None, 0)."""
     nbytes = nv.load().axn_gemm_workspace_bytes(op, M, N, K)
     if nbytes == 0:
         return None, 0
     return torch.empty(nbytes, dtype=torch.uint8, device=device), nbytes
 
 
-def gemm_fwd(x, w, bias=None, activation=None, save_z=False):
+def gemm_fwd(x, w, bias=None, activation=None, save_z=False, out_f32=False):
     """Y = act(X W^T + b).  x [M,K], w [N,K]; bf16, fp16 or fp32 (both the same).
     Returns (y, z) with z the saved pre-activation (None unless activation and
-    save_z)."""
+    save_z).  out_f32 (16-bit operands with a bias): y is fp32, the sum with the fp32
+    bias left unrounded, as type promotion leaves the reference's `x + bias`
+    (axonn/intra_layer/fully_connected.py:348) under autocast."""
     _require_gpu(x, w, bias)
     if x.dtype != w.dtype:
         raise TypeError("input is %s but weight is %s" % (x.dtype, w.dtype))
@@ -102,16 +103,24 @@ def gemm_fwd(x, w, bias=None, activation=None, save_z=False):
     if M == 0:  # an empty batch: nothing to launch (the library takes M >= 1)
         y = torch.empty((0, N), dtype=x.dtype, device=x.device)
         return y, (torch.empty_like(y) if want_z else None)
+    if out_f32 and (bias is None or x.dtype not in _GEMM16):
+        raise ValueError("out_f32 is the promotion of a 16-bit product by an fp32 bias")
     if _ragged16(x.dtype, N, K):
         bp = None if bias is None else _pad8(bias.reshape(1, -1), 1).reshape(-1)
-        y, z = gemm_fwd(_pad8(x, 1), _pad8(_pad8(w, 1), 0), bp, activation, save_z)
+        y, z = gemm_fwd(_pad8(x, 1), _pad8(_pad8(w, 1), 0), bp, activation, save_z, out_f32)
         return y[:, :N].contiguous(), (None if z is None else z[:, :N].contiguous())
     if x.dtype in _GEMM16:
         x, ldx = _prep_bf16(x)
         w, ldw = _prep_bf16(w)
+        z = torch.empty((M, N), dtype=x.dtype, device=x.device) if want_z else None
+        if out_f32:
+            y = torch.empty((M, N), dtype=torch.float32, device=x.device)
+            nv.call("axn_gemm_fwd_f32out", nv.ptr(x), nv.ptr(w), nv.ptr(bias), nv.ptr(y), nv.ptr(z),
+                    nv.dtype_code(x.dtype), M, N, K, ldx, ldw, N, epi, nv.current_stream())
+            return y, z
         y = torch.empty((M, N), dtype=x.dtype, device=x.device)
-        z = torch.empty_like(y) if want_z else None
-        ws, ws_bytes = _split_workspace(GEMM_FWD, M, N, K, x.device)
+        # (the contraction is only divided for a plain product: an epilogue runs unsplit)
+        ws, ws_bytes = _split_workspace(GEMM_FWD, M, N, K, x.device) if epi == nv.EPI_NONE else (None, 0)
         if ws is not None:
             nv.call("axn_gemm_fwd_ws", nv.ptr(x), nv.ptr(w), nv.ptr(bias), nv.ptr(y), nv.ptr(z),
                     nv.dtype_code(x.dtype), M, N, K, ldx, ldw, N, epi, nv.ptr(ws), ws_bytes,

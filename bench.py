@@ -616,16 +616,20 @@ def bench_adam(args, torch, nv, lib, stream, time_loop):
     a = torch.empty(1 << 30, dtype=torch.float32, device="cuda").normal_()
     b = torch.empty_like(a)
     nb = a.numel() * 4.0
+    probe_lib = nv.load_probe()
+
     def probe(kind, src, dst):
-        return time_loop(lambda: nv.check(lib.axn_stream_probe(kind, src.data_ptr(), dst.data_ptr(),
-                                                               int(nb), stream)), 5, 2)
+        def run():
+            if probe_lib.axn_probe_stream(kind, src.data_ptr(), dst.data_ptr(), int(nb), stream) != 0:
+                raise RuntimeError("axn_probe_stream failed")
+        return time_loop(run, 5, 2)
 
     out["hbm_reference_streams"] = {
         "copy_gbs": round(2 * nb / time_loop(lambda: b.copy_(a), 5, 2) / 1e9, 1),
         "elementwise_1r1w_gbs": round(2 * nb / time_loop(lambda: torch.mul(a, 2.0, out=b), 5, 2) / 1e9, 1),
         "fill_gbs": round(nb / time_loop(lambda: b.fill_(1.0), 5, 2) / 1e9, 1),
         # the library's own plain streams in the optimizer kernels' access pattern
-        # (axn_stream_probe: 16-byte vectors, grid-stride, non-temporal stores)
+        # (libaxn_probe_gfx950.so: 16-byte vectors, one per lane, non-temporal stores)
         "probe_read_gbs": round(nb / probe(0, a, b) / 1e9, 1),
         "probe_fill_gbs": round(nb / probe(1, a, b) / 1e9, 1),
         "probe_copy_gbs": round(2 * nb / probe(2, a, b) / 1e9, 1),

@@ -30,7 +30,7 @@
 extern "C" {
 #endif
 
-#define AXN_ABI_VERSION 11
+#define AXN_ABI_VERSION 12
 
 #if defined(__GNUC__)
 #define AXN_API __attribute__((visibility("default")))
@@ -129,32 +129,31 @@ AXN_API int axn_gemm_wgrad_f16(const void* dY, const void* X, void* dW, int64_t 
                        int64_t N, int64_t K, int64_t lddy, int64_t ldx, int64_t lddw,
                        int beta, int dw_dtype, void* stream);
 
-/* Variants of the three GEMMs that may divide the contraction among workgroups, given
- * a workspace.  No reference counterpart: torch picks such kernels inside its GEMM library.
- *   - A problem whose count of 256 x 256 output tiles is not a multiple of the CU count
- *     ends in a round of tiles that leaves CUs idle.  With a workspace, problems of at
- *     least one tile per CU run as one workgroup per CU with an equal share of the
- *     (tile, 64-deep stage) units each; a tile shared by two workgroups has its earlier
- *     stages' fp32 sums handed over through the workspace (flag per wave, the later
- *     workgroup starts its accumulators from them).  Every sum has an order fixed by the
- *     launch: results are reproducible bit for bit.  All epilogues.
- *   - A problem with few output tiles (a short batch, a narrow shard) leaves most CUs
- *     without work: the contraction is cut into 2, 4 or 8 parts whose fp32 partial
- *     products a second pass adds in a fixed order (epilogue NONE only).
+/* Forward with the result in fp32.  Under autocast the reference's product is 16-bit and
+ * its bias an fp32 parameter, so `x + bias` (fully_connected.py:348) is promoted to fp32:
+ * this is that sum - Y = X W^T + b (AXN_EPI_BIAS) or gelu of it (AXN_EPI_BIAS_GELU; other
+ * epilogues AXN_EINVAL) - added in fp32 to the fp32 accumulators and stored unrounded.
+ *   X, W, Zsave of `dtype` (AXN_BF16 or AXN_F16), bias fp32, Y [M,N] fp32 (ld ldy, a
+ *   multiple of 8); requirements otherwise as axn_gemm_fwd. */
+AXN_API int axn_gemm_fwd_f32out(const void* X, const void* W, const float* bias, float* Y,
+                        void* Zsave, int dtype, int64_t M, int64_t N, int64_t K, int64_t ldx,
+                        int64_t ldw, int64_t ldy, int epilogue, void* stream);
+
+/* Variants of the three GEMMs that divide the contraction among workgroups, given a
+ * workspace.  No reference counterpart: torch picks such kernels inside its GEMM library.
+ *   A problem with few output tiles (a short batch, a narrow shard) leaves most CUs
+ *   without work: the contraction is cut into 2, 4 or 8 parts whose fp32 partial
+ *   products a second pass adds in a fixed order (epilogue NONE only; results are
+ *   reproducible bit for bit).
  *   axn_gemm_workspace_bytes(op, M, N, K): bytes the call below would use for dense
- *   operands, 0 if it would do neither.  op, M, N, K as in the call.
+ *   operands and epilogue NONE, 0 if it would not split.  op, M, N, K as in the call.
  *   axn_gemm_*_ws: arguments as axn_gemm_fwd / _dgrad / _wgrad, plus dtype (AXN_BF16 or
  *   AXN_F16) of the 16-bit operands and results, and the workspace (16-byte aligned, used
  *   by this call alone until it has finished; contents need not be initialised).
- *   workspace == NULL, or a shape that does not profit: the call is the plain GEMM.
- *   The first scheme is OFF unless asked for (axn_gemm_set_shared_tiles(1), or
- *   AXN_GEMM_STREAMK=always in the environment when the library is loaded): on MI355X,
- *   which runs these kernels power-limited, it measured 0..10 % slower than whole rounds
- *   plus a second launch for the rest; it takes problems of k x 256 + 128 tiles, k >= 0. */
+ *   workspace == NULL, an epilogue, or a shape that does not profit: the call is the
+ *   plain GEMM. */
 typedef enum axn_gemm_op { AXN_GEMM_FWD = 0, AXN_GEMM_DGRAD = 1, AXN_GEMM_WGRAD = 2 } axn_gemm_op;
 AXN_API size_t axn_gemm_workspace_bytes(int op, int64_t M, int64_t N, int64_t K);
-/* Process-wide switch of the shared-tile scheme above; returns the previous setting. */
-AXN_API int axn_gemm_set_shared_tiles(int enable);
 AXN_API int axn_gemm_fwd_ws(const void* X, const void* W, const float* bias, void* Y, void* Zsave,
                     int dtype, int64_t M, int64_t N, int64_t K, int64_t ldx, int64_t ldw,
                     int64_t ldy, int epilogue, void* workspace, size_t workspace_bytes,
@@ -319,11 +318,12 @@ AXN_API int axn_mt_scan(const void* const* h_g, const int64_t* h_sizes, int64_t 
                 size_t workspace_bytes, void* stream);
 
 /* The same scan with the norm's order as an argument: total_norm = (sum |g * inv_scale|^p)^(1/p)
- * for any finite p = norm_type, which is what the reference's clipping accepts
+ * for p = norm_type, which is what the reference's get_total_norm accepts
  * (axonn/intra_layer/gradient_normalization.py:18-34 takes torch.norm(g, norm_type) per
  * gradient and the norm_type-norm of those; :74-87 the coefficient).  p = 0 follows
- * torch.norm's meaning there: the number of gradients that have a non-zero element.
- * p = inf is not taken (the reference raises NotImplementedError, :38-39): AXN_EINVAL.
+ * torch.norm's meaning there: the number of gradients that have a non-zero element;
+ * p = +inf / -inf give the largest / smallest |g * inv_scale| (`sumsq` then holds that
+ * value, a NaN element makes it NaN as in torch).  A NaN order: AXN_EINVAL.
  * axn_mt_scan is this call with norm_type = 2.  Calls that accumulate into one result
  * must name the same order. */
 AXN_API int axn_mt_scan_norm(const void* const* h_g, const int64_t* h_sizes, int64_t n,
@@ -390,19 +390,6 @@ AXN_API int axn_mt_adam(const void* const* h_g, void* const* h_p, void* const* h
 AXN_API int axn_mt_scale(void* const* h_g, const int64_t* h_sizes, int64_t n,
                  int g_dtype, float inv_scale, const axn_scan_result* scan,
                  int use_clip, void* stream);
-
-/* ------------------------------------------------------------------------
- * Measurement aid, no counterpart in the reference: plain streaming kernels (one 16-byte
- * vector per lane, non-temporal accesses, each in the launch shape that measured fastest
- * for it), so that a benchmark can put the optimizer step's rate beside what the memory
- * system of the same GPU gives a plain read, fill or copy.
- *   AXN_PROBE_READ: reads `bytes` from src (dst: 4 writable bytes, never written for
- *                   finite data); AXN_PROBE_FILL: writes `bytes` of zeros to dst;
- *   AXN_PROBE_COPY: copies `bytes` from src to dst (src == dst: in place).
- * Pointers 16-byte aligned; bytes is rounded down to a multiple of 16.
- * ------------------------------------------------------------------------ */
-typedef enum axn_probe_kind { AXN_PROBE_READ = 0, AXN_PROBE_FILL = 1, AXN_PROBE_COPY = 2 } axn_probe_kind;
-AXN_API int axn_stream_probe(int kind, const void* src, void* dst, size_t bytes, void* stream);
 
 #ifdef __cplusplus
 }

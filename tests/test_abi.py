@@ -46,18 +46,7 @@ def test_workspace_queries():
     assert lib.axn_gemm_workspace_bytes(1, 512, 8192, 3584) == 4 * 512 * 3584 * 4   # dgrad, 112 tiles
     assert lib.axn_gemm_workspace_bytes(0, 512, 8192, 3584) == 2 * 512 * 8192 * 4   # fwd, 128 tiles of 256 x 128, 2 parts
     assert lib.axn_gemm_workspace_bytes(2, 512, 8192, 3584) == 0                    # wgrad, 448 large tiles
-    # tiles shared by two workgroups (k x 256 + 128 tiles): off unless switched on
-    shares = 16384 + 256 * 256 * 256 * 4    # flags + one slot of fp32 partial sums per workgroup
-    assert lib.axn_gemm_workspace_bytes(0, 4096, 6144, 4096) == 0
-    old = lib.axn_gemm_set_shared_tiles(1)
-    try:
-        assert old == 0
-        assert lib.axn_gemm_workspace_bytes(0, 4096, 14336, 4096) == shares         # 896 = 3 x 256 + 128 tiles
-        assert lib.axn_gemm_workspace_bytes(0, 4096, 6144, 4096) == shares          # 384: one round and a half
-        assert lib.axn_gemm_workspace_bytes(0, 4096, 4096, 4096) == 0               # whole rounds
-        assert lib.axn_gemm_workspace_bytes(1, 8192, 5120, 2560) == 0               # 320 tiles: not half a round
-    finally:
-        assert lib.axn_gemm_set_shared_tiles(old) == 1
+    assert lib.axn_gemm_workspace_bytes(0, 4096, 6144, 4096) == 0                   # 384 large tiles: no split
     assert lib.axn_gemm_workspace_bytes(0, 4096, 4096, 4096) == 0                   # one whole round
     assert lib.axn_gemm_workspace_bytes(0, 100, 128, 1024) == 0                     # ragged: no split
     assert lib.axn_gemm_workspace_bytes(0, 128, 128, 512) == 0                      # contraction too short
@@ -96,6 +85,13 @@ def test_gemm_argument_errors():
     assert lib.axn_gemm_dgrad(A, A, None, 8, 8, 8, 8, 8, 8, None) == nv.AXN_EINVAL
     assert lib.axn_gemm_wgrad(A, A, A, 8, 8, 8, 8, 8, 8, 2, nv.BF16, None) == nv.AXN_EINVAL
     assert lib.axn_gemm_wgrad(A, A, A, 8, 8, 8, 8, 8, 8, 0, nv.F16, None) == nv.AXN_EINVAL
+    # fp32 result: the promotion of an fp32 bias, so only with a bias epilogue
+    fo = lib.axn_gemm_fwd_f32out
+    assert fo(A, A, A, A, None, nv.BF16, 8, 8, 8, 8, 8, 8, nv.EPI_NONE, None) == nv.AXN_EINVAL
+    assert "BIAS" in _err()
+    assert fo(A, A, A, A, None, nv.F32, 8, 8, 8, 8, 8, 8, nv.EPI_BIAS, None) == nv.AXN_EINVAL
+    assert fo(A, A, None, A, None, nv.F16, 8, 8, 8, 8, 8, 8, nv.EPI_BIAS, None) == nv.AXN_EINVAL
+    assert fo(A, A, A, A, None, nv.BF16, 8, 12, 8, 8, 8, 16, nv.EPI_BIAS, None) == nv.AXN_ESHAPE
     # the fp16 entry points share the checks; dW there is fp16 or fp32, never bf16
     assert lib.axn_gemm_fwd_f16(A, A, None, A, None, 8, 12, 8, 8, 8, 16, 0, None) == nv.AXN_ESHAPE
     assert "axn_gemm_fwd_f16" in _err()
@@ -253,13 +249,18 @@ def test_scan_variants_argument_errors():
     assert "scratch" in _err() and "axn_mt_scan" in _err()
 
 
-def test_stream_probe_argument_errors():
-    lib = nv.load()
-    assert lib.axn_stream_probe(7, A, A, 1024, None) == nv.AXN_EINVAL
-    assert lib.axn_stream_probe(2, None, A, 1024, None) == nv.AXN_EINVAL
-    assert lib.axn_stream_probe(1, None, None, 1024, None) == nv.AXN_EINVAL
-    assert lib.axn_stream_probe(2, ctypes.c_void_p(0x1008), A, 1024, None) == nv.AXN_EALIGN
-    assert lib.axn_stream_probe(1, None, A, 0, None) == nv.AXN_OK     # nothing to do, nothing launched
+def test_probe_library_loads_and_checks_its_arguments():
+    """The benchmark-only library (include/axn_probe.h) is built beside the product
+    library, exports what its header declares and rejects bad arguments before any launch."""
+    text = open(os.path.join(ROOT, "include", "axn_probe.h")).read()
+    assert re.findall(r"AXN_PROBE_API\s+int\s+(axn_\w+)\s*\(", text) == ["axn_probe_stream"]
+    assert "axn_probe" not in open(os.path.join(ROOT, "include", "axn.h")).read()
+    lib = nv.load_probe()
+    assert lib.axn_probe_stream(7, A, A, 1024, None) == -1
+    assert lib.axn_probe_stream(2, None, A, 1024, None) == -1
+    assert lib.axn_probe_stream(1, None, None, 1024, None) == -1
+    assert lib.axn_probe_stream(2, ctypes.c_void_p(0x1008), A, 1024, None) == -2
+    assert lib.axn_probe_stream(1, None, A, 0, None) == 0     # nothing to do, nothing launched
 
 
 def test_adam_hparams_struct_layout():

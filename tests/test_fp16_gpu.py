@@ -131,8 +131,10 @@ def test_linear_layer_in_half_precision(use_autocast):
         xin = x.clone().requires_grad_(True)
         with torch.autocast("cuda", dtype=torch.float16):
             y = layer(xin)
-        assert y.dtype == torch.float16
-        y.backward(dy.half())
+        # the fp32 bias promotes the 16-bit product to fp32, as the reference's `x + bias`
+        # does under autocast (axonn/intra_layer/fully_connected.py:348)
+        assert y.dtype == torch.float32
+        y.backward(dy)
         w_used, x_used, dy_used = layer.weight.detach().half(), x.half(), dy.half()
     else:
         layer = layer.half()

@@ -82,6 +82,34 @@ def test_fused_epilogues_match_oracle(M, N, K, epilogue):
         assert z is None
 
 
+@pytest.mark.parametrize("M,N,K", [(64, 64, 64), (300, 136, 96), (512, 768, 128), (4096, 6144, 256)])
+@pytest.mark.parametrize("epilogue", ["bias", "bias_gelu"])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_forward_with_fp32_result_matches_oracle(M, N, K, epilogue, dtype):
+    """The forward whose sum with the fp32 bias stays fp32 (what type promotion makes of the
+    reference's `x + bias` under autocast): only fp32 accumulation error is left, on every
+    tile shape (register-staged, 128 x 128, whole rounds of 256 x 256 plus a rest)."""
+    from axonn_amd import ops
+
+    g = torch.Generator().manual_seed(M + N + K)
+    X = torch.randn(M, K, generator=g).to(dtype)
+    W = (torch.randn(N, K, generator=g) * 0.2).to(dtype)
+    b = torch.randn(N, generator=g) * 0.5
+    act = "gelu" if "gelu" in epilogue else None
+    yo, zo = ol.linear_forward(np64(X), np64(W).reshape(-1), (N, K), bias=b.double().numpy(),
+                               activation=act)
+    y, z = ops.gemm_fwd(X.cuda(), W.cuda(), bias=b.cuda(), activation=act, save_z=True, out_f32=True)
+    assert y.dtype == torch.float32 and y.shape == (M, N)
+    assert rel(np64(y), yo) < F32_TOL
+    if act:
+        assert z.dtype == dtype and rel(np64(z), zo) < BF16_TOL
+    # the 16-bit result of the same call is this one, rounded once
+    y16, _ = ops.gemm_fwd(X.cuda(), W.cuda(), bias=b.cuda(), activation=act)
+    assert torch.equal(y16, y.to(dtype))
+    with pytest.raises(ValueError):
+        ops.gemm_fwd(X.cuda(), W.cuda(), out_f32=True)
+
+
 def test_dgelu_dbias_matches_oracle():
     from axonn_amd import ops
 

@@ -97,7 +97,7 @@ def _device_asm(tmp_path_factory, name):
     subprocess.run(cmd, check=True, capture_output=True, timeout=900)
     text = out.read_text()
     kernels = {}
-    for m in re.finditer(r"^(_ZN3axn\S+):\s", text, re.M):
+    for m in re.finditer(r"^(_ZN\S+):\s", text, re.M):
         end = text.find(".end_amdhsa_kernel", m.end())
         if end > 0 and ".amdhsa_kernel" in text[m.end():end]:
             kernels[m.group(1)] = text[m.end():end]
@@ -105,7 +105,7 @@ def _device_asm(tmp_path_factory, name):
     return kernels
 
 
-@pytest.mark.parametrize("source", ["optim", "embedding"])
+@pytest.mark.parametrize("source", ["stream_probe", "embedding"])
 def test_hand_written_stores_are_followed_by_their_wait_states(tmp_path_factory, source):
     """A store of more than 8 bytes needs wait states before its data registers are written
     again.  The compiler inserts them for its own stores, not for a store inside an asm

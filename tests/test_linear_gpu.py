@@ -179,6 +179,39 @@ def test_autocast_bf16_with_fp32_master_weights():
     assert rel(layer.weight.grad.view(128, 128), seq.weight.grad) < 1e-2
 
 
+@pytest.mark.parametrize("amp_dtype", [torch.bfloat16, torch.float16])
+def test_autocast_with_an_fp32_bias_returns_fp32_as_the_reference_does(amp_dtype):
+    """fp32 parameters under autocast, with a bias: the reference's product is 16-bit and
+    its `x + bias` (fully_connected.py:348) is promoted to fp32 - torch.nn.Linear, whose
+    addmm autocast casts as a whole, returns the 16-bit type instead.  Values against
+    torch.nn.Linear in fp32 (<= 1e-2), dtypes asserted, gradients in the parameters' fp32."""
+    layer, seq = make_pair(128, 256, True, torch.float32)
+    with torch.no_grad():
+        layer.bias.normal_(0, 0.5)
+        seq.bias.copy_(layer.bias)
+    torch.manual_seed(1)
+    X = torch.randn(64, 128).cuda().requires_grad_(True)
+    G = torch.randn(64, 256).cuda()
+    with torch.autocast("cuda", dtype=amp_dtype):
+        Y = layer(X)
+        # the reference's composition, spelled out with torch ops
+        want = torch.matmul(X, seq.weight.t()) + seq.bias
+    assert want.dtype == torch.float32 and Y.dtype == torch.float32
+    Xs = X.detach().clone().requires_grad_(True)
+    Ys = seq(Xs)
+    assert rel(Y, Ys) < 1e-2 and rel(Y, want) < 1e-2
+    Y.backward(G)
+    Ys.backward(G)
+    assert layer.weight.grad.dtype == torch.float32 and layer.bias.grad.dtype == torch.float32
+    assert X.grad.dtype == torch.float32
+    assert rel(X.grad, Xs.grad) < 1e-2
+    assert rel(layer.weight.grad.view(256, 128), seq.weight.grad) < 1e-2
+    assert rel(layer.bias.grad, seq.bias.grad) < 1e-2
+    # a 16-bit layer (bias cast with the module) keeps its own type, as `x + bias` does there
+    half = layer.to(amp_dtype)
+    assert half(X.detach().to(amp_dtype)).dtype == amp_dtype
+
+
 def test_two_layer_mlp_step_matches_cpu_path():
     """The 2-layer MLP configuration (batch 64, 1024 -> 4096 GELU -> 1024, MSE,
     one Adam step) in fp32 against the torch CPU restatement."""

@@ -646,20 +646,24 @@ def test_stream_probes_read_fill_copy():
 
     from axonn_amd import _native as nv
 
-    lib = nv.load()
+    lib = nv.load_probe()
     stream = nv.current_stream()
+
+    def run(kind, src, dst, nbytes):
+        assert lib.axn_probe_stream(kind, src, dst, nbytes, stream) == 0
+
     for n in (4, 1000, 64 * 4 * 1000 + 12, 1 << 22):   # floats
         g = torch.Generator(device="cuda").manual_seed(n)
         src = torch.randn(n + 8, generator=g, device="cuda")
         dst = torch.full((n + 8,), 7.0, device="cuda")
         nbytes = n * 4
-        nv.check(lib.axn_stream_probe(2, src.data_ptr(), dst.data_ptr(), nbytes, stream))
+        run(2, src.data_ptr(), dst.data_ptr(), nbytes)
         assert torch.equal(dst[:n], src[:n]) and bool((dst[n:] == 7.0).all())
         keep = src.clone()
-        nv.check(lib.axn_stream_probe(2, src.data_ptr(), src.data_ptr(), nbytes, stream))
+        run(2, src.data_ptr(), src.data_ptr(), nbytes)
         assert torch.equal(src, keep)
         sink = torch.full((4,), 3.0, device="cuda")
-        nv.check(lib.axn_stream_probe(0, src.data_ptr(), sink.data_ptr(), nbytes, stream))
+        run(0, src.data_ptr(), sink.data_ptr(), nbytes)
         assert torch.equal(src, keep) and bool((sink == 3.0).all())
-        nv.check(lib.axn_stream_probe(1, None, dst.data_ptr(), nbytes, stream))
+        run(1, None, dst.data_ptr(), nbytes)
         assert bool((dst[:n] == 0.0).all()) and bool((dst[n:] == 7.0).all())
