@@ -8,7 +8,10 @@ coefficient.  With one rank per group the total is the p-norm over all gradients
 here one multi-tensor kernel reads the gradients once (sum of |g|^p in fp32 per
 workgroup, fp64 across workgroups), leaves norm and coefficient on the device, and
 a second multi-tensor kernel scales the gradients in place - no host
-synchronisation.  Any finite p; p = inf raises as in the reference (:38-39).
+synchronisation.  `get_total_norm` takes any order, +inf and -inf included (the largest
+and the smallest |g|), as the reference's passes any order on to torch.norm (:18-34);
+`clip_grad_norm_` raises for p = inf as the reference does (:38-39), and for p = -inf,
+where the reference's `norm ** norm_type` (:74-85) has no meaning.
 """
 
 from collections import defaultdict
@@ -21,8 +24,6 @@ from .. import ops
 
 def get_total_norm(tensors, norm_type=2.0, error_if_nonfinite=False):
     """p-norm over a list of tensors (gradient_normalization.py:18-34)."""
-    if norm_type == inf or norm_type == -inf:
-        raise NotImplementedError
     if len(tensors) == 0:
         return torch.tensor(0.0)
     result = _scan(tensors, 0.0, norm_type)
@@ -49,7 +50,7 @@ def _scan(grads, max_norm, norm_type=2.0):
 
 
 def clip_grad_norm_(parameters, max_norm, norm_type=2.0, error_if_nonfinite=False):
-    if norm_type == inf:
+    if norm_type == inf or norm_type == -inf:
         raise NotImplementedError
     if isinstance(parameters, torch.Tensor):
         parameters = [parameters]

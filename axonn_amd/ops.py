@@ -548,7 +548,8 @@ def _check_list(tensors, dtype=None):
 def mt_scan(grads, inv_scale=1.0, max_norm=0.0, result=None, accumulate=False, norm_type=2.0,
             workspace=True):
     """Overflow flag, sum of |g|^p, p-norm and clip coefficient of a list of gradients of
-    ONE dtype, left on the device in a ScanResult.  workspace=False takes the entry point
+    ONE dtype, left on the device in a ScanResult (p = +inf / -inf: the largest / smallest
+    |g| in place of the sum).  workspace=False takes the entry point
     that keeps its partial results in the library's own device array (no allocation here
     or there; 2-norm only, sizes up to the array's limit)."""
     if len(grads) == 0:
@@ -560,8 +561,8 @@ def mt_scan(grads, inv_scale=1.0, max_norm=0.0, result=None, accumulate=False, n
         result = ScanResult(device)
         accumulate = False
     norm_type = float(norm_type)
-    if norm_type in (float("inf"), float("-inf")) or norm_type != norm_type:
-        raise NotImplementedError("the norm's order must be finite")
+    if norm_type != norm_type:
+        raise ValueError("the norm's order is NaN")
     if not workspace:
         if norm_type != 2.0:
             raise ValueError("the entry point without a workspace computes the 2-norm")

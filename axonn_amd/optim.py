@@ -132,10 +132,12 @@ class CPUAdam(Optimizer):
             self._views = []
             self._params = all_params
             self._grad_views = []   # flat 1-D views, one per parameter: what the scan walks
+            self._linked = []       # the `.grad` tensors installed here, one per parameter
             for p in all_params:
                 n = p.numel()
                 flat_view = self.model_grads_fp16[offset:offset + n]
                 p.grad = flat_view.view(p.shape)
+                self._linked.append(p.grad)
                 self._views.append((offset, n))
                 if n:
                     self._grad_views.append(flat_view)
@@ -169,13 +171,15 @@ class CPUAdam(Optimizer):
         it.  Code that rebinds `.grad` (`model.zero_grad()` sets it to None by default, a
         cast makes a new tensor) breaks that link without an error: backward would then
         write elsewhere and the step would apply zeros.  A gradient that has moved is
-        copied into its slice and the view is installed again; a missing one is zeroed
-        (a parameter without a gradient takes no step in the reference either,
-        axonn/optim.py:103-105 walks p.grad)."""
+        copied into its slice and the view is installed again; a missing one counts as
+        zero: the step runs over the whole flat buffer, as the reference's does
+        (axonn/optim.py:157-190), so momentum and weight decay still move that parameter."""
         flat = self.model_grads_fp16
         base, esz = flat.data_ptr(), flat.element_size()
-        for p, (offset, n) in zip(self._params, self._views):
+        for i, (p, (offset, n)) in enumerate(zip(self._params, self._views)):
             g = p.grad
+            if g is self._linked[i]:   # the view installed by this class: nothing was rebound
+                continue
             if g is not None and g.data_ptr() == base + offset * esz and g.numel() == n \
                     and g.dtype == flat.dtype and g.is_contiguous():
                 continue
@@ -188,6 +192,7 @@ class CPUAdam(Optimizer):
                                        % (n, g.numel()))
                 view.copy_(g)
             p.grad = view
+            self._linked[i] = p.grad
 
     @torch.no_grad()
     def step(self, closure=None):

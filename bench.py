@@ -70,9 +70,101 @@ def parse():
                          "embedding, small_mlp); default: all")
     ap.add_argument("--no-main-set", action="store_true",
                     help="skip the Llama-3-8B-shaped set (value is null): for profiles of the other shapes")
+    ap.add_argument("--no-power", action="store_true",
+                    help="skip the power / clock telemetry legs (about 6 s)")
     ap.add_argument("--no-launch-events", action="store_true",
                     help="do not bracket every launch with events (no per-kernel figures)")
     return ap.parse_args()
+
+
+class PowerSampler:
+    """Samples the GPU's socket power (hwmon power1_input, microwatts) in a thread while a
+    loop runs, and reads the reported per-XCD gfx clocks from `amd-smi metric` once during it.
+    Everything is optional: a box that does not expose a value reports null for it."""
+
+    def __init__(self):
+        import glob
+        self.power_file = self.cap_file = None
+        for d in sorted(glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*")):
+            if os.path.exists(os.path.join(d, "power1_input")):
+                self.power_file = os.path.join(d, "power1_input")
+                cap = os.path.join(d, "power1_cap")
+                self.cap_file = cap if os.path.exists(cap) else None
+                break
+
+    @staticmethod
+    def _read(path):
+        try:
+            with open(path) as f:
+                return int(f.read().strip())
+        except (OSError, ValueError):
+            return None
+
+    @staticmethod
+    def xcd_clocks_mhz():
+        import subprocess
+        try:
+            out = subprocess.run(["amd-smi", "metric", "-g", "0", "--clock", "--json"],
+                                 stdout=subprocess.PIPE, stderr=subprocess.DEVNULL, text=True,
+                                 timeout=20).stdout
+            data = json.loads(out)
+            gpu = (data.get("gpu_data") if isinstance(data, dict) else data)[0]
+            clk = gpu["clock"]
+            vals = []
+            for i in range(16):
+                c = clk.get("gfx_%d" % i)
+                if not c:
+                    break
+                v = c["clk"]["value"] if isinstance(c["clk"], dict) else c["clk"]
+                if isinstance(v, (int, float)):
+                    vals.append(int(v))
+            return vals or None
+        except Exception:   # noqa: BLE001 - telemetry is best effort
+            return None
+
+    def measure(self, torch, fn, flops_per_call, seconds=2.5):
+        """Runs fn() back to back for `seconds`; returns the rate, the mean socket power over
+        the second half of the loop, and the gfx clocks read in the middle of it."""
+        import threading
+        rows, stop = [], threading.Event()
+
+        def sample():
+            while not stop.is_set():
+                if self.power_file:
+                    rows.append((time.perf_counter(), self._read(self.power_file)))
+                time.sleep(0.02)
+
+        clocks = {}
+
+        def read_clocks():
+            time.sleep(seconds * 0.5)
+            clocks["mhz"] = self.xcd_clocks_mhz()
+
+        th, tc = threading.Thread(target=sample, daemon=True), threading.Thread(target=read_clocks, daemon=True)
+        torch.cuda.synchronize()
+        th.start()
+        tc.start()
+        t0 = time.perf_counter()
+        calls = 0
+        while time.perf_counter() - t0 < seconds:
+            for _ in range(4):
+                fn()
+            calls += 4
+            torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        stop.set()
+        th.join()
+        tc.join(30)
+        late = [w for t, w in rows if w is not None and t >= t0 + 0.5 * (t1 - t0) and t <= t1]
+        cap = self._read(self.cap_file) if self.cap_file else None
+        mhz = clocks.get("mhz")
+        return {"tflops": round(flops_per_call * calls / (t1 - t0) / 1e12, 1),
+                "socket_power_w": round(sum(late) / len(late) / 1e6, 1) if late else None,
+                "socket_power_cap_w": round(cap / 1e6, 1) if cap else None,
+                "power_samples": len(late),
+                "gfx_clock_mhz_per_xcd": mhz,
+                "gfx_clock_mhz_mean": round(sum(mhz) / len(mhz)) if mhz else None,
+                "seconds": round(t1 - t0, 2)}
 
 
 class Layer:
@@ -243,6 +335,18 @@ def main():
                    "value": round(total_flops / lib_elapsed / 1e12, 2), "unit": "TFLOP/s",
                    "ms_per_step": round(lib_elapsed * 1e3, 4),
                    "ours_over_library": round(value / (total_flops / lib_elapsed / 1e12), 4)}
+    # Socket power and reported clocks while the step runs back to back, and while the vendor
+    # library runs the same products: the part runs these kernels at its power cap, which
+    # is what sets the rate (outside every timed region).
+    power = None
+    if main_set and not args.no_power:
+        sampler = PowerSampler()
+        power = {"source": "hwmon power1_input / power1_cap; amd-smi metric --clock (gfx_N clk per XCD)",
+                 "gfx_clock_max_mhz": 2400,
+                 "this_library": sampler.measure(torch, lambda: step(False), total_flops)}
+        if not args.no_library_baseline:
+            power["vendor_library"] = sampler.measure(torch, library_step, total_flops)
+
     def time_loop(fn, n, w=3):
         for _ in range(w):
             fn()
@@ -443,7 +547,7 @@ def main():
     if not args.no_cpu_baseline:
         cpu = cpu_baseline(torch) if main_set else None
         if adam is not None:
-            adam["cpu_baseline"] = cpu_adam_baseline(torch)
+            adam["cpu_baseline"] = cpu_adam_baseline(torch, adam_sizes(int(args.adam_elements)))
         key = "mlp_64x1024x4096x1024_fp32_train_step"
         if key in shapes:
             shapes[key]["cpu_baseline"] = cpu_small_mlp_baseline(torch)
@@ -464,6 +568,7 @@ def main():
         "roofline": roofline,
         "cpu_baseline": cpu,
         "library_baseline": library,
+        "power": power,
         "adam": adam,
         "shapes": shapes,
     }
@@ -688,24 +793,59 @@ def cpu_baseline(torch):
                       "(%.1f s of CPU work)" % (reps, secs * reps)}
 
 
-def cpu_adam_baseline(torch):
+def cpu_adam_baseline(torch, sizes):
+    """The torch-CPU restatement of the optimizer step on the benchmark's own tensor list:
+    all of it when the host has the memory (about 21 bytes per element for the states, the
+    gradients and the step's temporaries), else the first eighth of the list; the sample
+    says which.  One untimed step, then two timed."""
     from oracle import torch_cpu as ot
 
-    n = 1 << 24
+    def available_bytes():
+        try:
+            import psutil
+            return psutil.virtual_memory().available
+        except Exception:   # noqa: BLE001
+            return 0
+
+    total = sum(sizes)
+    avail = available_bytes()
+    if avail >= 40 * total:          # 2x headroom over the ~21 B/element the step touches
+        used, what = list(sizes), "all %d tensors" % len(sizes)
+    elif avail >= 40 * sum(sizes[:len(sizes) // 8]):
+        used = list(sizes[:len(sizes) // 8])
+        what = "the first %d of the %d tensors (host memory: %.0f GB available)" % (
+            len(used), len(sizes), avail / 1e9)
+    else:
+        used, what = [1 << 24], "one tensor of 2^24 elements (host memory: %.0f GB available)" % (avail / 1e9)
+    # values do not matter for the rate: every tensor is tiled from one random block
     g = torch.Generator().manual_seed(0)
-    p = torch.randn(n, generator=g) * 0.02
-    gr = (torch.randn(n, generator=g) * 1e-3 * 65536.0).bfloat16()
-    m, v = torch.zeros(n), torch.zeros(n)
-    ot.optimizer_step([gr], [p], [m], [v], 1, 65536.0, max_norm=1.0)
+    block = 1 << 22
+    base_p = torch.randn(block, generator=g) * 0.02
+    base_g = (torch.randn(block, generator=g) * 1e-3 * 65536.0).bfloat16()
+
+    def tiled(base, n):
+        out = torch.empty(n, dtype=base.dtype)
+        k = n // block
+        if k:
+            out[:k * block].view(k, block).copy_(base.expand(k, block))
+        out[k * block:].copy_(base[:n - k * block])
+        return out
+
+    ps = [tiled(base_p, n) for n in used]
+    gs = [tiled(base_g, n) for n in used]
+    ms = [torch.zeros(n) for n in used]
+    vs = [torch.zeros(n) for n in used]
+    n = sum(used)
+    ot.optimizer_step(gs, ps, ms, vs, 1, 65536.0, max_norm=1.0)
     t0 = time.perf_counter()
-    reps = 3
+    reps = 2
     for i in range(reps):
-        ot.optimizer_step([gr], [p], [m], [v], i + 2, 65536.0, max_norm=1.0)
+        ot.optimizer_step(gs, ps, ms, vs, i + 2, 65536.0, max_norm=1.0)
     secs = (time.perf_counter() - t0) / reps
     return {"value": round(30.0 * n / secs / 1e9, 2), "unit": "GB/s",
             "cores": torch.get_num_threads(), "kind": "port",
-            "sample": "torch-CPU unscale + overflow check + clip + Adam + bf16 cast on %d elements "
-                      "(1/77 of the workload), %d timed steps" % (n, reps)}
+            "sample": "torch-CPU unscale + overflow check + clip + Adam + bf16 cast on %s = %d of "
+                      "%d elements, %d timed steps of %.2f s" % (what, n, total, reps, secs)}
 
 
 if __name__ == "__main__":

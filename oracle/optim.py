@@ -103,11 +103,15 @@ def unscale_gradients(grads, dtype, loss_scale):
 
 # ----------------------------------------------------------- grad norm -------
 def _norm(x, norm_type):
-    """torch.norm(x, p) of a flat float64 vector for finite p: (sum |x|^p)^(1/p); p = 0
-    counts the non-zero elements."""
+    """torch.norm(x, p) of a flat float64 vector: (sum |x|^p)^(1/p); p = 0 counts the
+    non-zero elements, p = +inf / -inf are the largest / smallest |x| (NaN if any is)."""
     x = np.abs(np.asarray(x, dtype=np.float64).reshape(-1))
     if norm_type == 0:
         return float(np.count_nonzero(x))
+    if norm_type == np.inf:
+        return float(np.max(x))
+    if norm_type == -np.inf:
+        return float(np.min(x))
     with np.errstate(divide="ignore", over="ignore"):
         return float(np.sum(x ** norm_type) ** (1.0 / norm_type))
 
@@ -115,7 +119,7 @@ def _norm(x, norm_type):
 def get_total_norm(tensors, dtype="f64", norm_type=2.0):
     """gradient_normalization.py:18-34: the norm_type-norm of the stacked per-tensor
     norm_type-norms, each torch.norm returning the tensor's dtype.  The reference passes
-    any finite order through to torch.norm (inf is refused earlier, :38-39)."""
+    any order through to torch.norm (clip_grad_norm_ refuses inf earlier, :38-39)."""
     if len(tensors) == 0:
         return 0.0
     per = [round_to(_norm(t, norm_type), dtype) for t in tensors]

@@ -226,16 +226,15 @@ def test_multi_tensor_argument_errors():
 
 
 def test_scan_variants_argument_errors():
-    """The norm's order must be finite; the entry point without a workspace rejects what
-    its built-in array cannot hold before it touches the device."""
+    """The norm's order may be anything but NaN; the entry point without a workspace rejects
+    what its built-in array cannot hold before it touches the device."""
     lib = nv.load()
     ptrs = (ctypes.c_void_p * 2)(0x1000, 0x2000)
     sizes = (ctypes.c_int64 * 2)(4, 4)
     res = ctypes.c_void_p(0x3000)
-    for bad in (float("inf"), float("-inf"), float("nan")):
-        assert lib.axn_mt_scan_norm(ptrs, sizes, 2, nv.BF16, 1.0, 0.0, bad, 0, res, A, 4096,
-                                    None) == nv.AXN_EINVAL
-        assert "finite" in _err()
+    assert lib.axn_mt_scan_norm(ptrs, sizes, 2, nv.BF16, 1.0, 0.0, float("nan"), 0, res, A, 4096,
+                                None) == nv.AXN_EINVAL
+    assert "NaN" in _err()
     assert lib.axn_mt_scan_norm(ptrs, sizes, 2, nv.BF16, 1.0, 0.0, 3.0, 0, res, A, 0,
                                 None) == nv.AXN_EINVAL          # workspace too small
     assert lib.axn_mt_scan_noalloc(ptrs, sizes, 2, 9, 1.0, 0.0, 0, res, None) == nv.AXN_EINVAL

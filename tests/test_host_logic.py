@@ -157,7 +157,8 @@ def test_clip_grad_norm_argument_handling():
     from axonn_amd.intra_layer.gradient_normalization import get_total_norm
 
     with pytest.raises(NotImplementedError):
-        get_total_norm([torch.zeros(2)], float("inf"))
+        clip_grad_norm_([], 1.0, norm_type=float("-inf"))
+    assert float(get_total_norm([], float("inf"))) == 0.0               # any order, as the reference
     assert float(clip_grad_norm_([], 1.0, norm_type=1.0)) == 0.0        # any finite order is taken
     assert float(get_total_norm([], 3.0)) == 0.0
     assert float(clip_grad_norm_([torch.nn.Parameter(torch.zeros(2))], 1.0)) == 0.0  # no grads

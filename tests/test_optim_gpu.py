@@ -626,6 +626,31 @@ def test_clip_grad_norm_any_finite_order(p):
         assert abs(float(get_total_norm(gs, p)) - w) <= 2e-5 * w
 
 
+@pytest.mark.parametrize("p", [float("inf"), float("-inf")])
+def test_total_norm_of_infinite_order(p):
+    """get_total_norm passes +inf and -inf through as the reference's does
+    (gradient_normalization.py:18-34): the largest / smallest magnitude over every
+    gradient, exact in every dtype, over tensors of several chunks and of mixed dtypes, NaN
+    if an element is; clip_grad_norm_ refuses them."""
+    from axonn_amd.intra_layer import clip_grad_norm_
+    from axonn_amd.intra_layer.gradient_normalization import get_total_norm
+
+    g = torch.Generator(device="cuda").manual_seed(3)
+    gs = [torch.randn(n, device="cuda", generator=g) + 0.001 for n in (33, 200001, 12, 4096)]
+    want = oo.get_total_norm([t.double().cpu().numpy() for t in gs], norm_type=p)
+    ref = torch.norm(torch.stack([torch.norm(t, p) for t in gs]), p)
+    assert float(get_total_norm(gs, p)) == want == float(ref)
+    mixed = [gs[0].bfloat16(), gs[1], gs[2].half(), gs[3].bfloat16()]
+    want = oo.get_total_norm([t.double().cpu().numpy() for t in mixed], norm_type=p)
+    assert float(get_total_norm(mixed, p)) == np.float32(want)
+    gs[1][150000] = 123.0 if p > 0 else 0.0
+    assert float(get_total_norm(gs, p)) == (123.0 if p > 0 else 0.0)
+    gs[3][5] = float("nan")
+    assert np.isnan(float(get_total_norm(gs, p)))
+    with pytest.raises(NotImplementedError):
+        clip_grad_norm_([torch.nn.Parameter(gs[0])], 1.0, norm_type=p)
+
+
 def test_order_zero_counts_gradients_with_a_nonzero_element():
     from axonn_amd.intra_layer.gradient_normalization import get_total_norm
 

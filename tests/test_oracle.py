@@ -268,6 +268,23 @@ def test_norm_of_norms_equals_flat_norm():
     assert oo.get_total_norm([]) == 0.0
 
 
+@pytest.mark.parametrize("p", [float("inf"), float("-inf")])
+def test_total_norm_of_infinite_order_matches_torch(p):
+    """get_total_norm with p = +inf / -inf against the reference's own expression, the
+    torch.norm of the stacked per-tensor torch.norms (gradient_normalization.py:22-25),
+    and against the closed form (largest / smallest magnitude); a NaN element gives NaN."""
+    rng = np.random.default_rng(11)
+    ts = [rng.standard_normal(n) + 0.01 for n in (3, 400, 7, 1)]
+    tt = [torch.from_numpy(t) for t in ts]
+    want = torch.norm(torch.stack([torch.norm(t, p) for t in tt]), p)
+    assert oo.get_total_norm(ts, norm_type=p) == float(want)
+    flat = np.abs(np.concatenate(ts))
+    assert oo.get_total_norm(ts, norm_type=p) == (flat.max() if p > 0 else flat.min())
+    ts[1][17] = np.nan
+    assert np.isnan(oo.get_total_norm(ts, norm_type=p))
+    assert bool(torch.isnan(torch.norm(torch.from_numpy(ts[1]), p)))
+
+
 @pytest.mark.parametrize("p", [1.0, 3.0, 0.5, 4.0, 1.5, -1.0, 0.0])
 def test_clip_of_any_finite_order_matches_torch(p):
     """The reference hands norm_type to torch.norm per gradient and once more over the
