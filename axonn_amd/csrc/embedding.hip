@@ -7,8 +7,10 @@
 // It is written as a gather as well, so that it needs no floating-point atomics
 // and its result does not depend on the order in which workgroups run:
 //   1. the token positions are sorted by id (stable LSD radix sort over the bits
-//      of the vocabulary size; rocPRIM's device routine - the one library call);
-//   2. the first sorted slot of every id present is recorded in row_start[V];
+//      of the vocabulary size, kernels below: no library call, no atomics on
+//      floating-point data, nothing but kernel launches);
+//   2. the first sorted slot of every id present is recorded in row_start[V] (by the
+//      sort's last pass: the smallest slot a row's tokens land in);
 //   3. one wave per 64 x 16 bytes of a dW row walks that row's run of sorted
 //      slots, adds the dY rows in ascending token order in fp32 and stores the
 //      row once; rows no token names are stored as zeros (beta = 0) or left alone
@@ -19,7 +21,6 @@
 #include "axn_internal.h"
 
 #include <cstring>
-#include <rocprim/device/device_radix_sort.hpp>
 
 namespace axn {
 namespace {
@@ -57,33 +58,286 @@ __global__ void __launch_bounds__(64 * WAVES_PER_BLOCK)
 }
 
 // ---- sorting the token positions by id ---------------------------------------
-// keys[i] = ids[i] (V for an id outside [0, V): those sort behind every row),
-// vals[i] = i, row_start[v] = -1, status = 0.
-__global__ void __launch_bounds__(256)
-    embedding_keys_kernel(const int64_t* __restrict__ ids, int* __restrict__ keys,
-                          int* __restrict__ vals, int* __restrict__ row_start, int* status,
-                          int64_t T, int64_t V) {
-  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (i < T) {
-    const int64_t id = ids[i];
-    keys[i] = (id >= 0 && id < V) ? (int)id : (int)V;
-    vals[i] = (int)i;
-  }
-  if (i < V) row_start[i] = -1;
-  if (i == 0) *status = 0;
+// Stable least-significant-digit radix sort of (key, position) pairs, keys over [0, V]
+// (V for an id outside [0, V): those sort behind every row), in 1 to 4 passes of at most
+// 10 bits.  A workgroup of 4 waves owns 256 G consecutive slots, wave w the w-th quarter of
+// them (G = 2 for batches up to 2^15 tokens, where short pieces give the sort more waves,
+// G = 8 beyond, where they keep the count arrays small).  Per pass:
+//   counts   hist[digit][workgroup] = slots of the workgroup whose key has that digit (pass
+//            0: counted by the kernel that writes the keys; later passes: counted by the
+//            previous pass's scatter with integer atomics, which add up to the same counts
+//            in any order)
+//   scan     exclusive prefix sum over the digit-major array: where the workgroup's slots
+//            of a digit go (a launch of its own beyond 2^17 tokens; up to there the array is
+//            small and every workgroup of the scatter sums what lies in front of it itself)
+//   scatter  every wave counts the digits of its quarter, which places the quarters of a
+//            digit one behind the other; then a wave walks its quarter 64 slots at a time
+//            in slot order: lanes with equal digits find one another with one ballot per
+//            digit bit, and a slot goes to (the running count of its digit) + (equal-digit
+//            lanes before it).  Slots of equal digit keep their order, which is what makes
+//            the sort stable and the order of every row's tokens ascending.
+constexpr int SORT_SHORT_BATCH = 1 << 15;   // tokens up to which a wave's quarter is 128 slots
+constexpr int SORT_FUSED_BATCH = 1 << 17;   // tokens (at most 64 workgroups) up to which no scan is launched
+constexpr int SORT_WAVES = 4;        // waves per workgroup
+constexpr int SORT_MAX_BITS = 10;    // digit width: 1024 counters per wave in LDS
+constexpr int SORT_MAX_PASSES = 4;
+
+struct SortPlan {
+  int passes;
+  int bits[SORT_MAX_PASSES], shift[SORT_MAX_PASSES];
+  int groups;                         // 64-slot groups per wave
+  bool fused_scan;                    // the scatter derives the prefix sums itself
+  int64_t nblk;                       // workgroups = units of the count arrays
+  size_t hist_ofs[SORT_MAX_PASSES];   // in ints, from the start of the histogram area
+  size_t hist_ints;
+};
+
+__device__ __forceinline__ int key_of_id(int64_t id, int64_t V) {
+  return (id >= 0 && id < V) ? (int)id : (int)V;
 }
 
-__global__ void __launch_bounds__(256)
-    embedding_row_start_kernel(const int* __restrict__ keys, int* __restrict__ row_start,
-                               int* status, int64_t T, int64_t V) {
-  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (i >= T) return;
-  const int k = keys[i];
-  if (i != 0 && keys[i - 1] == k) return;
-  if (k < V)
-    row_start[k] = (int)i;
-  else
-    *status = 1;
+// keys[i], vals[i] = i, pass 0's counts; row_start[v] = -1, status = 0, the later passes'
+// counts cleared.
+template <int G>
+__global__ void __launch_bounds__(64 * SORT_WAVES)
+    embedding_sort_prepare_kernel(const int64_t* __restrict__ ids, int* __restrict__ keys,
+                                  int* __restrict__ vals, int* __restrict__ row_start, int* status,
+                                  int* __restrict__ hist0, int* __restrict__ hist_rest,
+                                  int64_t hist_rest_ints, int64_t T, int64_t V, int64_t nblk,
+                                  int bits0, bool block_major) {
+  __shared__ int cnt[1 << SORT_MAX_BITS];
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  const int64_t gtid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t nthreads = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = gtid; i < hist_rest_ints; i += nthreads) hist_rest[i] = 0;
+  for (int64_t i = gtid; i < V; i += nthreads) row_start[i] = -1;
+  if (gtid == 0) *status = 0;
+  const int nd = 1 << bits0;
+  for (int d = threadIdx.x; d < nd; d += 64 * SORT_WAVES) cnt[d] = 0;
+  __syncthreads();
+  const int64_t blk = blockIdx.x;
+  if (blk < nblk) {
+    const int64_t first = (blk * SORT_WAVES + w) * (64 * G);
+    int64_t id[G];   // all loads of the wave in flight at once
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+      const int64_t i = first + g * 64 + lane;
+      id[g] = i < T ? ids[i] : 0;
+    }
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+      const int64_t i = first + g * 64 + lane;
+      if (i < T) {
+        const int key = key_of_id(id[g], V);
+        keys[i] = key;
+        vals[i] = (int)i;
+        atomicAdd(&cnt[key & (nd - 1)], 1);
+      }
+    }
+  }
+  __syncthreads();
+  if (blk < nblk)
+    for (int d = threadIdx.x; d < nd; d += 64 * SORT_WAVES)
+      hist0[block_major ? blk * nd + d : (int64_t)d * nblk + blk] = cnt[d];
+}
+
+// Inclusive prefix sum across the 64 lanes in six data-parallel-primitive adds (no LDS
+// round trip): shifts by 1, 2, 4, 8 inside the rows of 16 lanes (a lane the shift leaves
+// without a source adds 0), then lane 15's total into rows 1 and 3, then lane 31's into
+// rows 2 and 3.
+__device__ __forceinline__ int wave_inclusive_sum(int v) {
+  v += __builtin_amdgcn_update_dpp(0, v, 0x111, 0xf, 0xf, true);    // row_shr:1
+  v += __builtin_amdgcn_update_dpp(0, v, 0x112, 0xf, 0xf, true);    // row_shr:2
+  v += __builtin_amdgcn_update_dpp(0, v, 0x114, 0xf, 0xf, true);    // row_shr:4
+  v += __builtin_amdgcn_update_dpp(0, v, 0x118, 0xf, 0xf, true);    // row_shr:8
+  v += __builtin_amdgcn_update_dpp(0, v, 0x142, 0xa, 0xf, false);   // row_bcast:15 into rows 1, 3
+  v += __builtin_amdgcn_update_dpp(0, v, 0x143, 0xc, 0xf, false);   // row_bcast:31 into rows 2, 3
+  return v;
+}
+
+// In-place exclusive prefix sum over n ints, one workgroup of 1024 threads: tiles of 65536
+// entries, 4096 consecutive ones per wave held in registers as 16 rows of 64 lanes x 4 (every
+// access of a wave covers 1 KiB of consecutive bytes, every load of a tile in flight at
+// once, nothing read twice); rows are scanned across the lanes, the rows' totals along the
+// wave, the waves' totals across the workgroup, and a running total goes from tile to tile.
+__global__ void __launch_bounds__(1024) embedding_sort_scan_kernel(int* __restrict__ h, int64_t n) {
+  typedef int i32x4 __attribute__((ext_vector_type(4)));
+  constexpr int ROWS = 16;                // 16-byte vectors per thread and tile
+  __shared__ int wave_total[16];
+  const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+  int carry = 0;
+  for (int64_t tile = 0; tile < n; tile += 1024 * ROWS * 4) {
+    const int64_t lo = tile + (int64_t)w * (64 * ROWS * 4) + lane * 4;
+    i32x4 v[ROWS];
+#pragma unroll
+    for (int j = 0; j < ROWS; ++j) {
+      const int64_t i = lo + 256 * j;
+      if (i + 3 < n) {
+        v[j] = *(const i32x4*)(h + i);
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[j][e] = i + e < n ? h[i + e] : 0;
+      }
+    }
+    int excl[ROWS];   // sum of everything of this wave's part in front of v[j]
+    int wave_sum = 0;
+#pragma unroll
+    for (int j = 0; j < ROWS; ++j) {
+      const int s = v[j][0] + v[j][1] + v[j][2] + v[j][3];
+      const int incl = wave_inclusive_sum(s);
+      excl[j] = wave_sum + incl - s;
+      wave_sum += __builtin_amdgcn_readlane(incl, 63);
+    }
+    __syncthreads();   // the previous tile's totals have been read
+    if (lane == 0) wave_total[w] = wave_sum;
+    __syncthreads();
+    int before = carry, all = 0;
+    for (int k = 0; k < 16; ++k) {
+      if (k < w) before += wave_total[k];
+      all += wave_total[k];
+    }
+#pragma unroll
+    for (int j = 0; j < ROWS; ++j) {
+      const int64_t i = lo + 256 * j;
+      i32x4 o;
+      o[0] = before + excl[j];
+      o[1] = o[0] + v[j][0];
+      o[2] = o[1] + v[j][1];
+      o[3] = o[2] + v[j][2];
+      if (i + 3 < n) {
+        *(i32x4*)(h + i) = o;
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          if (i + e < n) h[i + e] = o[e];
+      }
+    }
+    carry += all;
+  }
+}
+
+// SCANNED: `base` holds the exclusive prefix sums of the counts (embedding_sort_scan_kernel
+// has run); otherwise it holds the counts themselves and every workgroup derives its own
+// part of the prefix sums from them - all digit-major rows in front of a digit's row and
+// the row up to this workgroup - which for few workgroups costs less than a launch.
+template <int G, bool SCANNED>
+__global__ void __launch_bounds__(64 * SORT_WAVES)
+    embedding_sort_scatter_kernel(const int* __restrict__ keys_in, const int* __restrict__ vals_in,
+                                  int* __restrict__ keys_out, int* __restrict__ vals_out,
+                                  const int* __restrict__ base, int* __restrict__ next_hist,
+                                  int* __restrict__ row_start, int* status, int64_t T, int64_t V,
+                                  int64_t nblk, int shift, int bits, int next_shift, int next_bits) {
+  __shared__ int cnt[SORT_WAVES][1 << SORT_MAX_BITS];
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  const int64_t blk = blockIdx.x;
+  const int nd = 1 << bits;
+  for (int d = threadIdx.x; d < SORT_WAVES * nd; d += 64 * SORT_WAVES) cnt[d / nd][d % nd] = 0;
+  const int64_t first = (blk * SORT_WAVES + w) * (64 * G);
+  int kreg[G], vreg[G];   // all loads of the wave in flight at once
+#pragma unroll
+  for (int g = 0; g < G; ++g) {
+    const int64_t i = first + g * 64 + lane;
+    const bool active = i < T;
+    kreg[g] = active ? keys_in[i] : 0;
+    vreg[g] = active ? vals_in[i] : 0;
+  }
+  __syncthreads();
+  // the digits of this wave's quarter
+#pragma unroll
+  for (int g = 0; g < G; ++g)
+    if (first + g * 64 + lane < T) atomicAdd(&cnt[w][(kreg[g] >> shift) & (nd - 1)], 1);
+  __syncthreads();
+  // counts -> first destination of each wave's slots of a digit; a thread sees to the
+  // digits t, t + 256, t + 512, t + 768 (at most 1024 digits, 256 threads)
+  int first_dest[4] = {0, 0, 0, 0};
+  if constexpr (SCANNED) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const int d = threadIdx.x + 256 * e;
+      if (d < nd) first_dest[e] = base[(int64_t)d * nblk + blk];
+    }
+  } else {
+    // The counts lie workgroup-major here ([workgroup][digit]: consecutive lanes read
+    // consecutive words).  A digit's slots start behind every slot of a smaller digit (the
+    // digits' totals, scanned over the workgroup in digit order) and behind the digit's
+    // slots of the workgroups in front of this one.
+    __shared__ int wave_total[4][SORT_WAVES];
+    int tot[4] = {0, 0, 0, 0}, pre[4] = {0, 0, 0, 0};
+#pragma unroll 8
+    for (int64_t b = 0; b < nblk; ++b) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int d = threadIdx.x + 256 * e;
+        const int c = d < nd ? base[b * nd + d] : 0;
+        tot[e] += c;
+        pre[e] += b < blk ? c : 0;
+      }
+    }
+    int incl[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      incl[e] = wave_inclusive_sum(tot[e]);
+      if (lane == 63) wave_total[e][w] = incl[e];
+    }
+    __syncthreads();
+    int run = 0;   // slots of the digits in front of digit 256 e + 64 w
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+#pragma unroll
+      for (int k = 0; k < SORT_WAVES; ++k) {
+        if (k == w) first_dest[e] = run + incl[e] - tot[e] + pre[e];
+        run += wave_total[e][k];
+      }
+    }
+  }
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const int d = threadIdx.x + 256 * e;
+    if (d < nd) {
+      int run = first_dest[e];
+#pragma unroll
+      for (int k = 0; k < SORT_WAVES; ++k) {
+        const int c = cnt[k][d];
+        cnt[k][d] = run;
+        run += c;
+      }
+    }
+  }
+  __syncthreads();
+  const uint64_t below = lane == 0 ? 0ull : (~0ull >> (64 - lane));
+#pragma unroll
+  for (int g = 0; g < G; ++g) {   // (every wave makes every trip: the barriers below)
+    const bool active = first + g * 64 + lane < T;
+    const int key = kreg[g];
+    const int val = vreg[g];
+    const int d = (key >> shift) & (nd - 1);
+    uint64_t same = __ballot(active);   // the lanes whose slot has this lane's digit
+    for (int b = 0; b < bits; ++b) {
+      const bool bit = (d >> b) & 1;
+      const uint64_t with = __ballot(active && bit);
+      same &= bit ? with : ~with;
+    }
+    const int off = active ? cnt[w][d] : 0;
+    __syncthreads();   // every lane has read its digit's count before any lane moves one on
+    if (active && lane == 63 - __builtin_clzll(same)) cnt[w][d] = off + __builtin_popcountll(same);
+    __syncthreads();
+    if (active) {
+      const int dest = off + __builtin_popcountll(same & below);
+      keys_out[dest] = key;
+      vals_out[dest] = val;
+      if (next_hist != nullptr) {
+        const int nx = (key >> next_shift) & ((1 << next_bits) - 1);
+        const int64_t nb = dest / (64 * G * SORT_WAVES);
+        atomicAdd(&next_hist[SCANNED ? (int64_t)nx * nblk + nb : (nb << next_bits) + nx], 1);
+      } else if (key < V) {
+        // last pass: the slots are final, and a row's run starts at the smallest of them
+        // (row_start holds -1 = the largest unsigned value until a slot arrives)
+        atomicMin((unsigned*)&row_start[key], (unsigned)dest);
+      } else {
+        *status = 1;   // an id outside the table
+      }
+    }
+  }
 }
 
 // ---- backward ------------------------------------------------------------------
@@ -302,15 +556,37 @@ constexpr size_t ALIGN = 256;
 inline size_t round_up(size_t n) { return (n + ALIGN - 1) / ALIGN * ALIGN; }
 
 struct Workspace {
-  int *keys_a, *keys_b, *vals_a, *vals_b, *row_start, *status;
-  void* sort_temp;
-  size_t sort_temp_bytes;
+  int *keys_a, *keys_b, *vals_a, *vals_b, *row_start, *status, *hist;
 };
 
-// The sort's own temporary storage is bounded here by arithmetic, so that the size
-// query needs no device: 16 bytes per token and 4 MiB cover rocPRIM's histograms
-// and block descriptors with a wide margin; the launch checks the real need.
-inline size_t sort_temp_bound(int64_t T) { return round_up((size_t)T * 16 + (4u << 20)); }
+int bits_for(int64_t V) {  // keys run over [0, V]
+  int b = 1;
+  while ((1LL << b) <= V) ++b;
+  return b;
+}
+
+// The passes of the sort: the key's bits in equal parts of at most SORT_MAX_BITS, and one
+// digit-major count array [2^bits][segments] per pass.
+SortPlan plan_sort(int64_t T, int64_t V) {
+  SortPlan pl;
+  const int total = bits_for(V);
+  pl.passes = (total + SORT_MAX_BITS - 1) / SORT_MAX_BITS;
+  pl.groups = T <= SORT_SHORT_BATCH ? 2 : 8;
+  pl.fused_scan = T <= SORT_FUSED_BATCH;
+  const int64_t per_block = 64 * pl.groups * SORT_WAVES;
+  pl.nblk = (T + per_block - 1) / per_block;
+  int shift = 0;
+  size_t ofs = 0;
+  for (int p = 0; p < SORT_MAX_PASSES; ++p) {
+    pl.bits[p] = p < pl.passes ? total / pl.passes + (p < total % pl.passes ? 1 : 0) : 0;
+    pl.shift[p] = shift;
+    pl.hist_ofs[p] = ofs;
+    shift += pl.bits[p];
+    if (p < pl.passes) ofs += ((size_t)1 << pl.bits[p]) * (size_t)pl.nblk;
+  }
+  pl.hist_ints = ofs;
+  return pl;
+}
 
 inline bool carve(void* ws, size_t ws_bytes, int64_t T, int64_t V, Workspace* out) {
   char* p = (char*)ws;
@@ -321,45 +597,64 @@ inline bool carve(void* ws, size_t ws_bytes, int64_t T, int64_t V, Workspace* ou
   out->vals_b = (int*)p; p += tok;
   out->row_start = (int*)p; p += round_up((size_t)V * sizeof(int));
   out->status = (int*)p; p += ALIGN;
-  out->sort_temp = p;
-  out->sort_temp_bytes = sort_temp_bound(T);
-  return (size_t)(p - (char*)ws) + out->sort_temp_bytes <= ws_bytes;
-}
-
-int bits_for(int64_t V) {  // keys run over [0, V]
-  int b = 1;
-  while ((1LL << b) <= V) ++b;
-  return b;
+  out->hist = (int*)p; p += round_up(plan_sort(T, V).hist_ints * sizeof(int));
+  return (size_t)(p - (char*)ws) <= ws_bytes;
 }
 
 // Fills ws with the sorted (key, position) pairs and row_start; on return
 // *keys and *vals point at the sorted arrays.
 int sort_token_positions(const int64_t* ids, int64_t T, int64_t V, const Workspace& w,
                          const int** keys, const int** vals, hipStream_t stream) {
-  const int64_t span = T > V ? T : V;
-  hipLaunchKernelGGL(embedding_keys_kernel, dim3((unsigned)((span + 255) / 256)), dim3(256), 0,
-                     stream, ids, w.keys_a, w.vals_a, w.row_start, w.status, T, V);
-  AXN_HIP_TRY(hipGetLastError());
-  *keys = w.keys_a;
-  *vals = w.vals_a;
-  if (T == 0) return AXN_OK;
-  rocprim::double_buffer<int> k(w.keys_a, w.keys_b), v(w.vals_a, w.vals_b);
-  size_t need = 0;
-  AXN_HIP_TRY(rocprim::radix_sort_pairs(nullptr, need, k, v, (size_t)T, 0, (unsigned)bits_for(V),
-                                        stream));
-  if (need > w.sort_temp_bytes) {
-    set_error("embedding: the sort needs %zu bytes of temporary storage, %zu reserved", need,
-              w.sort_temp_bytes);
+  const SortPlan pl = plan_sort(T, V);
+  if (pl.nblk >= (1LL << 31) ||
+      pl.hist_ints >= ((size_t)1 << 40)) {
+    set_error("embedding: too many tokens to sort (%lld)", (long long)T);
     return AXN_ELIMIT;
   }
-  need = w.sort_temp_bytes;
-  AXN_HIP_TRY(rocprim::radix_sort_pairs(w.sort_temp, need, k, v, (size_t)T, 0,
-                                        (unsigned)bits_for(V), stream));
-  *keys = k.current();
-  *vals = v.current();
-  hipLaunchKernelGGL(embedding_row_start_kernel, dim3((unsigned)((T + 255) / 256)), dim3(256), 0,
-                     stream, *keys, w.row_start, w.status, T, V);
+  const dim3 block(64 * SORT_WAVES);
+  const int64_t seg_blocks = pl.nblk;
+  // (at least enough workgroups to fill row_start at a good rate when the batch is short)
+  int64_t fill_blocks = (V + 4 * 256 - 1) / (4 * 256);
+  if (fill_blocks > 1024) fill_blocks = 1024;
+  const int64_t prep_blocks = seg_blocks > fill_blocks ? seg_blocks : (fill_blocks > 0 ? fill_blocks : 1);
+  int* hist_rest = w.hist + pl.hist_ofs[1];
+  const int64_t hist_rest_ints = pl.passes > 1 ? (int64_t)(pl.hist_ints - pl.hist_ofs[1]) : 0;
+  if (pl.groups == 2)
+    hipLaunchKernelGGL(embedding_sort_prepare_kernel<2>, dim3((unsigned)prep_blocks), block, 0, stream, ids,
+                       w.keys_a, w.vals_a, w.row_start, w.status, w.hist, hist_rest, hist_rest_ints, T, V,
+                       pl.nblk, pl.bits[0], pl.fused_scan);
+  else
+    hipLaunchKernelGGL(embedding_sort_prepare_kernel<8>, dim3((unsigned)prep_blocks), block, 0, stream, ids,
+                       w.keys_a, w.vals_a, w.row_start, w.status, w.hist, hist_rest, hist_rest_ints, T, V,
+                       pl.nblk, pl.bits[0], pl.fused_scan);
   AXN_HIP_TRY(hipGetLastError());
+  const int *kin = w.keys_a, *vin = w.vals_a;
+  int *kout = w.keys_b, *vout = w.vals_b;
+  if (T > 0) {
+    for (int p = 0; p < pl.passes; ++p) {
+      int* hist = w.hist + pl.hist_ofs[p];
+      const int64_t n = ((int64_t)1 << pl.bits[p]) * pl.nblk;
+      if (!pl.fused_scan) {
+        hipLaunchKernelGGL(embedding_sort_scan_kernel, dim3(1), dim3(1024), 0, stream, hist, n);
+        AXN_HIP_TRY(hipGetLastError());
+      }
+      const bool more = p + 1 < pl.passes;
+      void (*scatter)(const int*, const int*, int*, int*, const int*, int*, int*, int*, int64_t, int64_t,
+                      int64_t, int, int, int, int) =
+          pl.fused_scan ? (pl.groups == 2 ? embedding_sort_scatter_kernel<2, false>
+                                          : embedding_sort_scatter_kernel<8, false>)
+                        : embedding_sort_scatter_kernel<8, true>;
+      hipLaunchKernelGGL(scatter, dim3((unsigned)seg_blocks), block, 0, stream, kin, vin, kout, vout,
+                         (const int*)hist, more ? w.hist + pl.hist_ofs[p + 1] : nullptr, w.row_start,
+                         w.status, T, V, pl.nblk, pl.shift[p], pl.bits[p], more ? pl.shift[p + 1] : 0,
+                         more ? pl.bits[p + 1] : 0);
+      AXN_HIP_TRY(hipGetLastError());
+      const int* tk = kin; kin = kout; kout = (int*)tk;
+      const int* tv = vin; vin = vout; vout = (int*)tv;
+    }
+  }
+  *keys = kin;
+  *vals = vin;
   return AXN_OK;
 }
 
@@ -368,7 +663,7 @@ int sort_token_positions(const int64_t* ids, int64_t T, int64_t V, const Workspa
 size_t embedding_workspace_bytes(int64_t T, int64_t V) {
   if (T < 0 || V <= 0) return 0;
   return 4 * round_up((size_t)T * sizeof(int)) + round_up((size_t)V * sizeof(int)) + ALIGN +
-         sort_temp_bound(T);
+         round_up(plan_sort(T, V).hist_ints * sizeof(int));
 }
 
 int launch_embedding_fwd(const int64_t* ids, const void* W, void* out, int elem_bytes, int64_t T,

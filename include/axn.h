@@ -234,10 +234,10 @@ AXN_API int axn_embedding_fwd(const int64_t* ids, const void* W, void* out, int 
                       int64_t T, int64_t V, int64_t H, int64_t ldw, int64_t ldo,
                       int32_t* status, void* stream);
 
-/* Workspace of the two entry points below (token positions sorted by id).
- * Both call a library sort (rocPRIM), which may clear its own storage with
- * memset operations: keep them out of captured HIP graphs.  Every other entry
- * point of this library launches kernels only and can be captured. */
+/* Workspace of the two entry points below (token positions sorted by id: four int32 per
+ * token, one per table row, and the sort's digit counts - 2 to 8 bytes per token and pass).
+ * Like every entry point of this library they launch kernels only (the sort is a radix sort
+ * of the library's own) and can be captured in a HIP graph. */
 AXN_API size_t axn_embedding_workspace_bytes(int64_t T, int64_t V);
 
 /* Backward.  Replaces the autograd of the same F.embedding call

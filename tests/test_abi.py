@@ -52,10 +52,12 @@ def test_workspace_queries():
     assert lib.axn_gemm_workspace_bytes(0, 128, 128, 512) == 0                      # contraction too short
     assert lib.axn_gemm_workspace_bytes(0, 128, 128, 4096) == 8 * 128 * 128 * 4
     assert lib.axn_gemm_workspace_bytes(3, 128, 128, 4096) == 0 and lib.axn_gemm_workspace_bytes(0, 0, 8, 8) == 0
-    # embedding: four int32 arrays over the tokens, one over the rows, the sort's own storage
+    # embedding: four int32 arrays over the tokens, one over the rows, and the sort's digit
+    # counts (17 key bits = two passes of 9 and 8 bits, one count per digit and 512 tokens)
     T, V = 16384, 128256
     need = lib.axn_embedding_workspace_bytes(T, V)
-    assert 4 * T * 4 + V * 4 + 16 * T <= need <= 4 * T * 4 + V * 4 + 16 * T + (8 << 20)
+    counts = (512 + 256) * (T // 512) * 4
+    assert 4 * T * 4 + V * 4 + counts <= need <= 4 * T * 4 + V * 4 + counts + 4096
     assert lib.axn_embedding_workspace_bytes(0, V) >= V * 4
     assert lib.axn_embedding_workspace_bytes(T, 0) == 0 and lib.axn_embedding_workspace_bytes(-1, V) == 0
 

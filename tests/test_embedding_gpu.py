@@ -97,6 +97,29 @@ def test_backward_equals_the_sequential_sum_bit_for_bit(dy_dtype, dw_dtype, T, V
     assert np.array_equal(host(dW), want)
 
 
+@pytest.mark.parametrize("T,V", [(700, 3), (513, 1023), (5000, 1024), (40000, 70000), (3000, (1 << 21) + 5),
+                                 (100000, 200), ((1 << 18) + 77, 5000), (300000, 1 << 20)])
+def test_backward_over_every_shape_of_the_sort(T, V):
+    """The token positions are sorted by id with the library's own radix sort: one pass
+    (up to 10 key bits), two (11 to 20) and three (21 and more), token counts that end
+    inside a segment, both segment lengths (128 slots up to 2^18 tokens, 512 beyond), and ids
+    drawn from a few hot rows so that runs cross segments.  The row sums depend on the order of their terms: equal to the sequential
+    loop bit for bit means every row's tokens came out in ascending order."""
+    from axonn_amd import ops
+
+    g = torch.Generator(device="cuda").manual_seed(T + V)
+    ids = torch.randint(0, V, (T,), device="cuda", generator=g)
+    hot = torch.randint(0, V, (7,), device="cuda", generator=g)
+    pick = torch.randint(0, 7, (T,), device="cuda", generator=g)
+    ids = torch.where(torch.rand(T, device="cuda", generator=g) < 0.3, hot[pick], ids)
+    ids[-1] = V - 1
+    ids[0] = 0
+    dy = torch.randn(T, 8, device="cuda", generator=g)
+    dW = ops.embedding_bwd(ids, dy, V)
+    want = oe.embedding_backward(ids.cpu().numpy(), host(dy), V)
+    assert np.array_equal(host(dW), want)
+
+
 def test_backward_padding_row_repeated_ids_and_determinism():
     """A tenth of the tokens name one row, another tenth the padding row; the sum of 400
     terms depends on its order, and the kernel's order is the token order."""

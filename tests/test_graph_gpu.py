@@ -2,7 +2,8 @@
 the fused epilogue, dgrad, accumulating wgrad, gradient scan, Adam) is replayed several
 times, with eager work and synchronisations between the replays, and every replay must
 equal the eager step on the same inputs bit for bit.  The library issues no memset, copy,
-allocation or synchronisation of its own, so a capture holds kernel nodes only.
+allocation or synchronisation of its own, so a capture holds kernel nodes only; that
+includes the embedding's weight gradient and max_norm, whose sort is the library's own.
 """
 
 import pytest
@@ -123,3 +124,44 @@ def test_captured_tile_kernels_replay_like_eager(M, N, K):
         torch.cuda.synchronize()
         for got, exp, name in zip(outs, want, ("y", "dx", "dw")):
             assert torch.equal(got, exp), (replay, name)
+
+
+def test_captured_embedding_backward_and_renorm_replay_like_eager():
+    """The embedding's weight gradient (sort of the token positions, row starts, row sums)
+    and the max_norm pass under capture, replayed on new ids and gradients."""
+    from axonn_amd import ops
+
+    T, V, H = 3000, 5000, 64
+    g = torch.Generator(device="cuda").manual_seed(5)
+    ids = torch.randint(0, V, (T,), device="cuda", generator=g)
+    dy = torch.randn(T, H, device="cuda", generator=g)
+    W = torch.randn(V, H, device="cuda", generator=g)
+
+    def work(table):
+        dW = ops.embedding_bwd(ids, dy, V, padding_idx=3)
+        ops.embedding_renorm_(table, ids, 1.5)
+        return dW
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        work(W.clone())
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    live = W.clone()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out = work(live)
+    for replay in range(3):
+        ids.copy_(torch.randint(0, V, (T,), device="cuda", generator=g))
+        ids[replay::7] = 11          # a long run that moves from replay to replay
+        dy.copy_(torch.randn(T, H, device="cuda", generator=g))
+        live.copy_(W)
+        twin = W.clone()
+        want = work(twin)            # eager
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, want), replay
+        assert torch.equal(live, twin), replay
+        assert not torch.equal(live, W)
