@@ -54,6 +54,8 @@ SYMBOLS = {
     "axn_gemm_wgrad": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _int, _int, _vp]),
     "axn_gemm_fwd_f16": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _int,
                                 _vp]),
+    "axn_gemm_bwd": (_int, [_vp, _vp, _vp, _vp, _vp, _int, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64,
+                            _int, _int, _vp]),
     "axn_gemm_fwd_f32out": (_int, [_vp, _vp, _vp, _vp, _vp, _int, _i64, _i64, _i64, _i64, _i64, _i64,
                                    _int, _vp]),
     "axn_gemm_dgrad_f16": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _vp]),

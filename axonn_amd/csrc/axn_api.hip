@@ -240,6 +240,34 @@ int axn_gemm_wgrad_f16(const void* dY, const void* X, void* dW, int64_t M, int64
                        dw_dtype, stream);
 }
 
+int axn_gemm_bwd(const void* dY, const void* W, const void* X, void* dX, void* dW, int dtype,
+                 int64_t M, int64_t N, int64_t K, int64_t lddy, int64_t ldw, int64_t ldx,
+                 int64_t lddx, int64_t lddw, int beta, int dw_dtype, void* stream) {
+  const char* name = "axn_gemm_bwd";
+  REQUIRE(dtype == AXN_BF16 || dtype == AXN_F16, AXN_EINVAL, "%s: dtype must be bf16 or fp16", name);
+  const bool half = dtype == AXN_F16;
+  int rc = check_gemm(name, dY, W, dX, M, N, K, lddy, ldw, lddx, N, K, K);
+  if (rc) return rc;
+  rc = check_gemm(name, dY, X, dW, M, N, K, lddy, ldx, lddw, N, K, K);
+  if (rc) return rc;
+  REQUIRE(beta == 0 || beta == 1, AXN_EINVAL, "%s: beta must be 0 or 1", name);
+  REQUIRE(dw_dtype == dtype || dw_dtype == AXN_F32, AXN_EINVAL, "%s: dW must be %s or fp32", name,
+          half ? "fp16" : "bf16");
+  GemmArgs gd = {}, gw = {};
+  gd.A = (const uint16_t*)dY;
+  gd.B = (const uint16_t*)W;
+  gd.C = dX;
+  gd.M = (int)M, gd.N = (int)K, gd.Kc = (int)N;
+  gd.lda = lddy, gd.ldb = ldw, gd.ldc = lddx;
+  gw.A = (const uint16_t*)dY;
+  gw.B = (const uint16_t*)X;
+  gw.C = dW;
+  gw.M = (int)N, gw.N = (int)K, gw.Kc = (int)M;
+  gw.lda = lddy, gw.ldb = ldx, gw.ldc = lddw;
+  gw.beta = beta;
+  return launch_gemm_backward(gd, gw, half, dw_dtype == AXN_F32, (hipStream_t)stream);
+}
+
 // ---- split-contraction variants --------------------------------------------------
 static void fill_gemm_args(GemmArgs& g, int op, const void* a, const void* b, void* c, int64_t M,
                            int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc) {

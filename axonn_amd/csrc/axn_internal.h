@@ -91,6 +91,8 @@ struct GemmArgs {
   int64_t lda, ldb, ldc;
   int tiles_m, tiles_n;
   int beta;  // 0: C = AB ; 1: C += AB
+  // First workgroup of this problem in a launch that runs two problems (launch_gemm_backward).
+  int wg_first;
   // Split of the contraction over workgroups (splits > 1): workgroup id / tiles is the
   // split, which covers k_split contraction elements and writes its fp32 partial
   // product to C + split * M * ldc.  0 or 1: no split.
@@ -125,6 +127,11 @@ int launch_gemm_f16(GemmLayout layout, const GemmArgs& args, int epilogue, bool 
 // adds them in split order, adds the old output if args.beta, and stores args.C in
 // out_dtype.  No epilogue.
 int gemm_splits(GemmLayout layout, const GemmArgs& args, bool* wide_tiles = nullptr);
+// dX = dY W and dW (+)= dY^T X of one layer, args as for GEMM_NN and GEMM_TN.  Results are
+// those of the two separate launches bit for bit; when the two problems' tile counts leave
+// CUs idle one after the other but not together, they run as ONE launch (see gemm_bf16.hip).
+int launch_gemm_backward(const GemmArgs& dgrad, const GemmArgs& wgrad, bool half, bool dw_f32,
+                         hipStream_t stream);
 int launch_gemm_splitk(GemmLayout layout, const GemmArgs& args, bool half, int out_dtype,
                        int splits, bool wide_tiles, float* ws, hipStream_t stream);
 

@@ -60,12 +60,22 @@ def _compute_dtype(*tensors):
     return dt
 
 
-def _weight_grad(grad_2d, input_2d, original_weight):
-    """dW = dY^T X in the parameter's dtype, flat, either returned to autograd or
-    - under overlap_reduce_scatter - accumulated straight into weight.grad."""
+def _backward_products(grad_2d, w, input_2d, original_weight, need_input, need_weight):
+    """dX = dY W and dW = dY^T X as AsyncLinear.backward needs them (:140, :147-151).  dW
+    comes in the parameter's dtype, flat, either returned to autograd or - under
+    overlap_reduce_scatter - accumulated straight into weight.grad.  When both are asked
+    for they go through one entry point (ops.gemm_bwd).  Returns (dX, dW for autograd)."""
+    if not need_weight:
+        return (ops.gemm_dgrad(grad_2d, w) if need_input else None), None
     out_dtype = original_weight.dtype
     if out_dtype not in (torch.float32, grad_2d.dtype):
         out_dtype = grad_2d.dtype  # the kernels write dW in the operands' type or in fp32
+
+    def products(**kw):
+        if need_input:
+            return ops.gemm_bwd(grad_2d, w, input_2d, **kw)
+        return None, ops.gemm_wgrad(grad_2d, input_2d, **kw)
+
     if overlap_communication.OVERLAP_REDUCE_SCATTER:
         grad = original_weight.grad
         # the kernel writes 16-byte vectors: a gradient that is a view at an odd offset
@@ -75,17 +85,21 @@ def _weight_grad(grad_2d, input_2d, original_weight):
             and grad.numel() == original_weight.numel() and grad.data_ptr() % 16 == 0
         )
         if fusable:
-            ops.gemm_wgrad(grad_2d, input_2d, out=grad, accumulate=True)
+            dx, _ = products(out=grad, accumulate=True)
         elif grad is None and out_dtype == original_weight.dtype:
-            original_weight.grad = ops.gemm_wgrad(
-                grad_2d, input_2d, out_dtype=out_dtype
-            ).reshape(original_weight.shape)
+            dx, dw = products(out_dtype=out_dtype)
+            original_weight.grad = dw.reshape(original_weight.shape)
         else:
-            dw = ops.gemm_wgrad(grad_2d, input_2d, out_dtype=out_dtype).reshape(-1)
-            overlap_communication.accumulate_later(original_weight, dw)
-        return None
-    dw = ops.gemm_wgrad(grad_2d, input_2d, out_dtype=out_dtype).reshape(-1)
-    return _reduce_scatter(dw, dim=0, process_group=None, overlap_comm=False)
+            dx, dw = products(out_dtype=out_dtype)
+            overlap_communication.accumulate_later(original_weight, dw.reshape(-1))
+        return dx, None
+    dx, dw = products(out_dtype=out_dtype)
+    return dx, _reduce_scatter(dw.reshape(-1), dim=0, process_group=None, overlap_comm=False)
+
+
+def _weight_grad(grad_2d, input_2d, original_weight):
+    """The weight gradient alone (callers that compute the input gradient by other means)."""
+    return _backward_products(grad_2d, None, input_2d, original_weight, False, True)[1]
 
 
 class AsyncLinear(Function):
@@ -124,12 +138,11 @@ class AsyncLinear(Function):
         dt = ctx.compute_dtype
         w = w_cast if w_cast is not None else weight.to(dt)
         g = grad_output.reshape(-1, grad_output.shape[-1]).to(dt)
-        grad_input, grad_weight = None, None
         get_world_size(ctx.backward_all_reduce_group)
-        if ctx.needs_input_grad[0]:
-            grad_input = ops.gemm_dgrad(g, w).reshape(ctx.input_shape)
-        if ctx.needs_input_grad[1]:
-            grad_weight = _weight_grad(g, x, original_weight)
+        grad_input, grad_weight = _backward_products(g, w, x, original_weight,
+                                                     ctx.needs_input_grad[0], ctx.needs_input_grad[1])
+        if grad_input is not None:
+            grad_input = grad_input.reshape(ctx.input_shape)
         return grad_input, grad_weight, None, None, None, None, None
 
 
@@ -173,11 +186,10 @@ class FusedLinear(Function):
         grad_bias = None
         if z is not None or want_dbias:
             g, grad_bias = ops.dgelu_dbias(g, z, want_dbias=want_dbias)
-        grad_input, grad_weight = None, None
-        if ctx.needs_input_grad[0]:
-            grad_input = ops.gemm_dgrad(g, w).reshape(ctx.input_shape)
-        if ctx.needs_input_grad[1]:
-            grad_weight = _weight_grad(g, x, original_weight)
+        grad_input, grad_weight = _backward_products(g, w, x, original_weight,
+                                                     ctx.needs_input_grad[0], ctx.needs_input_grad[1])
+        if grad_input is not None:
+            grad_input = grad_input.reshape(ctx.input_shape)
         return grad_input, grad_weight, grad_bias, None, None
 
 

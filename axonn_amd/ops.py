@@ -234,6 +234,46 @@ def gemm_wgrad(dy, x, out=None, accumulate=False, out_dtype=None):
     return out
 
 
+def gemm_bwd(dy, w, x, out=None, accumulate=False, out_dtype=None):
+    """(dX, dW) = (dY W, dY^T X) of one layer, dW optionally accumulated into `out`: the two
+    products of AsyncLinear.backward (axonn/intra_layer/fully_connected.py:140, :147-151)
+    through ONE entry point, which runs both in a single launch where their tile counts
+    would each leave CUs idle in a launch of their own.  Results equal gemm_dgrad and
+    gemm_wgrad bit for bit; shapes the joint entry point does not take go through those."""
+    _require_gpu(dy, w, x, out)
+    M, N = dy.shape
+    K = w.shape[1]
+    plain16 = (dy.dtype in _GEMM16 and dy.dtype == w.dtype == x.dtype and M > 0
+               and not _ragged16(dy.dtype, N, K)
+               and nv.load().axn_gemm_workspace_bytes(GEMM_DGRAD, M, N, K) == 0
+               and nv.load().axn_gemm_workspace_bytes(GEMM_WGRAD, M, N, K) == 0)
+    if not plain16:
+        return gemm_dgrad(dy, w), gemm_wgrad(dy, x, out=out, accumulate=accumulate, out_dtype=out_dtype)
+    if x.shape != (M, K) or w.shape[0] != N:
+        raise ValueError("shapes do not match: dY %s, W %s, X %s" % (tuple(dy.shape), tuple(w.shape),
+                                                                     tuple(x.shape)))
+    if out is not None:
+        if out.numel() != N * K or not out.is_contiguous():
+            raise ValueError("`out` must be a contiguous tensor of %d elements" % (N * K))
+        out_dtype = out.dtype
+    elif accumulate:
+        raise ValueError("accumulate=True needs `out`")
+    if out_dtype is None:
+        out_dtype = dy.dtype
+    if out_dtype not in (dy.dtype, torch.float32):
+        raise TypeError("dW must be %s or fp32, got %s" % (dy.dtype, out_dtype))
+    dy, lddy = _prep_bf16(dy)
+    w, ldw = _prep_bf16(w)
+    x, ldx = _prep_bf16(x)
+    dx = torch.empty((M, K), dtype=dy.dtype, device=dy.device)
+    if out is None:
+        out = torch.empty((N, K), dtype=out_dtype, device=dy.device)
+    nv.call("axn_gemm_bwd", nv.ptr(dy), nv.ptr(w), nv.ptr(x), nv.ptr(dx), nv.ptr(out), nv.dtype_code(dy.dtype),
+            M, N, K, lddy, ldw, ldx, K, K, 1 if accumulate else 0, nv.dtype_code(out_dtype),
+            nv.current_stream())
+    return dx, out
+
+
 def dgelu_dbias(dy, z=None, want_dbias=True, dbias_out=None, accumulate=False):
     """dZ = dY * gelu'(Z) (when z is given) and dbias = column sums of dZ (fp32).
     Returns (dz, dbias); dz is dy itself when z is None."""

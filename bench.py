@@ -398,8 +398,11 @@ def main():
                     nv.check(lib.axn_dgelu_dbias(L.dY.data_ptr(), L.Z.data_ptr(), L.dZ.data_ptr(),
                                                  nv.BF16, L.db.data_ptr(), L.M, L.N, L.N,
                                                  1 if mb else 0, ws.data_ptr(), ws_bytes, stream))
-                    dgrad(L, L.dZ)
-                    wgrad(L, 1 if mb else 0, L.dZ)
+                    # dX and the accumulated dW through the entry point for both (one launch here:
+                    # 320 + 200 tiles of 256 x 256 leave CUs idle one after the other)
+                    nv.check(lib.axn_gemm_bwd(L.dZ.data_ptr(), L.W.data_ptr(), L.X.data_ptr(),
+                                              L.dX.data_ptr(), L.dW.data_ptr(), nv.BF16, L.M, L.N, L.K,
+                                              L.N, L.K, L.K, L.K, L.K, 1 if mb else 0, nv.BF16, stream))
 
             t = time_loop(mlp_shard_step, max(args.steps // 4, 3)) / 4
             shapes["mlp_shard_8192x5120x2560_bias_gelu"] = {

@@ -129,6 +129,18 @@ AXN_API int axn_gemm_wgrad_f16(const void* dY, const void* X, void* dW, int64_t 
                        int64_t N, int64_t K, int64_t lddy, int64_t ldx, int64_t lddw,
                        int beta, int dw_dtype, void* stream);
 
+/* Input gradient and weight gradient of one layer in one call: what AsyncLinear.backward
+ * computes (axonn/intra_layer/fully_connected.py:140 and :147-151, with beta = 1 the
+ * accumulation of overlap_communication.py:42-45).  Arguments as axn_gemm_dgrad and
+ * axn_gemm_wgrad together (dtype AXN_BF16 or AXN_F16 for dY, W, X, dX; dW of dw_dtype), the
+ * results are theirs bit for bit.  Shapes whose two tile counts would each leave CUs idle
+ * in a launch of their own (8192 x 5120 x 2560: 320 and 200 tiles of 256 x 256 on 256 CUs)
+ * run as ONE launch, the longer tiles first, so that a CU takes a tile of the other product
+ * as soon as it is free; any other shape is the two calls one after the other. */
+AXN_API int axn_gemm_bwd(const void* dY, const void* W, const void* X, void* dX, void* dW,
+                 int dtype, int64_t M, int64_t N, int64_t K, int64_t lddy, int64_t ldw,
+                 int64_t ldx, int64_t lddx, int64_t lddw, int beta, int dw_dtype, void* stream);
+
 /* Forward with the result in fp32.  Under autocast the reference's product is 16-bit and
  * its bias an fp32 parameter, so `x + bias` (fully_connected.py:348) is promoted to fp32:
  * this is that sum - Y = X W^T + b (AXN_EPI_BIAS) or gelu of it (AXN_EPI_BIAS_GELU; other

@@ -87,6 +87,14 @@ def test_gemm_argument_errors():
     assert lib.axn_gemm_dgrad(A, A, None, 8, 8, 8, 8, 8, 8, None) == nv.AXN_EINVAL
     assert lib.axn_gemm_wgrad(A, A, A, 8, 8, 8, 8, 8, 8, 2, nv.BF16, None) == nv.AXN_EINVAL
     assert lib.axn_gemm_wgrad(A, A, A, 8, 8, 8, 8, 8, 8, 0, nv.F16, None) == nv.AXN_EINVAL
+    # both gradients in one call: the checks of the two calls
+    fb = lib.axn_gemm_bwd
+    assert fb(A, A, A, A, A, nv.F32, 8, 8, 8, 8, 8, 8, 8, 8, 0, nv.F32, None) == nv.AXN_EINVAL
+    assert fb(A, A, A, A, A, nv.BF16, 8, 8, 8, 8, 8, 8, 8, 8, 2, nv.BF16, None) == nv.AXN_EINVAL
+    assert fb(A, A, A, A, A, nv.BF16, 8, 8, 8, 8, 8, 8, 8, 8, 0, nv.F16, None) == nv.AXN_EINVAL
+    assert fb(A, A, None, A, A, nv.BF16, 8, 8, 8, 8, 8, 8, 8, 8, 0, nv.BF16, None) == nv.AXN_EINVAL
+    assert fb(A, A, A, A, A, nv.BF16, 8, 12, 8, 16, 8, 8, 8, 8, 0, nv.BF16, None) == nv.AXN_ESHAPE
+    assert "axn_gemm_bwd" in _err()
     # fp32 result: the promotion of an fp32 bias, so only with a bias epilogue
     fo = lib.axn_gemm_fwd_f32out
     assert fo(A, A, A, A, None, nv.BF16, 8, 8, 8, 8, 8, 8, nv.EPI_NONE, None) == nv.AXN_EINVAL

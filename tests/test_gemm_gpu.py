@@ -676,3 +676,35 @@ def test_every_block_of_long_contraction_shapes(name):
     assert blocks_ok(ops.gemm_dgrad(dY, W), dY.float() @ W.float(), 1e-2)
     assert blocks_ok(ops.gemm_wgrad(dY, X), dY.float().t() @ X.float(), 1e-2)
     assert blocks_ok(ops.gemm_wgrad(dY, X, out_dtype=torch.float32), dY.float().t() @ X.float(), 1e-4)
+
+
+@pytest.mark.parametrize("M,N,K", [(8192, 5120, 2560),     # 320 + 200 tiles: one launch for both
+                                   (4096, 2560, 2560),     # 160 + 100 tiles: one launch
+                                   (4096, 4096, 4096),     # whole rounds: the two launches
+                                   (512, 768, 256), (100, 72, 40)])   # small tiles, ragged
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_backward_in_one_call_equals_the_two_calls(M, N, K, dtype):
+    """axn_gemm_bwd (dX and dW of one layer; one launch for both where the tile counts
+    would leave CUs idle one after the other) against axn_gemm_dgrad and axn_gemm_wgrad:
+    bit for bit, with a fresh and an accumulated dW, 16-bit and fp32; and against the oracle
+    on sampled rows of the large shapes."""
+    from axonn_amd import ops
+
+    g = torch.Generator(device="cuda").manual_seed(M + N)
+    X = torch.randn(M, K, device="cuda", generator=g).to(dtype)
+    W = (torch.randn(N, K, device="cuda", generator=g) * 0.05).to(dtype)
+    dY = (torch.randn(M, N, device="cuda", generator=g) * 0.01).to(dtype)
+    dx, dw = ops.gemm_bwd(dY, W, X)
+    assert torch.equal(dx, ops.gemm_dgrad(dY, W)) and torch.equal(dw, ops.gemm_wgrad(dY, X))
+    for out_dtype in (dtype, torch.float32):
+        acc = torch.randn(N, K, device="cuda", generator=g).to(out_dtype)
+        twin = acc.clone()
+        dx2, _ = ops.gemm_bwd(dY, W, X, out=acc, accumulate=True)
+        ops.gemm_wgrad(dY, X, out=twin, accumulate=True)
+        assert torch.equal(dx2, dx) and torch.equal(acc, twin)
+    rows = torch.randint(0, M, (8,), generator=torch.Generator().manual_seed(1)).tolist()
+    want = np64(dY[rows]) @ np64(W)
+    assert rel(np64(dx[rows]), want) < BF16_TOL
+    cols = torch.randint(0, N, (8,), generator=torch.Generator().manual_seed(2)).tolist()
+    want = np64(dY[:, cols]).T @ np64(X)
+    assert rel(np64(dw[cols]), want) < BF16_TOL

@@ -450,6 +450,9 @@ def test_mlp_backward_with_accumulating_weight_gradients(monkeypatch):
     calls = []
     real = ops.gemm_wgrad
     monkeypatch.setattr(ops, "gemm_wgrad", lambda *a, **k: (calls.append(k.get("accumulate", False)), real(*a, **k))[1])
+    # (a layer that also needs its input gradient asks for both through ops.gemm_bwd)
+    real_bwd = ops.gemm_bwd
+    monkeypatch.setattr(ops, "gemm_bwd", lambda *a, **k: (calls.append(k.get("accumulate", False)), real_bwd(*a, **k))[1])
     fused = run()
     # three weights, two micro-batches: the first assigns, the second accumulates in the kernel
     assert sorted(calls) == [False] * 3 + [True] * 3, calls
