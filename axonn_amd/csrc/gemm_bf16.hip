@@ -37,6 +37,9 @@
 // bounds checks, one barrier per step, epilogue transposed through LDS; ragged shapes,
 // contractions that are not multiples of 64, operands of 2 GiB and more.
 #include <atomic>
+#include <functional>
+#include <queue>
+#include <vector>
 #include <utility>
 
 #include "axn_internal.h"
@@ -783,12 +786,13 @@ __global__ void __launch_bounds__(256) gemm_f16_rest_kernel(const GemmArgs g) {
 }
 
 // Weight gradient and input gradient of one layer in one launch, 256 x 256 tiles: the
-// workgroups [0, gd.wg_first) compute dW = dY^T X (gw), the others dX = dY W (gd).  The
-// dispatcher hands workgroups out in index order, so the CUs take the weight gradient's
-// tiles first and then the input gradient's as they become free.
+// workgroups [gw.wg_first, gw.wg_first + gw's tiles) compute dW = dY^T X, the others dX = dY W.
+// The host puts the problem with the longer tiles first; the dispatcher hands workgroups
+// out in index order, so a CU takes a tile of the other product as soon as it is free.
 template <bool HALF, bool DW_F32>
 __global__ void __launch_bounds__(256) gemm_backward_kernel(const GemmArgs gw, const GemmArgs gd) {
-  if ((int)blockIdx.x < gd.wg_first)
+  const int b = (int)blockIdx.x;
+  if (b >= gw.wg_first && b < gw.wg_first + gw.tiles_m * gw.tiles_n)
     solo_gemm<256, 256, false, false, AXN_EPI_NONE, DW_F32, HALF>(gw);
   else
     solo_gemm<256, 256, true, false, AXN_EPI_NONE, false, HALF>(gd);
@@ -1225,25 +1229,25 @@ double stages_alone(long long tiles, long long stages) {
   return (double)((full + 1) * stages);
 }
 // The same for one launch that holds both problems, longer tiles first: every CU takes the
-// next tile when it is free.
+// next tile when it is free (a heap of the CUs' busy times: a few thousand steps).
 double stages_together(long long t1, long long s1, long long t2, long long s2) {
   if (s1 < s2) {
     std::swap(t1, t2);
     std::swap(s1, s2);
   }
-  long long busy_until[256] = {0};
+  std::priority_queue<long long, std::vector<long long>, std::greater<long long>> cus;
+  for (int c = 0; c < 256; ++c) cus.push(0);
+  long long end = 0;
   auto place = [&](long long tiles, long long stages) {
     for (long long i = 0; i < tiles; ++i) {
-      int best = 0;
-      for (int c = 1; c < 256; ++c)
-        if (busy_until[c] < busy_until[best]) best = c;
-      busy_until[best] += stages;
+      const long long t = cus.top() + stages;
+      cus.pop();
+      cus.push(t);
+      end = t > end ? t : end;
     }
   };
   place(t1, s1);
   place(t2, s2);
-  long long end = 0;
-  for (int c = 0; c < 256; ++c) end = busy_until[c] > end ? busy_until[c] : end;
   return (double)end;
 }
 
@@ -1260,11 +1264,27 @@ int launch_backward(const GemmArgs& gd_in, const GemmArgs& gw_in, bool dw_f32, h
     const long long td = (long long)(gd.M / 256) * (gd.N / 256), tw = (long long)(gw.M / 256) * (gw.N / 256);
     const long long sd = gd.Kc / 64, sw = gw.Kc / 64;
     // one launch when that ends at least 5 % earlier than the two launches (measured on
-    // MI355X at 8192 x 5120 x 2560: 320 tiles of 80 stages and 200 of 128)
-    if (td + tw <= 4096 && td + tw < (1LL << 20) &&
-        stages_together(tw, sw, td, sd) < 0.95 * (stages_alone(td, sd) + stages_alone(tw, sw))) {
-      gw.tiles_m = gw.M / 256, gw.tiles_n = gw.N / 256, gw.wg_first = 0;
-      gd.tiles_m = gd.M / 256, gd.tiles_n = gd.N / 256, gd.wg_first = (int)tw;
+    // MI355X at 8192 x 5120 x 2560: 320 tiles of 80 stages and 200 of 128); the answer for
+    // the last few shapes is kept, a training loop asks for the same ones again and again
+    struct Planned {
+      long long td, tw, sd, sw;
+      bool together;
+    };
+    static thread_local Planned last[4] = {};
+    static thread_local int next_slot = 0;
+    int hit = -1;
+    for (int i = 0; i < 4; ++i)
+      if (last[i].td == td && last[i].tw == tw && last[i].sd == sd && last[i].sw == sw) hit = i;
+    if (hit < 0) {
+      hit = next_slot;
+      next_slot = (next_slot + 1) % 4;
+      last[hit] = {td, tw, sd, sw,
+                   td + tw <= 4096 && stages_together(tw, sw, td, sd) <
+                                          0.95 * (stages_alone(td, sd) + stages_alone(tw, sw))};
+    }
+    if (last[hit].together) {
+      gw.tiles_m = gw.M / 256, gw.tiles_n = gw.N / 256, gw.wg_first = sw >= sd ? 0 : (int)td;
+      gd.tiles_m = gd.M / 256, gd.tiles_n = gd.N / 256, gd.wg_first = sw >= sd ? (int)tw : 0;
       gw.splits = gd.splits = 0;
       constexpr size_t lds = 5 * 256 * 64 * 2;
       void (*kern)(const GemmArgs, const GemmArgs) =

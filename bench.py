@@ -5,8 +5,9 @@
 
 A step is one forward + backward pass over the Llama-3-8B-shaped Linear set
 (4096 tokens; QKV 4096->6144, O 4096->4096, gate and up 4096->14336, down
-14336->4096; bf16 operands, fp32 accumulate, no bias): 15 GEMM launches through
-the C ABI of libaxn_gfx950.so on operands already resident in HBM.  `value` is
+14336->4096; bf16 operands, fp32 accumulate, no bias): 15 GEMMs through the C ABI
+of libaxn_gfx950.so - axn_gemm_fwd per layer, then axn_gemm_bwd (dX and dW) per
+layer - on operands already resident in HBM.  `value` is
 the aggregate TFLOP/s over the set (algorithmic 6 M N K per layer).
 
 The same run also times, outside the main timed region and reported in extra
@@ -19,8 +20,8 @@ keys of the one JSON line:
             embedding lookup and its weight gradient at the Llama-3 vocabulary
   cpu_baseline  the torch-CPU restatement of the same layer math on the host cores
 
-Every GEMM launch of the timed region is bracketed by HIP events on the launch
-stream; `roofline` reports the kernel with the largest share of the time.
+The calls of every fourth step of the timed region are bracketed by HIP events on the
+launch stream; `roofline` reports the kind of call with the largest share of the time.
 """
 
 import argparse
@@ -42,7 +43,7 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 # file, scaled by what the same counters read for the 1 GiB copy below
 # (profiles/gemm_adam_llama_set_pmc.txt has the runs and the arithmetic).  The
 # counters sit between L2 and the fabric, so hits in the memory-side cache are included.
-TRAFFIC_BYTES_PER_LAUNCH = {"fwd": 634663897, "dgrad": 587559040, "wgrad": 664873790}
+TRAFFIC_BYTES_PER_LAUNCH = {"fwd": 634663897, "bwd": 587559040 + 664873790}   # bwd: dX and dW of a layer
 ADAM_TRAFFIC_BYTES_PER_STEP = 39000439559   # scan + update, 1.3e9 elements: 1.000 x 30 B/element
 TRAFFIC_SOURCE = "profiles/gemm_adam_llama_set_pmc.txt"
 
@@ -208,14 +209,13 @@ def main():
                                   None if L.Z is None else L.Z.data_ptr(),
                                   L.M, L.N, L.K, L.K, L.K, L.N, epi, stream))
 
-    def dgrad(L, dY=None):
-        nv.check(lib.axn_gemm_dgrad((dY if dY is not None else L.dY).data_ptr(), L.W.data_ptr(),
-                                    L.dX.data_ptr(), L.M, L.N, L.K, L.N, L.K, L.K, stream))
-
-    def wgrad(L, beta=0, dY=None):
-        nv.check(lib.axn_gemm_wgrad((dY if dY is not None else L.dY).data_ptr(), L.X.data_ptr(),
-                                    L.dW.data_ptr(), L.M, L.N, L.K, L.N, L.K, L.K, beta, nv.BF16,
-                                    stream))
+    def bwd(L):
+        # dX and dW of a layer through the entry point for both (AsyncLinear.backward): two
+        # launches (four where both end in a rest), or one where the library finds that the
+        # two tile counts together fill whole rounds (here: the down projection, 896 + 896)
+        nv.check(lib.axn_gemm_bwd(L.dY.data_ptr(), L.W.data_ptr(), L.X.data_ptr(), L.dX.data_ptr(),
+                                  L.dW.data_ptr(), nv.BF16, L.M, L.N, L.K, L.N, L.K, L.K, L.K, L.K, 0,
+                                  nv.BF16, stream))
 
     selected = None if args.shapes is None else set(args.shapes.split(","))
 
@@ -237,7 +237,7 @@ def main():
     def ev():
         return torch.cuda.Event(enable_timing=True)
 
-    spans = {"fwd": [], "dgrad": [], "wgrad": []}  # (start, end, flops) per launch
+    spans = {"fwd": [], "bwd": []}  # (start, end, flops) per call
     # One event between consecutive launches: launch j of a step runs between events j
     # and j + 1, so a span is the kernel plus the gap to the next launch (3-5 us).  Half
     # the event traffic of a start/stop pair per launch, which cost 2.5 % of the step.
@@ -250,7 +250,7 @@ def main():
         fn(L)
         e = ev()
         e.record()
-        spans[kind].append((chain["last"], e, L.flops / 3.0))
+        spans[kind].append((chain["last"], e, L.flops / 3.0 * (2 if kind == "bwd" else 1)))
         chain["last"] = e
 
     def step(record):
@@ -259,8 +259,7 @@ def main():
         for L in layers:
             timed("fwd", fwd, L) if record else fwd(L)
         for L in reversed(layers):
-            timed("dgrad", dgrad, L) if record else dgrad(L)
-            timed("wgrad", wgrad, L) if record else wgrad(L)
+            timed("bwd", bwd, L) if record else bwd(L)
 
     for _ in range(args.warmup if main_set else 0):
         step(False)
@@ -291,8 +290,9 @@ def main():
         # of this instance and the rest on 256 x 128 tiles (gemm_bf16_rest_kernel) or, for r <= 64,
         # on its <128, ...> twin; the events bracket the call.
         kernel_names = {"fwd": "gemm_bf16_solo_kernel<256, true, true, 0, false> (Y = X W^T)",
-                        "dgrad": "gemm_bf16_solo_kernel<256, true, false, 0, false> (dX = dY W)",
-                        "wgrad": "gemm_bf16_solo_kernel<256, false, false, 0, false> (dW = dY^T X)"}
+                        "bwd": "axn_gemm_bwd = gemm_bf16_solo_kernel<256, true, false, 0, false> (dX = dY W) + "
+                               "gemm_bf16_solo_kernel<256, false, false, 0, false> (dW = dY^T X); for the down "
+                               "projection both in one launch (gemm_backward_kernel<false, false>)"}
         roofline = {
             "bound": "mfma", "kernel": kernel_names[dom],
             "achieved": round(kinds[dom]["tflops"], 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
@@ -305,7 +305,8 @@ def main():
             "traffic_counts": "bytes between the 8 XCD-private L2s and the fabric (FETCH_SIZE + WRITE_SIZE), "
                               "reads served by the 256 MB memory-side cache included: each L2 pulls its own "
                               "copy of a shared operand panel, so this bounds HBM bytes from above",
-            "algorithmic_bytes_per_launch": round(sum(2.0 * (L[1] * L[3] + L[2] * L[3] + L[1] * L[2])
+            "algorithmic_bytes_per_launch": round((2 if dom == "bwd" else 1) *
+                                                  sum(2.0 * (L[1] * L[3] + L[2] * L[3] + L[1] * L[2])
                                                       for L in LLAMA_SET) / len(LLAMA_SET)),
             "per_kernel": {k: {"avg_us": round(v["avg_us"], 1), "tflops": round(v["tflops"], 1),
                                "frac": round(v["tflops"] / PEAK_BF16_TFLOPS, 4)}
@@ -372,10 +373,9 @@ def main():
                 nv.check(lib.axn_gemm_fwd_f16(X.data_ptr(), W.data_ptr(), None, Y.data_ptr(), None,
                                               L.M, L.N, L.K, L.K, L.K, L.N, nv.EPI_NONE, stream))
             for L, (X, W, dY, Y, dX, dW) in zip(reversed(layers), reversed(half)):
-                nv.check(lib.axn_gemm_dgrad_f16(dY.data_ptr(), W.data_ptr(), dX.data_ptr(), L.M, L.N,
-                                                L.K, L.N, L.K, L.K, stream))
-                nv.check(lib.axn_gemm_wgrad_f16(dY.data_ptr(), X.data_ptr(), dW.data_ptr(), L.M, L.N,
-                                                L.K, L.N, L.K, L.K, 0, nv.F16, stream))
+                nv.check(lib.axn_gemm_bwd(dY.data_ptr(), W.data_ptr(), X.data_ptr(), dX.data_ptr(),
+                                          dW.data_ptr(), nv.F16, L.M, L.N, L.K, L.N, L.K, L.K, L.K, L.K, 0,
+                                          nv.F16, stream))
 
         t = time_loop(fp16_step, max(args.steps // 2, 3))
         shapes["llama_set_fp16"] = {"ms_per_step": round(t * 1e3, 4),
