@@ -43,8 +43,8 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 # file, scaled by what the same counters read for the 1 GiB copy below
 # (profiles/gemm_adam_llama_set_pmc.txt has the runs and the arithmetic).  The
 # counters sit between L2 and the fabric, so hits in the memory-side cache are included.
-TRAFFIC_BYTES_PER_LAUNCH = {"fwd": 634663897, "bwd": 587559040 + 664873790}   # bwd: dX and dW of a layer
-ADAM_TRAFFIC_BYTES_PER_STEP = 39000439559   # scan + update, 1.3e9 elements: 1.000 x 30 B/element
+TRAFFIC_BYTES_PER_LAUNCH = {"fwd": 634588622, "bwd": 1246730803}   # bwd: a call = dX and dW of a layer
+ADAM_TRAFFIC_BYTES_PER_STEP = 38997215093   # scan + update, 1.3e9 elements: 1.000 x 30 B/element
 TRAFFIC_SOURCE = "profiles/gemm_adam_llama_set_pmc.txt"
 
 LLAMA_SET = [  # (name, M, N, K), gate and up are two layers of one shape
@@ -347,6 +347,14 @@ def main():
                  "this_library": sampler.measure(torch, lambda: step(False), total_flops)}
         if not args.no_library_baseline:
             power["vendor_library"] = sampler.measure(torch, library_step, total_flops)
+        # one forward GEMM of whole rounds and a rest (gate projection, 896 tiles) back to back:
+        # the kernel alone, and the vendor library's kernel for the same product
+        G = layers[2]
+        power["forward_gate_4096x14336x4096"] = {
+            "this_library": sampler.measure(torch, lambda: fwd(G), G.flops / 3.0, seconds=2.0)}
+        if not args.no_library_baseline:
+            power["forward_gate_4096x14336x4096"]["vendor_library"] = sampler.measure(
+                torch, lambda: torch.matmul(G.X, G.W.t(), out=G.Y), G.flops / 3.0, seconds=2.0)
 
     def time_loop(fn, n, w=3):
         for _ in range(w):
