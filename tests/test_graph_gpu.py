@@ -126,6 +126,46 @@ def test_captured_tile_kernels_replay_like_eager(M, N, K):
             assert torch.equal(got, exp), (replay, name)
 
 
+def test_captured_joint_backward_replays_like_eager():
+    """axn_gemm_bwd at a shape that runs dX and dW as ONE launch (160 + 100 tiles of 256 x 256)
+    under capture: the host's choice of the launch is made at capture time, the replays run
+    the same kernel on new operands and must equal the eager call bit for bit."""
+    from axonn_amd import ops
+
+    M, N, K = 4096, 2560, 2560
+    g = torch.Generator(device="cuda").manual_seed(9)
+    X = torch.randn(M, K, device="cuda", generator=g).bfloat16()
+    W = (torch.randn(N, K, device="cuda", generator=g) * 0.05).bfloat16()
+    dY = (torch.randn(M, N, device="cuda", generator=g) * 0.01).bfloat16()
+    acc = torch.zeros(N, K, device="cuda")
+
+    def work(dw):
+        dx, _ = ops.gemm_bwd(dY, W, X, out=dw, accumulate=True)
+        return dx
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        work(torch.zeros_like(acc))
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out = work(acc)
+    assert not acc.any()                      # capturing runs nothing
+    twin = torch.zeros_like(acc)
+    for replay in range(3):
+        X.copy_(torch.randn(M, K, device="cuda", generator=g).bfloat16())
+        dY.copy_((torch.randn(M, N, device="cuda", generator=g) * 0.01).bfloat16())
+        want = work(twin)                     # eager, accumulating like the replays
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, want), replay
+        assert torch.equal(acc, twin), replay
+    assert acc.abs().sum() > 0
+
+
 def test_captured_embedding_backward_and_renorm_replay_like_eager():
     """The embedding's weight gradient (sort of the token positions, row starts, row sums)
     and the max_norm pass under capture, replayed on new ids and gradients."""

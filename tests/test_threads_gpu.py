@@ -38,8 +38,11 @@ def _work(s, rounds):
     for it in range(rounds):
         y, z = ops.gemm_fwd(s["X"], s["W"], bias=s["b"], activation="gelu", save_z=True)
         dz, db = ops.dgelu_dbias(s["dY"], z, want_dbias=True)
-        dx = ops.gemm_dgrad(dz, s["W"])
-        ops.gemm_wgrad(dz, s["X"], out=dW, accumulate=True)
+        if it % 2:   # the two gradient products through their own entry points, or through the joint one
+            dx = ops.gemm_dgrad(dz, s["W"])
+            ops.gemm_wgrad(dz, s["X"], out=dW, accumulate=True)
+        else:
+            dx, _ = ops.gemm_bwd(dz, s["W"], s["X"], out=dW, accumulate=True)
         scan = ops.mt_scan([s["G"]], inv_scale=1.0 / 64.0, max_norm=1.0)
         ops.mt_adam([s["G"]], [P], [M], [V], [PL], ops.adam_hparams(it + 1, 1e-3, 0.9, 0.999, 1e-8, 0.0),
                     inv_scale=1.0 / 64.0, scan=scan)
