@@ -479,8 +479,8 @@ def main():
                 chk = nv.check
                 gate_up_one_launch()
                 chk(lib.axn_gemm_fwd(P(act), P(wd), None, P(y), None, Mt, H, I, I, I, H, nv.EPI_NONE, stream))
-                chk(lib.axn_gemm_dgrad(P(dy), P(wd), P(dact), Mt, H, I, H, I, I, stream))
-                chk(lib.axn_gemm_wgrad(P(dy), P(act), P(dwd), Mt, H, I, H, I, I, 0, nv.BF16, stream))
+                chk(lib.axn_gemm_bwd(P(dy), P(wd), P(act), P(dact), P(dwd), nv.BF16, Mt, H, I, H, I, I, I, I, 0,
+                                     nv.BF16, stream))
                 chk(lib.axn_swiglu_bwd(P(dact), P(gt), P(up), P(dgt), P(dup), nv.BF16, Mt, I, I, stream))
                 chk(lib.axn_gemm_dgrad_pair(P(dgt), P(wg), P(dup), P(wu), P(dx1), nv.BF16, Mt, I, I, H, I, H, H,
                                             stream))
