@@ -267,7 +267,9 @@ def test_fp32_gemms_match_oracle(M, N, K):
 @pytest.mark.parametrize("M,N,K", [(128, 128, 64), (256, 384, 192), (512, 256, 320), (4096, 3072, 128),
                                    (4096, 3072, 320), (4608, 4096, 64),
                                    (4096, 6144, 4096), (4096, 256, 6144), (6144, 4096, 128),
-                                   (2304, 2048, 192), (2048, 4096, 64)])
+                                   (2304, 2048, 192), (2048, 4096, 64),
+                                   (4096, 14336, 128), (128, 14336, 4096), (192, 6144, 4096),
+                                   (2048, 12288, 64), (8192, 7168, 320)])
 def test_tile_kernels_every_output_block_with_epilogues(M, N, K):
     """Whole-tile shapes on the one-wave-per-SIMD kernel (128 x 128 tiles up to 128
     tiles of 256 x 256 and from 257 to 320 of them, else 256 x 256), checked element by
@@ -277,7 +279,12 @@ def test_tile_kernels_every_output_block_with_epilogues(M, N, K):
     one full round of large tiles and a rest of 128 for the small tile, cut along the
     output columns (forward of the first, dgrad of the second) or rows (wgrad of the
     first, forward of the third), with the bias and the saved pre-activation cut too.  The
-    last two have 72 and 128 large tiles in their forward: 256 x 128 tiles throughout."""
+    two after them have 72 and 128 large tiles in their forward: 256 x 128 tiles throughout.
+    384 and 896 large tiles also are 512 tiles of 192 and 1024 tiles of 224 columns, whole
+    rounds of workgroups: the forward takes those (256 x 192, 256 x 224), here with 1 to 64
+    contraction stages and grids of 8, 16 and 32 tile rows (the first shape of the paragraph
+    above and the last five, two of which have such a grid only in their weight gradient,
+    which keeps its rounds and rest)."""
     from axonn_amd import ops
 
     g = torch.Generator(device="cuda").manual_seed(M + N + K)
