@@ -184,58 +184,55 @@ struct OperandTile {
   }
 };
 
-// Epilogue of W = 8 or 4 consecutive columns of one output row, held in fp32: bias,
+// Epilogue of 8 consecutive columns of one output row, held in fp32: bias,
 // exact GELU with optional save of the pre-activation, accumulation into the
-// existing output (beta), conversion and one store per 16 bytes.
+// existing output (beta), conversion and one 16- or 32-byte store.
 // HALF: the 16-bit storage type is IEEE half instead of bfloat16.
-template <int W, int EPI, bool OUT_F32, bool HALF>
-__device__ __forceinline__ void store_cols(float (&v)[W], const GemmArgs& g, int row, int col) {
-  static_assert(W == 8 || W == 4, "columns per lane");
+template <int EPI, bool OUT_F32, bool HALF>
+__device__ __forceinline__ void store_row8(float (&v)[8], const GemmArgs& g, int row, int col) {
   using lp = std::conditional_t<HALF, _Float16, __bf16>;
-  typedef lp lpxw __attribute__((ext_vector_type(W)));
+  using lpx8 = std::conditional_t<HALF, f16x8, bf16x8>;
   const int64_t o = (int64_t)row * g.ldc + col;
   if (EPI == AXN_EPI_BIAS || EPI == AXN_EPI_BIAS_GELU) {
+    const f32x4 b0 = *(const f32x4*)(g.bias + col);
+    const f32x4 b1 = *(const f32x4*)(g.bias + col + 4);
 #pragma unroll
-    for (int h = 0; h < W / 4; ++h) {
-      const f32x4 b = *(const f32x4*)(g.bias + col + 4 * h);
-#pragma unroll
-      for (int e = 0; e < 4; ++e) v[4 * h + e] += b[e];
+    for (int e = 0; e < 4; ++e) {
+      v[e] += b0[e];
+      v[4 + e] += b1[e];
     }
   }
   if (EPI == AXN_EPI_BIAS_GELU || EPI == AXN_EPI_GELU) {
     if (g.Z != nullptr) {
-      lpxw z;
+      lpx8 z;
 #pragma unroll
-      for (int e = 0; e < W; ++e) z[e] = (lp)v[e];
-      *(lpxw*)(g.Z + o) = z;
+      for (int e = 0; e < 8; ++e) z[e] = (lp)v[e];
+      *(lpx8*)(g.Z + o) = z;
     }
 #pragma unroll
-    for (int e = 0; e < W; ++e) v[e] = gelu_exact(v[e]);
+    for (int e = 0; e < 8; ++e) v[e] = gelu_exact(v[e]);
   }
   if (OUT_F32) {
     float* C = (float*)g.C + o;
-#pragma unroll
-    for (int h = 0; h < W / 4; ++h) {
-      f32x4 x = {v[4 * h], v[4 * h + 1], v[4 * h + 2], v[4 * h + 3]};
-      if (g.beta) x += *(const f32x4*)(C + 4 * h);
-      *(f32x4*)(C + 4 * h) = x;
+    f32x4 o0 = {v[0], v[1], v[2], v[3]}, o1 = {v[4], v[5], v[6], v[7]};
+    if (g.beta) {
+      o0 += *(const f32x4*)C;
+      o1 += *(const f32x4*)(C + 4);
     }
+    *(f32x4*)C = o0;
+    *(f32x4*)(C + 4) = o1;
   } else {
     uint16_t* C = (uint16_t*)g.C + o;
     if (g.beta) {
-      const lpxw old = *(const lpxw*)C;
+      const lpx8 old = *(const lpx8*)C;
 #pragma unroll
-      for (int e = 0; e < W; ++e) v[e] += (float)old[e];
+      for (int e = 0; e < 8; ++e) v[e] += (float)old[e];
     }
-    lpxw y;
+    lpx8 y;
 #pragma unroll
-    for (int e = 0; e < W; ++e) y[e] = (lp)v[e];
-    *(lpxw*)C = y;
+    for (int e = 0; e < 8; ++e) y[e] = (lp)v[e];
+    *(lpx8*)C = y;
   }
-}
-template <int EPI, bool OUT_F32, bool HALF>
-__device__ __forceinline__ void store_row8(float (&v)[8], const GemmArgs& g, int row, int col) {
-  store_cols<8, EPI, OUT_F32, HALF>(v, g, row, col);
 }
 
 // Epilogue of the gate/up forward for 8 consecutive columns of one row: both
@@ -352,36 +349,16 @@ __device__ __forceinline__ s16x4 lds_read_tr16_b64(uint32_t addr) {
 // registers without a transpose through LDS.  Its K-major swizzle is
 // chunk ^ (((r >> 1) & 1) | ((r >> 3) & 3) << 1), which again gives the 16 rows
 // of a fragment quarter 16 distinct (row parity, chunk) pairs.
-//
-// ROWS = 192 and 224, K-major column operand only (tile shapes that turn a forward
-// problem's 256 x 256 tiles and a rest into whole rounds of workgroups): the tile simply has
-// fewer 128-byte rows.  A wave owns ROWS / 32 fragments; for ROWS = 224 these are three
-// fragment pairs from row 128 w on and the odd fragment 6 + w of the tile (w: the wave's
-// half): the rows 96 + 4 w + 8 (q / 4) + q % 4, read through addresses of their own, which
-// leave a lane with 4 consecutive output columns.
-template <bool KMAJOR, bool PERMUTED, int ROWS_ /* 256 or 128; 224 or 192 */>
+template <bool KMAJOR, bool PERMUTED, int ROWS_ /* 256 or 128 */>
 struct DeepOperand {
   static constexpr int ROWS = ROWS_;
   static constexpr int PK = 64;
-  static constexpr int BYTES = ROWS * PK * 2;      // 16 to 32 KiB
+  static constexpr int BYTES = ROWS * PK * 2;      // 32 or 16 KiB
   static constexpr int NW = 4;
-  static constexpr int DMA_N = BYTES / 1024 / NW;  // 4 to 8 copies per wave
+  static constexpr int DMA_N = BYTES / 1024 / NW;  // 8 or 4 copies per wave
   static constexpr int FR = ROWS / 32;             // 16-row fragments of a wave's half of the rows
-  static constexpr bool ODD = FR % 2 == 1;
-  static constexpr int NADDR = KMAJOR ? (ODD ? 4 : 2) : FR / 2;
+  static constexpr int NADDR = KMAJOR ? 2 : FR / 2;
   static constexpr int LPR = ROWS / 8;             // MN-major: lanes per contraction row of a copy
-  static_assert(ROWS == 256 || ROWS == 128 || ((ROWS == 192 || ROWS == 224) && KMAJOR && PERMUTED),
-                "192- and 224-row tiles: the K-major column operand");
-
-  // First tile row of the fragment pairs of wave half w, and of its odd fragment.
-  __device__ __forceinline__ static int wave_row0(int w) { return ODD ? 128 * w : (ROWS / 2) * w; }
-  __device__ __forceinline__ static int odd_row0(int w) { return 32 * (FR / 2) + 4 * w; }
-  // Tile row (column of the output, for the permuted operand: the first of the lane's 8 or
-  // 4) that fragment I of wave half w holds in lane-row l16 (permuted: lane-rows 4 l16 ..).
-  __device__ __forceinline__ static int out_index(int I, int w, int l16) {
-    if (PERMUTED) return (ODD && I == FR - 1 ? odd_row0(w) : wave_row0(w) + 32 * (I / 2)) + 8 * l16;
-    return wave_row0(w) + 16 * I + l16;
-  }
 
   __device__ __forceinline__ static int kmajor_swizzle(int row) {
     return PERMUTED ? (((row >> 1) & 1) | (((row >> 3) & 3) << 1)) : ((row >> 1) & 7);
@@ -418,33 +395,28 @@ struct DeepOperand {
                                              16, (int)voff, (int)(tile_ofs + IO * istride), 0, 0);
   }
 
-  // Per-lane LDS byte offsets (relative to the tile) the fragment reads of wave half w
-  // start from.
+  // Per-lane LDS byte offsets (relative to the tile) the fragment reads start from.
   //   K-major : a[s] for the 32-deep step s; fragments add whole rows (frag_offset),
-  //             which leave the swizzle unchanged.  a[2 + s]: the odd fragment.
+  //             which leave the swizzle unchanged.
   //   MN-major: a[i >> 1] for fragment i, step s adds 32 rows.  The 16 lanes of a
   //             block address contraction rows 8 (l / 16) + (l & 15) / 4 and 4
   //             columns each; the transposing read hands lane i of the block the
   //             column that lane 4 (i / 4) .. addressed, rows 8 (l / 16) + 0..3
   //             (second read: + 4..7).
-  __device__ __forceinline__ static void read_bases(uint32_t (&a)[NADDR], int w, int lane) {
+  __device__ __forceinline__ static void read_bases(uint32_t (&a)[NADDR], int wrow0, int lane) {
     const int q = lane & 15;
     if (KMAJOR) {
-      const int in_frag = PERMUTED ? 8 * (q >> 2) + (q & 3) : q;
+      const int r = wrow0 + (PERMUTED ? 8 * (q >> 2) + (q & 3) : q);
+      const int swz = kmajor_swizzle(r);
 #pragma unroll
-      for (int o = 0; o < (ODD ? 2 : 1); ++o) {
-        const int r = (o ? odd_row0(w) : wave_row0(w)) + in_frag;
-        const int swz = kmajor_swizzle(r);
-#pragma unroll
-        for (int st = 0; st < 2; ++st)
-          a[2 * o + st] = (uint32_t)(r * 128 + (((st * 4 + (lane >> 4)) ^ swz) << 4));
-      }
+      for (int st = 0; st < 2; ++st)
+        a[st] = (uint32_t)(r * 128 + (((st * 4 + (lane >> 4)) ^ swz) << 4));
     } else {
       const int kq = q >> 2;
       const int k = 8 * (lane >> 4) + kq;
 #pragma unroll
       for (int h = 0; h < NADDR; ++h) {
-        const int colbyte = (wave_row0(w) + h * 32 + (PERMUTED ? 8 : 4) * (lane & 3)) * 2;
+        const int colbyte = (wrow0 + h * 32 + (PERMUTED ? 8 : 4) * (lane & 3)) * 2;
         a[h] = (uint32_t)(k * (ROWS * 2) + ((((colbyte >> 6) ^ kq) << 6) | (colbyte & 63)));
       }
     }
@@ -454,9 +426,8 @@ struct DeepOperand {
   template <int ST, int I>
   __device__ __forceinline__ static void read_frag(bf16x8& f, const uint32_t (&a)[NADDR]) {
     if constexpr (KMAJOR) {
-      constexpr bool LONE = ODD && I == FR - 1;  // the odd fragment: addresses of its own
-      constexpr int row_ofs = LONE ? 0 : (PERMUTED ? 32 * (I >> 1) + 4 * (I & 1) : 16 * I);
-      f = lds_read_b128<row_ofs * 128>(a[(LONE ? 2 : 0) + ST]);
+      constexpr int row_ofs = PERMUTED ? 32 * (I >> 1) + 4 * (I & 1) : 16 * I;
+      f = lds_read_b128<row_ofs * 128>(a[ST]);
     } else {
       constexpr int col_ofs = PERMUTED ? 4 * (I & 1) : 16 * (I & 1);  // elements
       const s16x4 lo = lds_read_tr16_b64<ST * 32 * ROWS * 2 + col_ofs * 2>(a[I >> 1]);
@@ -468,43 +439,27 @@ struct DeepOperand {
 
 // Waits for every outstanding LDS read; the fragments flow through the
 // statement, so no MFMA on them can move above the wait.
-#define AXN_F4(f) "+v"(f[0]), "+v"(f[1]), "+v"(f[2]), "+v"(f[3])
-#define AXN_F6(f) AXN_F4(f), "+v"(f[4]), "+v"(f[5])
-#define AXN_F7(f) AXN_F6(f), "+v"(f[6])
-#define AXN_F8(f) AXN_F6(f), "+v"(f[6]), "+v"(f[7])
 __device__ __forceinline__ void wait_all_fragments(bf16x8 (&fa)[8], bf16x8 (&fb)[8]) {
-  asm volatile("s_waitcnt lgkmcnt(0)" : AXN_F8(fa), AXN_F8(fb));
-}
-__device__ __forceinline__ void wait_all_fragments(bf16x8 (&fa)[8], bf16x8 (&fb)[7]) {
-  asm volatile("s_waitcnt lgkmcnt(0)" : AXN_F8(fa), AXN_F7(fb));
-}
-__device__ __forceinline__ void wait_all_fragments(bf16x8 (&fa)[8], bf16x8 (&fb)[6]) {
-  asm volatile("s_waitcnt lgkmcnt(0)" : AXN_F8(fa), AXN_F6(fb));
+  asm volatile("s_waitcnt lgkmcnt(0)"
+               : "+v"(fa[0]), "+v"(fa[1]), "+v"(fa[2]), "+v"(fa[3]), "+v"(fa[4]), "+v"(fa[5]),
+                 "+v"(fa[6]), "+v"(fa[7]), "+v"(fb[0]), "+v"(fb[1]), "+v"(fb[2]), "+v"(fb[3]),
+                 "+v"(fb[4]), "+v"(fb[5]), "+v"(fb[6]), "+v"(fb[7]));
 }
 __device__ __forceinline__ void wait_all_fragments(bf16x8 (&fa)[8], bf16x8 (&fb)[4]) {
-  asm volatile("s_waitcnt lgkmcnt(0)" : AXN_F8(fa), AXN_F4(fb));
+  asm volatile("s_waitcnt lgkmcnt(0)"
+               : "+v"(fa[0]), "+v"(fa[1]), "+v"(fa[2]), "+v"(fa[3]), "+v"(fa[4]), "+v"(fa[5]),
+                 "+v"(fa[6]), "+v"(fa[7]), "+v"(fb[0]), "+v"(fb[1]), "+v"(fb[2]), "+v"(fb[3]));
 }
 __device__ __forceinline__ void wait_all_fragments(bf16x8 (&fa)[4], bf16x8 (&fb)[4]) {
-  asm volatile("s_waitcnt lgkmcnt(0)" : AXN_F4(fa), AXN_F4(fb));
+  asm volatile("s_waitcnt lgkmcnt(0)"
+               : "+v"(fa[0]), "+v"(fa[1]), "+v"(fa[2]), "+v"(fa[3]), "+v"(fb[0]), "+v"(fb[1]),
+                 "+v"(fb[2]), "+v"(fb[3]));
 }
-#undef AXN_F8
-#undef AXN_F7
-#undef AXN_F6
-#undef AXN_F4
 // Passes a row of accumulators through a statement (see the end of the kernel).
 __device__ __forceinline__ void settle_accumulators(f32x4 (&a)[8]) {
   asm volatile("s_nop 3"
                : "+a"(a[0]), "+a"(a[1]), "+a"(a[2]), "+a"(a[3]), "+a"(a[4]), "+a"(a[5]),
                  "+a"(a[6]), "+a"(a[7]));
-}
-__device__ __forceinline__ void settle_accumulators(f32x4 (&a)[7]) {
-  asm volatile("s_nop 3"
-               : "+a"(a[0]), "+a"(a[1]), "+a"(a[2]), "+a"(a[3]), "+a"(a[4]), "+a"(a[5]),
-                 "+a"(a[6]));
-}
-__device__ __forceinline__ void settle_accumulators(f32x4 (&a)[6]) {
-  asm volatile("s_nop 3"
-               : "+a"(a[0]), "+a"(a[1]), "+a"(a[2]), "+a"(a[3]), "+a"(a[4]), "+a"(a[5]));
 }
 __device__ __forceinline__ void settle_accumulators(f32x4 (&a)[4]) {
   asm volatile("s_nop 3" : "+a"(a[0]), "+a"(a[1]), "+a"(a[2]), "+a"(a[3]));
@@ -540,7 +495,7 @@ __device__ __forceinline__ void wait_vmcnt() {
 // Its ring has five slots of the larger (A) tile's size.
 template <int BM, int BN, bool A_KMAJOR, bool B_KMAJOR, int EPI, bool OUT_F32, bool HALF>
 __device__ __forceinline__ void solo_gemm(const GemmArgs& g) {
-  constexpr int WTN = BN / 2, FRM = BM / 32, FRN = BN / 32;
+  constexpr int WTM = BM / 2, WTN = BN / 2, FRM = BM / 32, FRN = BN / 32;
   constexpr int PK = 64, NSLOT = 5;
   constexpr int NM = FRM * FRN;         // MFMAs per step
   using OA = DeepOperand<A_KMAJOR, false, BM>;
@@ -551,10 +506,8 @@ __device__ __forceinline__ void solo_gemm(const GemmArgs& g) {
   constexpr int READ_EVERY = (NM / 2) / NFRAG;     // a fragment read every .. MFMAs, first half of a step
   constexpr int COPY_EVERY_A = (NM / 2) / NCA;     // a copy every .. MFMAs, second half
   constexpr int COPY_EVERY_B = (NM / 2) / NCB;
-  static_assert(((BM == 256 || BM == 128) && (BN == 256 || BN == 128) && BM >= BN) ||
-                    (BM == 256 && (BN == 192 || BN == 224) && A_KMAJOR && B_KMAJOR),
+  static_assert((BM == 256 || BM == 128) && (BN == 256 || BN == 128) && BM >= BN,
                 "tile sizes with a schedule below");
-  static_assert(NM % 2 == 0, "a step has two halves");
   static_assert(READ_EVERY >= 1 && COPY_EVERY_A >= 1 && COPY_EVERY_B >= 1, "schedule fits a step");
   // Gate/up forward: the B tile's 256 rows are, per 128-row half (one wave column), 64
   // rows of the gate weights and the 64 rows of the up weights with the same indices, so
@@ -596,8 +549,8 @@ __device__ __forceinline__ void solo_gemm(const GemmArgs& g) {
 
   const uint32_t lds0 = (uint32_t)(uintptr_t)LDS_PTR(char, lds);
   uint32_t ra0[OA::NADDR], rb0[OB::NADDR];
-  OA::read_bases(ra0, wm, lane);
-  OB::read_bases(rb0, wn, lane);
+  OA::read_bases(ra0, wm * WTM, lane);
+  OB::read_bases(rb0, wn * WTN, lane);
 #pragma unroll
   for (int i = 0; i < OA::NADDR; ++i) ra0[i] += lds0;
 #pragma unroll
@@ -784,11 +737,11 @@ __device__ __forceinline__ void solo_gemm(const GemmArgs& g) {
   // pair t, the 8 consecutive columns 32 t + 8 (l / 16) .. + 7 of row 16 i + l % 16:
   // they go out straight from the registers, 64 contiguous bytes per row and
   // instruction.
-  // (a 224-column tile leaves one block per row unpaired: 4 columns)
+  const int orow = m0 + wm * WTM + (lane & 15);
+  const int ocol = n0 + wn * WTN + 8 * (lane >> 4);
   if constexpr (SWIGLU) {
     // blocks 0..3 of a lane's row hold 64 gate columns, blocks 4..7 the up values of the
     // same columns
-    const int orow = m0 + OA::out_index(0, wm, lane & 15);
     const int hcol = n0 + wn * (WTN / 2) + 8 * (lane >> 4);
 #pragma unroll
     for (int i = 0; i < FRM; ++i)
@@ -803,22 +756,14 @@ __device__ __forceinline__ void solo_gemm(const GemmArgs& g) {
   } else {
     GemmArgs go = g;  // a split writes its own fp32 partial product
     if (OUT_F32 && g.splits > 1) go.C = (float*)g.C + (int64_t)split * g.M * g.ldc;
-    constexpr int EP = PAIR ? (int)AXN_EPI_NONE : EPI;
 #pragma unroll
-    for (int i = 0; i < FRM; ++i) {
-      const int orow = m0 + OA::out_index(i, wm, lane & 15);
+    for (int i = 0; i < FRM; ++i)
 #pragma unroll
       for (int t = 0; t < FRN / 2; ++t) {
         const f32x4 lo = acc[i][2 * t], hi = acc[i][2 * t + 1];
         float v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-        store_cols<8, EP, OUT_F32, HALF>(v, go, orow, n0 + OB::out_index(2 * t, wn, lane >> 4));
+        store_row8<(PAIR ? (int)AXN_EPI_NONE : EPI), OUT_F32, HALF>(v, go, orow + 16 * i, ocol + 32 * t);
       }
-      if constexpr (FRN % 2 == 1) {
-        const f32x4 x = acc[i][FRN - 1];
-        float v[4] = {x[0], x[1], x[2], x[3]};
-        store_cols<4, EP, OUT_F32, HALF>(v, go, orow, n0 + OB::out_index(FRN - 1, wn, lane >> 4));
-      }
-    }
   }
 }
 
@@ -838,14 +783,6 @@ __global__ void __launch_bounds__(256) gemm_bf16_rest_kernel(const GemmArgs g) {
 template <bool A_KMAJOR, bool B_KMAJOR, int EPI, bool OUT_F32>
 __global__ void __launch_bounds__(256) gemm_f16_rest_kernel(const GemmArgs g) {
   solo_gemm<256, 128, A_KMAJOR, B_KMAJOR, EPI, OUT_F32, true>(g);
-}
-
-// 256 x 192 and 256 x 224, forward layout: the tile shapes that make whole rounds of 256
-// workgroups out of a problem whose 256 x 256 tiles would end in a round that is at most
-// half full.
-template <int BM, int BN, bool A_KMAJOR, bool B_KMAJOR, int EPI, bool OUT_F32, bool HALF>
-__global__ void __launch_bounds__(256) gemm_rounds_kernel(const GemmArgs g) {
-  solo_gemm<BM, BN, A_KMAJOR, B_KMAJOR, EPI, OUT_F32, HALF>(g);
 }
 
 // Weight gradient and input gradient of one layer in one launch, 256 x 256 tiles: the
@@ -1058,23 +995,6 @@ int launch_rest(const GemmArgs& in, hipStream_t stream) {
   return AXN_OK;
 }
 
-template <int BM, int BN, bool AK, bool BKM, int EPI, bool OUT_F32, bool HALF>
-int launch_rounds(const GemmArgs& in, hipStream_t stream) {
-  GemmArgs g = in;
-  g.tiles_m = g.M / BM;
-  g.tiles_n = g.N / BN;
-  constexpr size_t lds = 5 * 256 * 64 * 2;  // five slots of the 256-row tile's size
-  void (*kern)(const GemmArgs) = gemm_rounds_kernel<BM, BN, AK, BKM, EPI, OUT_F32, HALF>;
-  {
-    static std::atomic<unsigned long long> lds_allowed{0};   // per template instance
-    const int rc = allow_lds((const void*)kern, lds, lds_allowed);
-    if (rc != AXN_OK) return rc;
-  }
-  hipLaunchKernelGGL(kern, dim3((unsigned)(g.tiles_m * g.tiles_n)), dim3(256), lds, stream, g);
-  AXN_HIP_TRY(hipGetLastError());
-  return AXN_OK;
-}
-
 // Kernel selection.  Problems made of whole 256 x 256 tiles, more than 128 of
 // them (half of the CUs) and not just above one round of 256, take the
 // one-wave-per-SIMD kernel at that tile size, 65..128 of them take it at 256 x 128;
@@ -1128,21 +1048,6 @@ int launch_shape(const GemmArgs& g, hipStream_t stream) {
   if (g.M % 256 == 0 && g.N % 256 == 0 && g.Kc % 64 == 0 && g.splits <= 1) {
     const long long tm = g.M / 256, tn = g.N / 256, tiles = tm * tn;
     const long long full = tiles / 256 * 256, rest = tiles - full;
-    if constexpr (AK && BKM && EPI != EPI_PAIR && EPI != EPI_SWIGLU) {
-      // Forward layout: a narrower tile that divides the problem into whole rounds of 256
-      // workgroups, if there is one.  Measured on the Llama-3-8B set's step: +1.5 % on its
-      // forward launches against full rounds and a rest (4096 x 6144: 512 tiles of 256 x 192,
-      // 4096 x 14336: 1024 of 256 x 224).  The same shapes for the weight gradient (192 and
-      // 224 rows of the contraction-strided row operand) measured 2..3 % slower than its
-      // rounds and rest, and are not built.
-      const int64_t a_span = (int64_t)g.M * g.lda * 2, b_span = (int64_t)g.N * g.ldb * 2;
-      if (full > 0 && rest > 0 && rest <= 128 && a_span < (1LL << 31) && b_span < (1LL << 31)) {
-        if (g.N % 224 == 0 && (tm * (g.N / 224)) % 256 == 0)
-          return launch_rounds<256, 224, true, true, EPI, OUT_F32, HALF>(g, stream);
-        if (g.N % 192 == 0 && (tm * (g.N / 192)) % 256 == 0)
-          return launch_rounds<256, 192, true, true, EPI, OUT_F32, HALF>(g, stream);
-      }
-    }
     if (full > 0 && rest > 0 && rest <= 128) {
       constexpr int64_t esz = OUT_F32 ? 4 : 2;
       GemmArgs g1 = g, g2 = g;

@@ -280,11 +280,9 @@ def test_tile_kernels_every_output_block_with_epilogues(M, N, K):
     output columns (forward of the first, dgrad of the second) or rows (wgrad of the
     first, forward of the third), with the bias and the saved pre-activation cut too.  The
     two after them have 72 and 128 large tiles in their forward: 256 x 128 tiles throughout.
-    384 and 896 large tiles also are 512 tiles of 192 and 1024 tiles of 224 columns, whole
-    rounds of workgroups: the forward takes those (256 x 192, 256 x 224), here with 1 to 64
-    contraction stages and grids of 8, 16 and 32 tile rows (the first shape of the paragraph
-    above and the last five, two of which have such a grid only in their weight gradient,
-    which keeps its rounds and rest)."""
+    The last five have 384 or 896 large tiles in their forward or weight gradient, with 1 to
+    64 contraction stages and grids of 8, 16, 32, 48 and 56 tile rows: one and three rounds
+    and a rest of 128."""
     from axonn_amd import ops
 
     g = torch.Generator(device="cuda").manual_seed(M + N + K)

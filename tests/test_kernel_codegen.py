@@ -26,13 +26,13 @@ def gemm_asm(tmp_path_factory):
     subprocess.run(cmd, check=True, capture_output=True, timeout=900)
     text = out.read_text()
     kernels = {}
-    for m in re.finditer(r"^(_ZN3axn\S*gemm_(?:(?:bf16|f16)_(?:solo|rest|swiglu)|backward|rounds)_kernel\S*):", text, re.M):
+    for m in re.finditer(r"^(_ZN3axn\S*gemm_(?:(?:bf16|f16)_(?:solo|rest|swiglu)|backward)_kernel\S*):", text, re.M):
         end = text.index(".end_amdhsa_kernel", m.end())
         kernels[m.group(1)] = text[m.end():end]
     # 7 layout/epilogue/output variants x 3 tile shapes (256 x 256, 128 x 128, 256 x 128) x 2 element
     # types (and the two-term input gradient as an eighth variant), and the gate/up forward of
-    # each type; the forward's 256 x 192 and 256 x 224 tiles: 6 epilogue/output variants x 2 x 2
-    assert len(kernels) >= 74, sorted(kernels)
+    # each type
+    assert len(kernels) >= 50, sorted(kernels)
     return kernels
 
 
@@ -75,8 +75,7 @@ def test_main_loop_mfma_operands_have_fixed_register_classes(gemm_asm):
     for name, body in gemm_asm.items():
         for s in _instructions(body):
             if s.startswith("v_mfma_f32_16x16x32_"):
-                half = ("gemm_f16_" in name or "gemm_backward_kernelILb1" in name   # <HALF, ...>
-                        or re.search(r"gemm_rounds_kernelI\S*Lb1EEEv", name) is not None)   # <..., HALF>
+                half = "gemm_f16_" in name or "gemm_backward_kernelILb1" in name   # <HALF, ...>
                 assert s.split()[0].endswith("_f16" if half else "_bf16"), (name, s)
                 ops = [o.strip() for o in s.split(None, 1)[1].split(",")]
                 assert ops[0].startswith("a[") and ops[3].startswith("a[") and ops[0] == ops[3], (name, s)
