@@ -78,17 +78,19 @@ __device__ __forceinline__ void static_for(F&& f) {
 }
 
 // Workgroup id -> output tile, XCD aware.  Consecutive workgroup ids go to
-// different XCDs, so ids are first regrouped per XCD into contiguous ranges of a tile
-// order (position_of_workgroup) that walks bands of GROUP_M tile rows (tile_of_position).
-__device__ __forceinline__ int position_of_workgroup(int pid, int nwg) {
+// different XCDs, so ids are first regrouped per XCD into contiguous ranges and
+// then walked in bands of GROUP_M tile rows.
+__device__ __forceinline__ void tile_of_workgroup(int pid, int tiles_m,
+                                                  int tiles_n, int& tm,
+                                                  int& tn) {
+  const int nwg = tiles_m * tiles_n;
   const int per = (nwg + NUM_XCD - 1) / NUM_XCD;
   int tall = nwg % NUM_XCD;
   if (tall == 0) tall = NUM_XCD;
   const int xcd = pid % NUM_XCD;
   const int local = pid / NUM_XCD;
-  return (xcd < tall) ? xcd * per + local : tall * per + (xcd - tall) * (per - 1) + local;
-}
-__device__ __forceinline__ void tile_of_position(int t, int tiles_m, int tiles_n, int& tm, int& tn) {
+  int t = (xcd < tall) ? xcd * per + local
+                       : tall * per + (xcd - tall) * (per - 1) + local;
   constexpr int GROUP_M = 8;
   const int in_group = GROUP_M * tiles_n;
   const int group = t / in_group;
@@ -97,11 +99,6 @@ __device__ __forceinline__ void tile_of_position(int t, int tiles_m, int tiles_n
   const int r = t - group * in_group;
   tm = first_m + r % gsz;
   tn = r / gsz;
-}
-__device__ __forceinline__ void tile_of_workgroup(int pid, int tiles_m,
-                                                  int tiles_n, int& tm,
-                                                  int& tn) {
-  tile_of_position(position_of_workgroup(pid, tiles_m * tiles_n), tiles_m, tiles_n, tm, tn);
 }
 
 // One operand tile: global -> registers -> LDS, and fragment reads.
@@ -496,11 +493,8 @@ __device__ __forceinline__ void wait_vmcnt() {
 // rounds of 256 x 256 tiles: a rest of r <= 128 large tiles makes 2 r <= 256 of these,
 // one per CU, and needs 3/4 of the global -> LDS bytes per MFMA of the 128 x 128 tile.
 // Its ring has five slots of the larger (A) tile's size.
-struct NoHook {
-  __device__ __forceinline__ void operator()() const {}
-};
-template <int BM, int BN, bool A_KMAJOR, bool B_KMAJOR, int EPI, bool OUT_F32, bool HALF, class Hook = NoHook>
-__device__ __forceinline__ void solo_gemm(const GemmArgs& g, int position = -1, Hook after_first_copies = {}) {
+template <int BM, int BN, bool A_KMAJOR, bool B_KMAJOR, int EPI, bool OUT_F32, bool HALF>
+__device__ __forceinline__ void solo_gemm(const GemmArgs& g) {
   constexpr int WTM = BM / 2, WTN = BN / 2, FRM = BM / 32, FRN = BN / 32;
   constexpr int PK = 64, NSLOT = 5;
   constexpr int NM = FRM * FRN;         // MFMAs per step
@@ -680,8 +674,7 @@ __device__ __forceinline__ void solo_gemm(const GemmArgs& g, int position = -1, 
       split = pid / (g.tiles_m * g.tiles_n);
       pid -= split * (g.tiles_m * g.tiles_n);
     }
-    if (position >= 0) tile_of_position(position, g.tiles_m, g.tiles_n, tm, tn);
-    else tile_of_workgroup(pid, g.tiles_m, g.tiles_n, tm, tn);
+    tile_of_workgroup(pid, g.tiles_m, g.tiles_n, tm, tn);
   }
   const int KP = (g.splits > 1 ? g.k_split : g.Kc) / PK;
   const int s0 = split * KP;
@@ -698,7 +691,6 @@ __device__ __forceinline__ void solo_gemm(const GemmArgs& g, int position = -1, 
     static_for<NCA>(copy_a); a_done();
     static_for<NCB>(copy_b); b_done();
   }
-  after_first_copies();
   // The accumulators are cleared here, while the first tiles are on their way: left
   // to itself the compiler clears them where they are first used, behind the wait.
 #pragma unroll
@@ -791,57 +783,6 @@ __global__ void __launch_bounds__(256) gemm_bf16_rest_kernel(const GemmArgs g) {
 template <bool A_KMAJOR, bool B_KMAJOR, int EPI, bool OUT_F32>
 __global__ void __launch_bounds__(256) gemm_f16_rest_kernel(const GemmArgs g) {
   solo_gemm<256, 128, A_KMAJOR, B_KMAJOR, EPI, OUT_F32, true>(g);
-}
-
-// Resident workgroups that take their tiles from a counter per XCD: a workgroup works through
-// its own XCD's range of the tile order and, once that is empty, takes tiles of the other
-// XCDs' ranges.  The next tile is asked for before the current one starts (the answer comes
-// back while it runs) and handed to the four waves through LDS between two tiles, when no
-// operand tile is in flight.
-__device__ int g_next_tile[NUM_XCD];
-__global__ void reset_next_tile_kernel() {
-  if (threadIdx.x < NUM_XCD) g_next_tile[threadIdx.x] = 0;
-}
-template <bool A_KMAJOR, bool B_KMAJOR, int EPI, bool OUT_F32, bool HALF>
-__global__ void __launch_bounds__(256) gemm_resident_kernel(const GemmArgs g) {
-  extern __shared__ __attribute__((aligned(16))) char lds[];
-  const int nwg = g.tiles_m * g.tiles_n;
-  const int per = (nwg + NUM_XCD - 1) / NUM_XCD;
-  int tall = nwg % NUM_XCD;
-  if (tall == 0) tall = NUM_XCD;
-  const int xcd = blockIdx.x % NUM_XCD;
-  auto first_of = [&](int x) { return x < tall ? x * per : tall * per + (x - tall) * (per - 1); };
-  auto count_of = [&](int x) { return x < tall ? per : per - 1; };
-  auto take = [&](int own) -> int {   // own: what the XCD's own counter returned
-    if (own < count_of(xcd)) return first_of(xcd) + own;
-    for (int v = 1; v < NUM_XCD; ++v) {
-      const int y = (xcd + v) % NUM_XCD;
-      const int r = atomicAdd(&g_next_tile[y], 1);
-      if (r < count_of(y)) return first_of(y) + r;
-    }
-    return -1;
-  };
-  int* box = (int*)lds;
-  const bool leader = threadIdx.x == 0;
-  if (leader) box[0] = take(atomicAdd(&g_next_tile[xcd], 1));
-  __syncthreads();
-  int pos = box[0];
-  __syncthreads();
-  while (pos >= 0) {
-    int own = 0;
-    // asked for behind the tile's first copies: the answer travels beside them
-    auto ask = [&]() {
-      asm volatile("" ::: "memory");
-      if (leader) own = atomicAdd(&g_next_tile[xcd], 1);
-      asm volatile("" ::: "memory");
-    };
-    solo_gemm<256, 256, A_KMAJOR, B_KMAJOR, EPI, OUT_F32, HALF>(g, pos, ask);
-    __syncthreads();   // every wave has read its last fragments
-    if (leader) box[0] = take(own);
-    __syncthreads();
-    pos = box[0];
-    __syncthreads();
-  }
 }
 
 // Weight gradient and input gradient of one layer in one launch, 256 x 256 tiles: the
@@ -1029,20 +970,6 @@ int launch_solo(const GemmArgs& in, hipStream_t stream) {
     if (rc != AXN_OK) return rc;
   }
   const int splits = g.splits > 1 ? g.splits : 1;
-#ifdef AXN_RESIDENT
-  if constexpr (TILE == 256 && EPI != EPI_PAIR && EPI != EPI_SWIGLU) {
-    if (splits == 1 && g.tiles_m * g.tiles_n > 256) {
-      void (*rk)(const GemmArgs) = gemm_resident_kernel<AK, BKM, EPI, OUT_F32, HALF>;
-      static std::atomic<unsigned long long> resident_allowed{0};
-      const int rc = allow_lds((const void*)rk, lds, resident_allowed);
-      if (rc != AXN_OK) return rc;
-      hipLaunchKernelGGL(reset_next_tile_kernel, dim3(1), dim3(64), 0, stream);
-      hipLaunchKernelGGL(rk, dim3(256), dim3(256), lds, stream, g);
-      AXN_HIP_TRY(hipGetLastError());
-      return AXN_OK;
-    }
-  }
-#endif
   hipLaunchKernelGGL(kern, dim3((unsigned)(g.tiles_m * g.tiles_n * splits)), dim3(256), lds, stream,
                      g);
   AXN_HIP_TRY(hipGetLastError());
