@@ -37,6 +37,7 @@
 // bounds checks, one barrier per step, epilogue transposed through LDS; ragged shapes,
 // contractions that are not multiples of 64, operands of 2 GiB and more.
 #include <atomic>
+#include <cmath>
 #include <functional>
 #include <queue>
 #include <vector>
@@ -1322,13 +1323,24 @@ int launch_gemm_f16(GemmLayout layout, const GemmArgs& g, int epilogue, bool out
   return launch_layout<true>(layout, g, epilogue, out_f32, stream);
 }
 
-// Few output tiles leave most CUs without work: tiles times splits of the contraction, each
-// split at least 512 deep.  Where the shape allows, 256 x 128 tiles with one workgroup per CU
-// (at most 256): measured on the skinny shard, forward 128 tiles x 2 parts 42.8 us against
-// 46.0 us unsplit on 256 small tiles, dgrad 56 tiles x 4 parts 44.5 us against 52.4 us on 112
-// small tiles x 4.  Otherwise 128 x 128 tiles, up to two workgroups per CU (512), only below
-// 129 tiles: with a workgroup on every second CU or more, the second pass costs more than
-// the split gains (measured at 256 small tiles: 35 -> 44 us).
+// Few output tiles leave most CUs without work: the contraction is cut into 2, 4 or 8 parts, each
+// at least 512 deep, on 128 x 128 tiles (up to two workgroups per CU) or 256 x 128 tiles (one).
+// Whether, into how many parts and on which tile to split the contraction of a problem with
+// few output tiles: the choice with the smallest estimated time.  The estimate (microseconds
+// on MI355X, operands coming from HBM) of a launch of w workgroups that each walk `stages`
+// 64-deep stages:
+//   main loop   stages x 0.77 (128 x 128 tiles, at most one workgroup per CU), x 1.33 (two
+//               per CU), x 0.93 (256 x 128 tiles: twice the output per stage), times the
+//               rounds of workgroups the launch takes;
+//   operands    never faster than their bytes at 6 TB/s, and at 47 % of that plus the rest in
+//               proportion to the CUs that have a workgroup;
+//   parts       2.1 + parts x 2.5 x (millions of output elements)^0.74 for writing the fp32
+//               partial products and for the pass that adds them.
+// The eight constants were fitted to the choices' measured times over 165 forward and
+// input-gradient problems of 128 to 1024 tokens and 2560 to 14336 features (every choice
+// timed on cold operands): the rule's pick is within 0.6 % of the fastest choice on average
+// and 13 % at worst; the rule it replaced (as many parts as fill the CUs, 256 x 128 tiles
+// first) was 4.4 % off on average and 44 % at worst.
 int gemm_splits(GemmLayout layout, const GemmArgs& g, bool* wide_tiles) {
   if (wide_tiles != nullptr) *wide_tiles = false;
   if (g.M % 128 || g.N % 128 || g.Kc % 64) return 1;
@@ -1336,20 +1348,39 @@ int gemm_splits(GemmLayout layout, const GemmArgs& g, bool* wide_tiles) {
   const int64_t a_span = (int64_t)(ak ? g.M : g.Kc) * g.lda * 2;
   const int64_t b_span = (int64_t)(bkm ? g.N : g.Kc) * g.ldb * 2;
   if (a_span >= (1LL << 31) || b_span >= (1LL << 31)) return 1;
-  if (g.M % 256 == 0) {
-    const long long wide = (long long)(g.M / 256) * (g.N / 128);
-    if (wide <= 128)
-      for (int s = 8; s >= 2; s >>= 1)
-        if (wide * s <= 256 && g.Kc % (64 * s) == 0 && g.Kc / s >= 512) {
-          if (wide_tiles != nullptr) *wide_tiles = true;
-          return s;
-        }
-  }
   const long long tiles = (long long)(g.M / 128) * (g.N / 128);
-  if (tiles > 128) return 1;
-  for (int s = 8; s >= 2; s >>= 1)
-    if (tiles * s <= 512 && g.Kc % (64 * s) == 0 && g.Kc / s >= 512) return s;
-  return 1;
+  const long long wide = g.M % 256 == 0 ? (long long)(g.M / 256) * (g.N / 128) : -1;
+  // beyond 128 tiles of either kind an unsplit launch already has a workgroup on half of the CUs
+  if (!(tiles <= 128 || (wide > 0 && wide <= 128))) return 1;
+  const double out_m = (double)g.M * g.N * 1e-6;
+  const double operand_mb = ((double)g.M + g.N) * g.Kc * 2e-6;
+  const double part_cost = 2.529 * std::pow(out_m, 0.736);
+  auto estimate = [&](int parts, bool wide_kind) {
+    const double stages = (double)g.Kc / 64 / parts;
+    const long long w = (wide_kind ? wide : tiles) * parts;
+    const double loop = wide_kind ? stages * 0.928 * (double)((w + 255) / 256)
+                                  : stages * (w <= 256 ? 0.771 : 1.332) * (double)((w + 511) / 512);
+    const double occupied = w >= 256 ? 1.0 : (double)w / 256;
+    const double stream = operand_mb / (5.998 * (0.465 + 0.535 * occupied));
+    return (loop > stream ? loop : stream) + (parts > 1 ? 2.143 + parts * part_cost : 0.0);
+  };
+  double best = estimate(1, false);
+  int best_parts = 1;
+  bool best_wide = false;
+  for (int parts = 2; parts <= 8; parts *= 2) {
+    if (g.Kc % (64 * parts) != 0 || g.Kc / parts < 512) continue;
+    for (int kind = 0; kind < 2; ++kind) {
+      if (kind == 0 ? tiles * parts > 512 : (wide <= 0 || wide * parts > 256)) continue;
+      const double t = estimate(parts, kind == 1);
+      if (t < best) {
+        best = t;
+        best_parts = parts;
+        best_wide = kind == 1;
+      }
+    }
+  }
+  if (wide_tiles != nullptr) *wide_tiles = best_wide;
+  return best_parts;
 }
 
 int launch_gemm_splitk(GemmLayout layout, const GemmArgs& in, bool half, int out_dtype,

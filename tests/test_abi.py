@@ -52,6 +52,12 @@ def test_workspace_queries():
     assert lib.axn_gemm_workspace_bytes(0, 128, 128, 512) == 0                      # contraction too short
     assert lib.axn_gemm_workspace_bytes(0, 128, 128, 4096) == 8 * 128 * 128 * 4
     assert lib.axn_gemm_workspace_bytes(3, 128, 128, 4096) == 0 and lib.axn_gemm_workspace_bytes(0, 0, 8, 8) == 0
+    # the parts are chosen by estimated time: a short contraction over an output that already has a
+    # workgroup for every CU is not split, few tiles take as many parts as still pay for their sums
+    assert lib.axn_gemm_workspace_bytes(0, 1024, 4096, 2560) == 0                   # 256 small tiles, 40 stages
+    assert lib.axn_gemm_workspace_bytes(0, 256, 2560, 2560) == 4 * 256 * 2560 * 4   # 40 small tiles: 4 parts
+    assert lib.axn_gemm_workspace_bytes(0, 512, 4096, 2560) == 2 * 512 * 4096 * 4   # 128 small tiles: 2, not 4
+    assert lib.axn_gemm_workspace_bytes(0, 256, 4096, 14336) == 8 * 256 * 4096 * 4  # long contraction: 8
     # embedding: four int32 arrays over the tokens, one over the rows, and the sort's digit
     # counts (17 key bits = two passes of 9 and 8 bits, one count per digit and 512 tokens)
     T, V = 16384, 128256
